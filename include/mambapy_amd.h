@@ -1,0 +1,162 @@
+/* C ABI of libmambapy_amd.so: hand-written gfx950 (MI355X) kernels for the selective-scan
+ * hot path of alxndrTL/mamba.py.
+ *
+ * The reference has no FFI for this path: its operator boundary is a set of Python
+ * symbols (cited per entry point below).  Each entry point here is what a ctypes binding
+ * placed behind that symbol calls.  Conventions:
+ *   - every pointer is a DEVICE pointer unless stated otherwise; the library allocates
+ *     and frees nothing, outputs and workspaces are caller-allocated;
+ *   - `stream` is a hipStream_t passed as void* (NULL = the null stream); all work is
+ *     enqueued on it and nothing synchronises the device;
+ *   - sizes are in elements, strides are ELEMENT strides of the tensor they describe;
+ *   - io_dtype selects the storage type of x, delta, B, C, z, y, dy and of their
+ *     gradients; A, D, delta_bias, the recurrent state and every accumulation are float32;
+ *   - the return value is MPA_OK or one of the MPA_ERR_* codes; nothing is thrown.
+ * All entry points are reentrant and keep no global state.
+ */
+#ifndef MAMBAPY_AMD_H
+#define MAMBAPY_AMD_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MPA_VERSION 100 /* major*10000 + minor*100 + patch */
+
+enum mpa_status {
+    MPA_OK = 0,
+    MPA_ERR_NULL_POINTER = 1,  /* a required pointer is NULL */
+    MPA_ERR_BAD_SHAPE = 2,     /* non-positive size, d_state above the supported maximum, ... */
+    MPA_ERR_BAD_DTYPE = 3,     /* io_dtype is not one of mpa_dtype */
+    MPA_ERR_BAD_STRIDE = 4,    /* a stride the kernels cannot honour (see each entry point) */
+    MPA_ERR_MISALIGNED = 5,    /* a pointer is not aligned to its element size */
+    MPA_ERR_WORKSPACE = 6,     /* workspace_bytes is smaller than the *_workspace_bytes query */
+    MPA_ERR_LAUNCH = 7         /* hipGetLastError() reported a launch failure */
+};
+
+enum mpa_dtype { MPA_F32 = 0, MPA_BF16 = 1 };
+
+/* Number of time steps between two saved states (see mpa_sscan_fwd: h_ckpt). */
+#define MPA_CKPT_STEPS 16
+/* Largest supported d_state (N). */
+#define MPA_MAX_DSTATE 256
+
+/* Shape and layout of one selective-scan call.  Logical shapes (mambapy/mamba.py:275-282):
+ *   x, delta, z, y, dy, dx, ddelta : (batch, seqlen, dim)      dim = ED = d_inner
+ *   A : (dim, dstate) contiguous float32;  D, delta_bias : (dim) contiguous float32
+ *   B, C, dB, dC : (batch, seqlen, dstate), innermost stride 1
+ * u_* strides apply to x, z (inputs);  d_* to delta;  y_* to y, dy;  g_* to dx, ddelta;
+ * bc_* to B and C;  dbc_* to dB and dC.
+ * The reference calls this path both with fresh channel-contiguous tensors
+ * (tests/compare_seq_pscan.py:24-29: strides (L*ED, ED, 1)) and, from MambaBlock.forward,
+ * with time-contiguous views (mambapy/mamba.py:217-221, 247, 264: strides (ED*L, 1, L)) and
+ * with B, C that are slices of one projection (mamba.py:245: row stride dt_rank+2N).
+ * Both layouts are honoured without a copy. */
+typedef struct mpa_sscan_shape {
+    int64_t batch, seqlen, dim, dstate;
+    int32_t io_dtype; /* enum mpa_dtype */
+    int32_t flags;    /* bit set of MPA_SSCAN_* */
+    int64_t u_sb, u_sl, u_sd;
+    int64_t d_sb, d_sl, d_sd;
+    int64_t y_sb, y_sl, y_sd;
+    int64_t g_sb, g_sl, g_sd;
+    int64_t bc_sb, bc_sl;
+    int64_t dbc_sb, dbc_sl;
+} mpa_sscan_shape;
+
+/* delta = softplus(delta + delta_bias) is applied inside the kernel (mamba.py:264-265);
+ * without the flag `delta` is used as given and delta_bias must be NULL. */
+#define MPA_SSCAN_DELTA_SOFTPLUS 1
+
+int mpa_version(void);
+/* Host string naming the GPU architecture the kernels were compiled for ("gfx950"). */
+const char* mpa_arch(void);
+/* Host string describing a status code. */
+const char* mpa_status_string(int status);
+
+/* ---- fused selective scan, forward ------------------------------------------------------
+ * Replaces MambaBlock.selective_scan(x, delta, A, B, C, D) (mambapy/mamba.py:274-295) and
+ * its sequential twin selective_scan_seq (:297-327): discretisation exp(delta*A) /
+ * delta*B*x, the scan that mambapy/pscan.py:151-186 performs on materialised
+ * (B,L,ED,N) tensors, and the readout y = C.h + D*x, in one pass that never writes a
+ * (B,L,ED,N) tensor.  Any seqlen >= 1 (no power-of-two padding, cf. pscan.py:165-174).
+ *   z        optional: y is multiplied by silu(z) (mamba.py:229-231); NULL = no gate.
+ *   h0       optional (batch, dim, dstate) float32 initial state; NULL = zeros (mamba.py:314).
+ *   h_ckpt   optional float32 buffer of mpa_sscan_ckpt_elems() elements: the state after
+ *            every MPA_CKPT_STEPS-th step, consumed by mpa_sscan_bwd; NULL when no
+ *            gradient is needed.
+ *   h_last   optional (batch, dim, dstate) float32: state after the last step, in the
+ *            layout of the decode cache `h` (mamba.py:335, 341).
+ */
+int mpa_sscan_fwd(const mpa_sscan_shape* s, const void* x, const void* delta, const float* A,
+                  const void* B, const void* C, const float* D, const void* z,
+                  const float* delta_bias, const float* h0, void* y, float* h_ckpt,
+                  float* h_last, void* stream);
+
+/* Number of float32 elements of the h_ckpt buffer for this shape. */
+int64_t mpa_sscan_ckpt_elems(const mpa_sscan_shape* s);
+
+/* ---- fused selective scan, backward -----------------------------------------------------
+ * Replaces what autograd records for mamba.py:284-293 plus PScan.backward
+ * (mambapy/pscan.py:188-224): given dy it writes dx, ddelta (io_dtype), dB, dC (io_dtype),
+ * dA (dim, dstate) and dD (dim) (float32, overwritten, not accumulated).
+ * h_ckpt is the buffer mpa_sscan_fwd filled for the same inputs.  The gate z, delta_bias /
+ * MPA_SSCAN_DELTA_SOFTPLUS and h0 must be the ones given to the forward call; dz (io_dtype,
+ * u-strides of g_*) is required when z is given, ddelta is then the gradient w.r.t. the
+ * raw (pre-softplus) delta, and ddelta_bias (dim) float32 is written when delta_bias is
+ * given.  `workspace` needs mpa_sscan_bwd_workspace_bytes() bytes, 256-byte aligned.
+ */
+int mpa_sscan_bwd(const mpa_sscan_shape* s, const void* x, const void* delta, const float* A,
+                  const void* B, const void* C, const float* D, const void* z,
+                  const float* delta_bias, const float* h0, const void* dy,
+                  const float* h_ckpt, void* dx, void* ddelta, float* dA, void* dB, void* dC,
+                  float* dD, void* dz, float* ddelta_bias, void* workspace,
+                  size_t workspace_bytes, void* stream);
+
+size_t mpa_sscan_bwd_workspace_bytes(const mpa_sscan_shape* s);
+
+/* ---- generic first-order scan -----------------------------------------------------------
+ * Replaces pscan = PScan.apply (mambapy/pscan.py:226; forward :151-186, backward :188-224)
+ * for callers that hold materialised A, X of logical shape (batch, seqlen, dim, dstate):
+ * H[t] = A[t]*H[t-1] + X[t], H[-1] = 0.  Strides are (sb, sl, sd, sn) element strides, one
+ * set per tensor; any seqlen.  H is a new tensor: inputs are never modified
+ * (pscan.py:167-174 clones).  Backward: gradX[t] = gradH[t] + A[t+1]*gradX[t+1],
+ * gradA[t] = H[t-1]*gradX[t], gradA[0] = 0 (pscan.py:216-222).
+ */
+typedef struct mpa_pscan_shape {
+    int64_t batch, seqlen, dim, dstate;
+    int32_t io_dtype;
+    int32_t reverse;          /* 1: scan from the last step to the first (pscan.py:94-149) */
+    int64_t a_st[4];          /* A     (sb, sl, sd, sn) */
+    int64_t x_st[4];          /* X or gradH */
+    int64_t h_st[4];          /* H (output of fwd, input of bwd) */
+    int64_t ga_st[4];         /* gradA */
+    int64_t gx_st[4];         /* gradX */
+} mpa_pscan_shape;
+
+int mpa_pscan_fwd(const mpa_pscan_shape* s, const void* A, const void* X, void* H, void* stream);
+int mpa_pscan_bwd(const mpa_pscan_shape* s, const void* A, const void* H, const void* gradH,
+                  void* gradA, void* gradX, void* stream);
+
+/* ---- decode step --------------------------------------------------------------------------
+ * Replaces the state update and readout of MambaBlock.ssm_step (mambapy/mamba.py:400-412)
+ * for one token: h' = exp(delta*A)*h + delta*B*x ; y = C.h' + D*x, optionally
+ * delta = softplus(delta + delta_bias) (mamba.py:398) and y *= silu(z) (mamba.py:373-375).
+ *   x, delta, z, y : (batch, dim) io_dtype contiguous;  B, C : (batch, dstate) io_dtype,
+ *   row stride bc_stride;  h_in, h_out : (batch, dim, dstate) float32 contiguous.
+ * h_in == NULL means zeros (mamba.py:405-406).  h_out may equal h_in (in-place update);
+ * with distinct buffers h_in is left untouched, which is the reference's behaviour
+ * (ssm_step returns a new tensor).
+ */
+int mpa_ssm_step(const void* x, const void* delta, const float* A, const void* B, const void* C,
+                 const float* D, const void* z, const float* delta_bias, const float* h_in,
+                 float* h_out, void* y, int64_t batch, int64_t dim, int64_t dstate,
+                 int64_t bc_stride, int32_t io_dtype, int32_t delta_softplus, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MAMBAPY_AMD_H */

@@ -1,0 +1,18 @@
+"""mambapy_amd: MI355X (gfx950) kernels for the selective-scan hot path of alxndrTL/mamba.py.
+
+The directory is named `mamba.py_amd`; import it as `mambapy_amd` (or
+`__graft_entry__.load_package()`).
+"""
+from . import _lib
+from .scan import PScan, pscan, selective_scan, selective_scan_fn, ssm_step, SelectiveScanFn
+
+__all__ = ["PScan", "pscan", "selective_scan", "selective_scan_fn", "ssm_step",
+           "SelectiveScanFn", "library_path", "library_version"]
+
+
+def library_path() -> str:
+    return _lib.LIB_PATH
+
+
+def library_version() -> int:
+    return _lib.load().mpa_version()

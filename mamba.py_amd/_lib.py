@@ -1,0 +1,77 @@
+"""ctypes binding of libmambapy_amd.so (declarations: include/mambapy_amd.h).
+
+There is no fallback: if the library is missing or cannot be loaded, importing the ops
+raises ImportError with the build command; nothing here computes on the CPU.
+"""
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "csrc", "libmambapy_amd.so")
+
+MPA_F32, MPA_BF16 = 0, 1
+MPA_SSCAN_DELTA_SOFTPLUS = 1
+MPA_CKPT_STEPS = 16
+MPA_MAX_DSTATE = 256
+
+EXPORTS = ("mpa_version", "mpa_arch", "mpa_status_string", "mpa_sscan_fwd",
+           "mpa_sscan_ckpt_elems", "mpa_sscan_bwd", "mpa_sscan_bwd_workspace_bytes",
+           "mpa_pscan_fwd", "mpa_pscan_bwd", "mpa_ssm_step")
+
+
+class SscanShape(ctypes.Structure):
+    _fields_ = [(n, ctypes.c_int64) for n in ("batch", "seqlen", "dim", "dstate")] + \
+               [("io_dtype", ctypes.c_int32), ("flags", ctypes.c_int32)] + \
+               [(n, ctypes.c_int64) for n in (
+                   "u_sb", "u_sl", "u_sd", "d_sb", "d_sl", "d_sd", "y_sb", "y_sl", "y_sd",
+                   "g_sb", "g_sl", "g_sd", "bc_sb", "bc_sl", "dbc_sb", "dbc_sl")]
+
+
+class PscanShape(ctypes.Structure):
+    _fields_ = [(n, ctypes.c_int64) for n in ("batch", "seqlen", "dim", "dstate")] + \
+               [("io_dtype", ctypes.c_int32), ("reverse", ctypes.c_int32)] + \
+               [(n, ctypes.c_int64 * 4) for n in ("a_st", "x_st", "h_st", "ga_st", "gx_st")]
+
+
+_lib = None
+
+
+def load():
+    """Open the library once; raise ImportError (never fall back) when it is not there."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise ImportError(
+            f"{LIB_PATH} is missing: build it with `python mamba.py_amd/build.py` "
+            "(needs hipcc; targets gfx950).  There is no CPU or PyTorch fallback.")
+    try:
+        lib = ctypes.CDLL(LIB_PATH)
+    except OSError as e:  # pragma: no cover - depends on the machine
+        raise ImportError(f"cannot load {LIB_PATH}: {e}") from e
+    vp, i64, i32, sz = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int32, ctypes.c_size_t
+    lib.mpa_version.restype = ctypes.c_int
+    lib.mpa_arch.restype = ctypes.c_char_p
+    lib.mpa_status_string.restype = ctypes.c_char_p
+    lib.mpa_status_string.argtypes = [ctypes.c_int]
+    sp = ctypes.POINTER(SscanShape)
+    lib.mpa_sscan_fwd.argtypes = [sp] + [vp] * 13
+    lib.mpa_sscan_ckpt_elems.argtypes = [sp]
+    lib.mpa_sscan_ckpt_elems.restype = i64
+    lib.mpa_sscan_bwd.argtypes = [sp] + [vp] * 20 + [sz, vp]
+    lib.mpa_sscan_bwd_workspace_bytes.argtypes = [sp]
+    lib.mpa_sscan_bwd_workspace_bytes.restype = sz
+    pp = ctypes.POINTER(PscanShape)
+    lib.mpa_pscan_fwd.argtypes = [pp] + [vp] * 4
+    lib.mpa_pscan_bwd.argtypes = [pp] + [vp] * 6
+    lib.mpa_ssm_step.argtypes = [vp] * 11 + [i64] * 4 + [i32, i32, vp]
+    for name in EXPORTS:
+        getattr(lib, name)
+    _lib = lib
+    return lib
+
+
+def check(status: int, what: str) -> None:
+    if status != 0:
+        msg = load().mpa_status_string(status).decode()
+        raise RuntimeError(f"{what} failed with status {status}: {msg}")

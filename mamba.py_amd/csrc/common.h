@@ -1,0 +1,92 @@
+// Shared device helpers for the gfx950 selective-scan kernels.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdlib.h>
+
+#include "../../include/mambapy_amd.h"
+
+namespace mpa {
+
+constexpr int kWave = 64;             // CDNA wavefront width
+constexpr int kTile = MPA_CKPT_STEPS; // time steps staged in LDS per iteration
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+
+struct bf16_t {
+    uint16_t bits;
+};
+
+__device__ __forceinline__ float to_float(float v) { return v; }
+__device__ __forceinline__ float to_float(bf16_t v) {
+    return __uint_as_float(static_cast<uint32_t>(v.bits) << 16);
+}
+
+template <typename T>
+__device__ __forceinline__ T from_float(float v);
+template <>
+__device__ __forceinline__ float from_float<float>(float v) {
+    return v;
+}
+// round-to-nearest-even; NaN stays NaN (quiet bit forced)
+template <>
+__device__ __forceinline__ bf16_t from_float<bf16_t>(float v) {
+    uint32_t u = __float_as_uint(v);
+    uint32_t r;
+    if ((u & 0x7fffffffu) > 0x7f800000u) {
+        r = (u >> 16) | 0x40u;
+    } else {
+        r = (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
+    }
+    return bf16_t{static_cast<uint16_t>(r)};
+}
+
+template <typename T>
+__device__ __forceinline__ float load_as_float(const void* p, int64_t i) {
+    return to_float(static_cast<const T*>(p)[i]);
+}
+template <typename T>
+__device__ __forceinline__ void store_from_float(void* p, int64_t i, float v) {
+    static_cast<T*>(p)[i] = from_float<T>(v);
+}
+
+// 2^x on the transcendental unit (v_exp_f32)
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+__device__ __forceinline__ float softplus_f(float v) {
+    // log(1 + e^v); linear above 20 like torch.nn.functional.softplus
+    return v > 20.0f ? v : log1pf(__expf(v));
+}
+__device__ __forceinline__ float sigmoid_f(float v) { return 1.0f / (1.0f + __expf(-v)); }
+
+__device__ __forceinline__ int wave_id() {
+    // threadIdx.x / 64, told to the compiler as wave-uniform
+    return __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x) >> 6);
+}
+
+inline int check_launch() { return hipGetLastError() == hipSuccess ? MPA_OK : MPA_ERR_LAUNCH; }
+
+inline bool aligned_to(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
+
+inline size_t dtype_size(int dt) { return dt == MPA_BF16 ? 2 : 4; }
+
+// states owned by one lane of a scan wave, chosen from the problem size so that the launch
+// fills the 1024 SIMDs of the chip (the only parallel axes are batch*dim and d_state)
+int pick_states_per_lane(int64_t batch, int64_t dim, int64_t dstate, int ns_max, const char* env);
+int padded_states(int64_t n);
+int validate_shape(const mpa_sscan_shape* s);
+
+// Kernels may use more LDS than the 64 KB a static __shared__ array can hold (gfx950 has
+// 160 KB per CU), so they take dynamic LDS; the limit is raised once per kernel.
+template <typename K>
+inline int allow_dynamic_lds(K kernel, size_t bytes) {
+    if (bytes > 160 * 1024) return MPA_ERR_BAD_SHAPE;
+    return hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                               hipFuncAttributeMaxDynamicSharedMemorySize,
+                               static_cast<int>(bytes)) == hipSuccess
+               ? MPA_OK
+               : MPA_ERR_LAUNCH;
+}
+
+}  // namespace mpa

@@ -1,0 +1,567 @@
+// Fused selective-scan backward for gfx950.
+//
+// Same decomposition as the forward pass: a workgroup owns 64 channels of one batch row and
+// its NW waves split d_state, NS states per lane.  The sequence is walked from the last
+// chunk of kTile steps to the first.  For each chunk a wave
+//   1. reloads the state at the chunk start from the checkpoints the forward pass wrote and
+//      recomputes the kTile steps, keeping a[t] and a[t]*h[t-1] of every step in registers
+//      (the recurrence is never inverted: dividing by a[t] amplifies rounding error);
+//   2. sweeps the chunk backwards with the reverse recurrence
+//          g[t] = dy[t]*C[t] + a[t+1]*g[t+1]
+//      and forms, per state and step,
+//          d(delta*A) = g*a*h[t-1]      -> dA += .*delta,  ddelta += .*A
+//          sum_n g*B                    -> dx = delta*., ddelta += x*.
+//          g*u (u = delta*x)            -> dB (summed over channels)
+//          dy*h[t]                      -> dC (summed over channels)
+// Reductions: over d_state across the NW waves through LDS (phase C, like the forward
+// readout); over the 64 channels of a wave by a wave-private LDS transposition every four
+// steps; over channel groups, batch and time by deterministic partial buffers that a small
+// second kernel sums (no floating-point atomics: results are bitwise reproducible).
+#include "common.h"
+
+namespace mpa {
+
+struct BwdParams {
+    const void* x;
+    const void* delta;
+    const void* Bm;
+    const void* C;
+    const void* z;
+    const void* dy;
+    const float* A;
+    const float* D;
+    const float* dbias;
+    const float* h0;
+    const float* ckpt;
+    void* dx;
+    void* ddelta;
+    void* dz;
+    float* partB;   // [CG][batch][L][N]
+    float* partC;   // [CG][batch][L][N]
+    float* partA;   // [batch][ED][N]
+    float* partD;   // [batch][ED]
+    float* partDb;  // [batch][ED]  (ddelta_bias)
+    int batch, L, ED, N, nchunks;
+    int softplus;
+    int in_tmajor, dy_tmajor, out_tmajor;
+    int64_t u_sb, u_sl, u_sd;
+    int64_t d_sb, d_sl, d_sd;
+    int64_t y_sb, y_sl, y_sd;
+    int64_t g_sb, g_sl, g_sd;
+    int64_t bc_sb, bc_sl;
+};
+
+constexpr int kPitchB = kWave + 1;
+constexpr int kRedPitch = kWave + 4;  // keeps 16-byte row alignment, conflict-free b128 reads
+
+__device__ __forceinline__ void wave_lds_sync() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+// LDS budget (160 KB per CU).  PS = steps per cross-wave reduction (phase C): a 16-wave
+// workgroup reduces twice per chunk so that its partial buffers stay at 8 steps.  kRows = rows
+// of one wave's channel-reduction buffer (two per state and step); RS = steps between two
+// channel reductions.
+template <int NS, int NW>
+struct BwdLds {
+    static constexpr int NP = NS * NW;
+    static constexpr int PS = NW == 16 ? kTile / 2 : kTile;
+    static constexpr int kRows = 128 / NW;
+    static constexpr int RS = kRows / (2 * NS);
+    static_assert(RS >= 1 && RS <= 4, "unsupported (NS, NW)");
+    static constexpr size_t floats(bool has_z) {
+        return (size_t)5 * kTile * kPitchB + (size_t)(has_z ? 3 : 2) * NW * PS * kPitchB +
+               2 * kTile * NP + (size_t)NW * kRows * kRedPitch;
+    }
+};
+
+template <typename IO, int NS, int NW, bool HAS_Z>
+__global__ void __launch_bounds__(NW* kWave) sscan_bwd_kernel(const BwdParams p) {
+    constexpr int NT = NW * kWave;
+    constexpr int NP = NS * NW;
+    constexpr int EPT = (kTile * kWave + NT - 1) / NT;
+    constexpr int BPT = (kTile * NP + NT - 1) / NT;
+    constexpr int PS = BwdLds<NS, NW>::PS;
+    constexpr int NSEG = kTile / PS;
+    constexpr int EPS = (PS * kWave + NT - 1) / NT;  // phase-C elements per thread
+    constexpr int kRows = BwdLds<NS, NW>::kRows;
+    constexpr int RS = BwdLds<NS, NW>::RS;
+    constexpr int LPR = kWave / kRows;  // lanes that share one reduction row
+    static_assert(kRows <= kWave && LPR >= 1, "reduction rows must fit one wave");
+
+    extern __shared__ float smem[];
+    typedef float Tile[kTile][kPitchB];
+    typedef float Part[PS][kPitchB];
+    typedef float TileN[kTile][NP];
+    typedef float RedBuf[kRows][kRedPitch];
+    Tile* sDelta = reinterpret_cast<Tile*>(smem);  // [1]
+    Tile* sU = sDelta + 1;
+    Tile* sX = sU + 1;
+    Tile* sDy = sX + 1;
+    Tile* sZg = sDy + 1;       // ungated dy when HAS_Z (else unused)
+    TileN* sB = reinterpret_cast<TileN*>(sZg + 1);
+    TileN* sC = sB + 1;
+    RedBuf* sR = reinterpret_cast<RedBuf*>(sC + 1);  // [NW]
+    Part* sP1 = reinterpret_cast<Part*>(sR + NW);     // [NW] sum_n g*B
+    Part* sP2 = sP1 + NW;      // [NW] sum_n g*a*h[t-1]*A*log2(e)
+    Part* sP3 = sP2 + NW;      // [NW] sum_n C*h, HAS_Z only
+
+    const int tid = threadIdx.x;
+    const int lane = tid & (kWave - 1);
+    const int w = wave_id();
+    const int b = blockIdx.y;
+    const int cg = blockIdx.x;
+    const int d0 = cg * kWave;
+    const int d = d0 + lane;
+    const bool dvalid = d < p.ED;
+
+    float A2[NS], ag[NS], dAacc[NS];
+#pragma unroll
+    for (int i = 0; i < NS; ++i) {
+        const int n = w * NS + i;
+        A2[i] = (dvalid && n < p.N) ? p.A[(int64_t)d * p.N + n] * kLog2e : 0.0f;
+        ag[i] = 0.0f;
+        dAacc[i] = 0.0f;
+    }
+    float dDacc[NSEG * EPS], dDbacc[NSEG * EPS];
+#pragma unroll
+    for (int k = 0; k < NSEG * EPS; ++k) dDacc[k] = dDbacc[k] = 0.0f;
+
+    float rX[EPT], rDl[EPT], rDy[EPT], rZ[EPT], rB[BPT], rC[BPT], rH[NS];
+
+    auto elem_map = [&](int idx, bool tmajor, int& tt, int& cc) {
+        if (tmajor) {
+            tt = idx % kTile;
+            cc = idx / kTile;
+        } else {
+            tt = idx / kWave;
+            cc = idx % kWave;
+        }
+    };
+
+    auto prefetch = [&](int c) {
+        const int t0 = c * kTile;
+        const int tl = min(kTile, p.L - t0);
+#pragma unroll
+        for (int k = 0; k < EPT; ++k) {
+            const int idx = tid + k * NT;
+            int tt, cc;
+            elem_map(idx, p.in_tmajor, tt, cc);
+            float xv = 0.0f, dv = 0.0f, dyv = 0.0f, zv = 0.0f;
+            if (idx < kTile * kWave && tt < tl && d0 + cc < p.ED) {
+                const int64_t t = t0 + tt;
+                const int64_t ch = d0 + cc;
+                xv = load_as_float<IO>(p.x, b * p.u_sb + t * p.u_sl + ch * p.u_sd);
+                dv = load_as_float<IO>(p.delta, b * p.d_sb + t * p.d_sl + ch * p.d_sd);
+                dyv = load_as_float<IO>(p.dy, b * p.y_sb + t * p.y_sl + ch * p.y_sd);
+                if (HAS_Z) zv = load_as_float<IO>(p.z, b * p.u_sb + t * p.u_sl + ch * p.u_sd);
+            }
+            rX[k] = xv;
+            rDl[k] = dv;
+            rDy[k] = dyv;
+            rZ[k] = zv;
+        }
+#pragma unroll
+        for (int k = 0; k < BPT; ++k) {
+            const int idx = tid + k * NT;
+            const int tt = idx / NP, n = idx % NP;
+            float bv = 0.0f, cv = 0.0f;
+            if (idx < kTile * NP && tt < tl && n < p.N) {
+                const int64_t off = b * p.bc_sb + (int64_t)(t0 + tt) * p.bc_sl + n;
+                bv = load_as_float<IO>(p.Bm, off);
+                cv = load_as_float<IO>(p.C, off);
+            }
+            rB[k] = bv;
+            rC[k] = cv;
+        }
+        // state at the start of chunk c = checkpoint written after chunk c-1
+#pragma unroll
+        for (int i = 0; i < NS; ++i) {
+            const int n = w * NS + i;
+            float hv = 0.0f;
+            if (dvalid && n < p.N) {
+                if (c > 0)
+                    hv = p.ckpt[(((int64_t)b * p.nchunks + (c - 1)) * p.N + n) * p.ED + d];
+                else if (p.h0)
+                    hv = p.h0[((int64_t)b * p.ED + d) * p.N + n];
+            }
+            rH[i] = hv;
+        }
+    };
+
+    // sDelta holds the delta the recurrence uses (after softplus); the raw value that the
+    // softplus derivative needs is recomputed from it: sigmoid(raw) = 1 - exp(-softplus(raw))
+    auto stage = [&](int tl) {
+#pragma unroll
+        for (int k = 0; k < EPT; ++k) {
+            const int idx = tid + k * NT;
+            int tt, cc;
+            elem_map(idx, p.in_tmajor, tt, cc);
+            if (idx < kTile * kWave) {
+                float dv = rDl[k];
+                const bool live = (tt < tl && d0 + cc < p.ED);
+                if (p.softplus && live) dv = softplus_f(dv + (p.dbias ? p.dbias[d0 + cc] : 0.0f));
+                float dyv = rDy[k];
+                if (HAS_Z) {
+                    const float zv = rZ[k];
+                    const float sg = sigmoid_f(zv);
+                    // keep the raw dy for dz; the recurrence sees dy * silu(z)
+                    sZg[0][tt][cc] = dyv;
+                    dyv = dyv * zv * sg;
+                }
+                sDelta[0][tt][cc] = dv;
+                sU[0][tt][cc] = dv * rX[k];
+                sX[0][tt][cc] = rX[k];
+                sDy[0][tt][cc] = dyv;
+            }
+        }
+#pragma unroll
+        for (int k = 0; k < BPT; ++k) {
+            const int idx = tid + k * NT;
+            if (idx < kTile * NP) {
+                sB[0][idx / NP][idx % NP] = rB[k];
+                sC[0][idx / NP][idx % NP] = rC[k];
+            }
+        }
+    };
+
+    const int last = p.nchunks - 1;
+    prefetch(last);
+    for (int c = last; c >= 0; --c) {
+        const int t0 = c * kTile;
+        const int tl = min(kTile, p.L - t0);
+        float h[NS];
+        // a tail chunk was prefetched with zero padding (delta = 0: a = 1, u = 0; dy = 0),
+        // which makes the padded steps exact no-ops in both sweeps
+        stage(tl);
+#pragma unroll
+        for (int i = 0; i < NS; ++i) h[i] = rH[i];
+        __syncthreads();
+        if (c > 0) prefetch(c - 1);
+
+        // ---- 1. recompute the chunk forward, keeping a and a*h[t-1] ----
+        float aS[kTile][NS], tS[kTile][NS];
+#pragma unroll
+        for (int tt = 0; tt < kTile; ++tt) {
+            const float dv = sDelta[0][tt][lane];
+            const float uv = sU[0][tt][lane];
+#pragma unroll
+            for (int i = 0; i < NS; ++i) {
+                const float a = fast_exp2(dv * A2[i]);
+                const float th = a * h[i];
+                aS[tt][i] = a;
+                tS[tt][i] = th;
+                h[i] = __builtin_fmaf(uv, sB[0][tt][w * NS + i], th);
+            }
+        }
+
+        // ---- 2. reverse sweep, in NSEG segments of PS steps, each followed by phase C ----
+#pragma unroll
+        for (int seg = NSEG - 1; seg >= 0; --seg) {
+#pragma unroll
+            for (int ts = PS - 1; ts >= 0; --ts) {
+                const int tt = seg * PS + ts;
+                const float dv = sDelta[0][tt][lane];
+                const float uv = sU[0][tt][lane];
+                const float dyv = sDy[0][tt][lane];
+                float gB = 0.0f, dd = 0.0f, yp = 0.0f;
+                const int slot = tt % RS;
+#pragma unroll
+                for (int i = 0; i < NS; ++i) {
+                    const float bv = sB[0][tt][w * NS + i];
+                    const float cv = sC[0][tt][w * NS + i];
+                    const float g = __builtin_fmaf(dyv, cv, ag[i]);
+                    const float hh = __builtin_fmaf(uv, bv, tS[tt][i]);
+                    const float gha = g * tS[tt][i];
+                    dAacc[i] = __builtin_fmaf(gha, dv, dAacc[i]);
+                    dd = __builtin_fmaf(gha, A2[i], dd);
+                    gB = __builtin_fmaf(g, bv, gB);
+                    ag[i] = aS[tt][i] * g;
+                    if (HAS_Z) yp = __builtin_fmaf(cv, hh, yp);
+                    sR[w][slot * 2 * NS + i][lane] = g * uv;
+                    sR[w][slot * 2 * NS + NS + i][lane] = dyv * hh;
+                }
+                sP1[w][ts][lane] = gB;
+                sP2[w][ts][lane] = dd;
+                if (HAS_Z) sP3[w][ts][lane] = yp;
+
+                if (slot == 0) {
+                    // channel reduction of the last RS steps: row r = (step, dB|dC, state);
+                    // LPR lanes share a row, each sums kWave/LPR consecutive channels
+                    wave_lds_sync();
+                    const int row = lane / LPR, part = lane % LPR;
+                    const float4* src =
+                        reinterpret_cast<const float4*>(&sR[w][row][part * (kWave / LPR)]);
+                    float s = 0.0f;
+#pragma unroll
+                    for (int j = 0; j < kWave / LPR / 4; ++j) {
+                        const float4 v = src[j];
+                        s += (v.x + v.y) + (v.z + v.w);
+                    }
+#pragma unroll
+                    for (int m = 1; m < LPR; m *= 2) s += __shfl_xor(s, m, kWave);
+                    const int rs = row / (2 * NS), o = row % (2 * NS);
+                    const int t = t0 + tt + rs;
+                    const int n = w * NS + (o % NS);
+                    if (part == 0 && t < p.L && n < p.N) {
+                        float* dst = (o < NS) ? p.partB : p.partC;
+                        dst[(((int64_t)cg * p.batch + b) * p.L + t) * p.N + n] = s;
+                    }
+                    wave_lds_sync();
+                }
+            }
+            __syncthreads();
+
+            // ---- phase C: sum over the waves, finish dx / ddelta (/ dz), accumulate dD ----
+#pragma unroll
+            for (int k = 0; k < EPS; ++k) {
+                const int idx = tid + k * NT;
+                int ts, cc;
+                if (p.out_tmajor) {
+                    ts = idx % PS;
+                    cc = idx / PS;
+                } else {
+                    ts = idx / kWave;
+                    cc = idx % kWave;
+                }
+                const int tt = seg * PS + ts;
+                if (idx < PS * kWave && tt < tl && d0 + cc < p.ED) {
+                    float gB = 0.0f, dd = 0.0f;
+#pragma unroll
+                    for (int ww = 0; ww < NW; ++ww) {
+                        gB += sP1[ww][ts][cc];
+                        dd += sP2[ww][ts][cc];
+                    }
+                    const float xv = sX[0][tt][cc];
+                    const float dv = sDelta[0][tt][cc];
+                    const float dyg = sDy[0][tt][cc];  // dy, already gated when HAS_Z
+                    const float Dv = p.D[d0 + cc];
+                    const int64_t t = t0 + tt;
+                    const int64_t ch = d0 + cc;
+                    const float dxv = __builtin_fmaf(dv, gB, Dv * dyg);
+                    float ddv = __builtin_fmaf(xv, gB, dd * kLn2);
+                    dDacc[seg * EPS + k] = __builtin_fmaf(dyg, xv, dDacc[seg * EPS + k]);
+                    if (p.softplus) {
+                        // d softplus(r)/dr = sigmoid(r) = 1 - exp(-softplus(r))
+                        ddv *= (1.0f - __expf(-dv));
+                        dDbacc[seg * EPS + k] += ddv;
+                    }
+                    store_from_float<IO>(p.dx, b * p.g_sb + t * p.g_sl + ch * p.g_sd, dxv);
+                    store_from_float<IO>(p.ddelta, b * p.g_sb + t * p.g_sl + ch * p.g_sd, ddv);
+                    if (HAS_Z) {
+                        float yp = 0.0f;
+#pragma unroll
+                        for (int ww = 0; ww < NW; ++ww) yp += sP3[ww][ts][cc];
+                        yp = __builtin_fmaf(Dv, xv, yp);  // pre-gate output
+                        const float zv =
+                            load_as_float<IO>(p.z, b * p.u_sb + t * p.u_sl + ch * p.u_sd);
+                        const float sg = sigmoid_f(zv);
+                        const float dyraw = sZg[0][tt][cc];
+                        // d(z*sigmoid(z))/dz = sg * (1 + z*(1-sg))
+                        const float dzv = dyraw * yp * sg * (1.0f + zv * (1.0f - sg));
+                        store_from_float<IO>(p.dz, b * p.g_sb + t * p.g_sl + ch * p.g_sd, dzv);
+                    }
+                }
+            }
+            __syncthreads();
+        }
+    }
+
+    // ---- epilogue: per-batch partials of dA, dD (and ddelta_bias) ----
+    if (dvalid) {
+#pragma unroll
+        for (int i = 0; i < NS; ++i) {
+            const int n = w * NS + i;
+            if (n < p.N) p.partA[((int64_t)b * p.ED + d) * p.N + n] = dAacc[i];
+        }
+    }
+    // dD: every thread holds sums for its fixed (step slot, channel) elements; reduce over
+    // the step slots through LDS (sDelta .. sDy are free now: use them as one [kTile] tile)
+    for (int pass = 0; pass < (p.softplus ? 2 : 1); ++pass) {
+#pragma unroll
+        for (int seg = 0; seg < NSEG; ++seg) {
+#pragma unroll
+            for (int k = 0; k < EPS; ++k) {
+                const int idx = tid + k * NT;
+                int ts, cc;
+                if (p.out_tmajor) {
+                    ts = idx % PS;
+                    cc = idx / PS;
+                } else {
+                    ts = idx / kWave;
+                    cc = idx % kWave;
+                }
+                if (idx < PS * kWave)
+                    sDelta[0][seg * PS + ts][cc] =
+                        pass == 0 ? dDacc[seg * EPS + k] : dDbacc[seg * EPS + k];
+            }
+        }
+        __syncthreads();
+        if (tid < kWave && d0 + tid < p.ED) {
+            float s = 0.0f;
+#pragma unroll
+            for (int tt = 0; tt < kTile; ++tt) s += sDelta[0][tt][tid];
+            float* dst = pass == 0 ? p.partD : p.partDb;
+            dst[(int64_t)b * p.ED + d0 + tid] = s;
+        }
+        __syncthreads();
+    }
+}
+
+// Sums the partial buffers: dB/dC over channel groups, dA/dD/ddelta_bias over the batch.
+template <typename IO>
+__global__ void __launch_bounds__(256) sscan_bwd_finish_kernel(
+    const float* partB, const float* partC, const float* partA, const float* partD,
+    const float* partDb, void* dB, void* dC, float* dA, float* dD, float* dDb, int CG, int batch,
+    int L, int ED, int N, int64_t dbc_sb, int64_t dbc_sl) {
+    const int64_t bln = (int64_t)batch * L * N;
+    const int64_t edn = (int64_t)ED * N;
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < bln) {
+        float sb = 0.0f, sc = 0.0f;
+        for (int g = 0; g < CG; ++g) {
+            sb += partB[g * bln + i];
+            sc += partC[g * bln + i];
+        }
+        const int n = (int)(i % N);
+        const int64_t bt = i / N;
+        const int64_t off = (bt / L) * dbc_sb + (bt % L) * dbc_sl + n;
+        store_from_float<IO>(dB, off, sb);
+        store_from_float<IO>(dC, off, sc);
+    } else if (i < bln + edn) {
+        const int64_t j = i - bln;
+        float s = 0.0f;
+        for (int bb = 0; bb < batch; ++bb) s += partA[bb * edn + j];
+        dA[j] = s;
+    } else if (i < bln + edn + ED) {
+        const int64_t j = i - bln - edn;
+        float s = 0.0f, sdb = 0.0f;
+        for (int bb = 0; bb < batch; ++bb) {
+            s += partD[(int64_t)bb * ED + j];
+            if (dDb) sdb += partDb[(int64_t)bb * ED + j];
+        }
+        dD[j] = s;
+        if (dDb) dDb[j] = sdb;
+    }
+}
+
+struct BwdWorkspace {
+    size_t offB, offC, offA, offD, offDb, total;
+};
+
+static BwdWorkspace bwd_workspace(const mpa_sscan_shape* s) {
+    const size_t cg = (size_t)(s->dim + kWave - 1) / kWave;
+    const size_t bln = (size_t)s->batch * s->seqlen * s->dstate;
+    const size_t ben = (size_t)s->batch * s->dim * s->dstate;
+    const size_t be = (size_t)s->batch * s->dim;
+    auto up = [](size_t v) { return (v + 63) / 64 * 64; };  // 256-byte granules of floats
+    BwdWorkspace w;
+    w.offB = 0;
+    w.offC = w.offB + up(cg * bln);
+    w.offA = w.offC + up(cg * bln);
+    w.offD = w.offA + up(ben);
+    w.offDb = w.offD + up(be);
+    w.total = (w.offDb + up(be)) * sizeof(float);
+    return w;
+}
+
+template <typename IO, int NS, int NW, bool HAS_Z>
+static int launch_bwd(const BwdParams& p, hipStream_t stream) {
+    dim3 grid((p.ED + kWave - 1) / kWave, p.batch);
+    dim3 block(NW * kWave);
+    constexpr size_t lds = sizeof(float) * BwdLds<NS, NW>::floats(HAS_Z);
+    static const int attr_rc = allow_dynamic_lds(sscan_bwd_kernel<IO, NS, NW, HAS_Z>, lds);
+    if (attr_rc != MPA_OK) return attr_rc;
+    hipLaunchKernelGGL((sscan_bwd_kernel<IO, NS, NW, HAS_Z>), grid, block, lds, stream, p);
+    return check_launch();
+}
+
+template <typename IO, bool HAS_Z>
+static int dispatch_bwd(const BwdParams& p, int ns, int nw, hipStream_t stream) {
+#define MPA_CASE(NS_, NW_) \
+    if (ns == NS_ && nw == NW_) return launch_bwd<IO, NS_, NW_, HAS_Z>(p, stream);
+    MPA_CASE(1, 16) MPA_CASE(2, 8) MPA_CASE(4, 4)
+    MPA_CASE(2, 16) MPA_CASE(4, 8)
+    MPA_CASE(4, 16)
+#undef MPA_CASE
+    return MPA_ERR_BAD_SHAPE;
+}
+
+}  // namespace mpa
+
+using namespace mpa;
+
+extern "C" size_t mpa_sscan_bwd_workspace_bytes(const mpa_sscan_shape* s) {
+    if (validate_shape(s) != MPA_OK) return 0;
+    return bwd_workspace(s).total;
+}
+
+extern "C" int mpa_sscan_bwd(const mpa_sscan_shape* s, const void* x, const void* delta,
+                             const float* A, const void* B, const void* C, const float* D,
+                             const void* z, const float* delta_bias, const float* h0,
+                             const void* dy, const float* h_ckpt, void* dx, void* ddelta,
+                             float* dA, void* dB, void* dC, float* dD, void* dz,
+                             float* ddelta_bias, void* workspace, size_t workspace_bytes,
+                             void* stream) {
+    int rc = validate_shape(s);
+    if (rc != MPA_OK) return rc;
+    if (s->dstate > 64) return MPA_ERR_BAD_SHAPE;  // backward keeps <= 4 states per lane
+    if (!x || !delta || !A || !B || !C || !D || !dy || !h_ckpt || !dx || !ddelta || !dA || !dB ||
+        !dC || !dD || !workspace)
+        return MPA_ERR_NULL_POINTER;
+    if (z && !dz) return MPA_ERR_NULL_POINTER;
+    const bool softplus = (s->flags & MPA_SSCAN_DELTA_SOFTPLUS) != 0;
+    if (!softplus && (delta_bias || ddelta_bias)) return MPA_ERR_BAD_SHAPE;
+    if (delta_bias && !ddelta_bias) return MPA_ERR_NULL_POINTER;
+    const size_t es = dtype_size(s->io_dtype);
+    if (!aligned_to(x, es) || !aligned_to(delta, es) || !aligned_to(B, es) || !aligned_to(C, es) ||
+        !aligned_to(dy, es) || !aligned_to(dx, es) || !aligned_to(ddelta, es) ||
+        !aligned_to(dB, es) || !aligned_to(dC, es) || (z && !aligned_to(z, es)) ||
+        (dz && !aligned_to(dz, es)) || !aligned_to(workspace, 256))
+        return MPA_ERR_MISALIGNED;
+    const BwdWorkspace ws = bwd_workspace(s);
+    if (workspace_bytes < ws.total) return MPA_ERR_WORKSPACE;
+
+    float* wsf = static_cast<float*>(workspace);
+    BwdParams p{};
+    p.x = x; p.delta = delta; p.Bm = B; p.C = C; p.z = z; p.dy = dy; p.A = A; p.D = D;
+    p.dbias = delta_bias; p.h0 = h0; p.ckpt = h_ckpt; p.dx = dx; p.ddelta = ddelta; p.dz = dz;
+    p.partB = wsf + ws.offB; p.partC = wsf + ws.offC; p.partA = wsf + ws.offA;
+    p.partD = wsf + ws.offD; p.partDb = wsf + ws.offDb;
+    p.batch = (int)s->batch; p.L = (int)s->seqlen; p.ED = (int)s->dim; p.N = (int)s->dstate;
+    p.nchunks = (p.L + kTile - 1) / kTile;
+    p.softplus = softplus ? 1 : 0;
+    p.u_sb = s->u_sb; p.u_sl = s->u_sl; p.u_sd = s->u_sd;
+    p.d_sb = s->d_sb; p.d_sl = s->d_sl; p.d_sd = s->d_sd;
+    p.y_sb = s->y_sb; p.y_sl = s->y_sl; p.y_sd = s->y_sd;
+    p.g_sb = s->g_sb; p.g_sl = s->g_sl; p.g_sd = s->g_sd;
+    p.bc_sb = s->bc_sb; p.bc_sl = s->bc_sl;
+    p.in_tmajor = (s->u_sd != 1 && s->u_sl == 1) ? 1 : 0;
+    p.out_tmajor = (s->g_sd != 1 && s->g_sl == 1) ? 1 : 0;
+
+    const int np = padded_states(s->dstate);
+    const int ns = pick_states_per_lane(s->batch, s->dim, s->dstate, 4, "MPA_BWD_NS");
+    const int nw = np / ns;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (s->io_dtype == MPA_F32)
+        rc = z ? dispatch_bwd<float, true>(p, ns, nw, st) : dispatch_bwd<float, false>(p, ns, nw, st);
+    else
+        rc = z ? dispatch_bwd<bf16_t, true>(p, ns, nw, st)
+               : dispatch_bwd<bf16_t, false>(p, ns, nw, st);
+    if (rc != MPA_OK) return rc;
+
+    const int cg = (p.ED + kWave - 1) / kWave;
+    const int64_t total = (int64_t)p.batch * p.L * p.N + (int64_t)p.ED * p.N + p.ED;
+    dim3 fgrid((unsigned)((total + 255) / 256));
+    if (s->io_dtype == MPA_F32)
+        hipLaunchKernelGGL(sscan_bwd_finish_kernel<float>, fgrid, dim3(256), 0, st, p.partB, p.partC,
+                           p.partA, p.partD, softplus && ddelta_bias ? p.partDb : nullptr, dB, dC, dA, dD,
+                           ddelta_bias, cg, p.batch, p.L, p.ED, p.N, s->dbc_sb, s->dbc_sl);
+    else
+        hipLaunchKernelGGL(sscan_bwd_finish_kernel<bf16_t>, fgrid, dim3(256), 0, st, p.partB, p.partC,
+                           p.partA, p.partD, softplus && ddelta_bias ? p.partDb : nullptr, dB, dC, dA, dD,
+                           ddelta_bias, cg, p.batch, p.L, p.ED, p.N, s->dbc_sb, s->dbc_sl);
+    return check_launch();
+}
