@@ -1,0 +1,168 @@
+#!/usr/bin/env python3
+"""Benchmark of the selective-scan hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c1|c0]
+
+One step = one forward + one backward of the fused selective scan over one batch of
+seeded synthetic input that is already resident in HBM.  Prints ONE JSON line.
+  value      algorithmic GB/s of forward+backward (bytes formula below / time per step)
+  roofline   the backward entry point (its two kernels), HIP-event time on the launch stream
+  cpu_baseline  the CPU restatement of the reference's Blelloch-scan path (oracle "port"),
+             timed on this host on a bounded sample of the same workload
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
+
+WORKLOADS = {
+    # name: (B, L, ED, N, dtype, seed, description)
+    "c0": (2, 64, 32, 16, "float32", 1000, "configs[0]: B=2 L=64 ED=32 N=16 fp32"),
+    "c1": (8, 2048, 1536, 16, "float32", 1001, "configs[1]: mamba-130m layer B=8 L=2048 ED=1536 N=16 fp32"),
+    "c2": (4, 4096, 4096, 16, "bfloat16", 1002,
+           "configs[2]: mamba-1.4b layer B=4 L=4096 ED=4096 N=16, bf16 I/O, fp32 state"),
+}
+
+# HBM bytes per launch of the backward entry point measured with rocprofv3 --pmc
+# (FETCH_SIZE + WRITE_SIZE, scaled by a copy kernel of known size); filled from the
+# summaries under profiles/.  None = not measured for that workload.
+MEASURED_TRAFFIC_BYTES = {}
+
+
+def algorithmic_bytes(B, L, ED, N, s):
+    """Bytes that must cross HBM: fwd reads x, delta, B, C, A, D and writes y; bwd reads
+    x, delta, dy, B, C, A, D and writes dx, ddelta, dB, dC, dA, dD (s = I/O element size;
+    A, D, dA, dD float32).  Checkpoints, partial buffers and recomputation are not counted."""
+    fwd = s * (3 * B * L * ED + 2 * B * L * N) + 4 * (ED * N + ED)
+    bwd = s * (5 * B * L * ED + 4 * B * L * N) + 4 * (2 * ED * N + 2 * ED)
+    return fwd, bwd
+
+
+def cpu_baseline(workload, torch, so):
+    """Time the reference's pure-PyTorch path (materialised tensors + Blelloch scan,
+    forward + backward, float32, all host threads) on a slice of the workload's channels:
+    channels are independent, so the slice is the same work per channel."""
+    B, L, ED, N, _, seed, _ = WORKLOADS[workload]
+    ed = min(ED, 128 if workload != "c0" else ED)
+    bs = min(B, 2)
+    threads = int(os.environ.get("OMP_NUM_THREADS") or os.cpu_count() or 1)
+    torch.set_num_threads(threads)
+    inp = so.make_inputs(bs, L, ed, N, seed=seed)
+    names = ("x", "delta", "A", "B", "C", "D")
+
+    def once():
+        args = [inp[k].clone().requires_grad_() for k in names]
+        y = so.selective_scan_blelloch(*args)
+        y.backward(inp["dy"])
+        return y
+
+    once()
+    reps, t0 = 0, time.perf_counter()
+    while reps < 3 or (time.perf_counter() - t0 < 6.0 and reps < 20):
+        once()
+        reps += 1
+    dt = (time.perf_counter() - t0) / reps
+    fwd, bwd = algorithmic_bytes(bs, L, ed, N, 4)
+    return {
+        "value": (fwd + bwd) / dt / 1e9, "unit": "GB/s", "cores": threads, "kind": "port",
+        "sample": f"B={bs} L={L} ED={ed} of {ED} channels N={N} fp32, fwd+bwd, "
+                  f"{reps} reps, {dt * 1e3:.1f} ms each; GB/s on the same algorithmic-bytes formula",
+        "tokens_per_s_at_full_width": bs * L / dt * ed / ED,
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS))
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on ONE GPU (one process, one MI355X); "
+                 "--gpus N with N > 1 is not supported.")
+
+    import torch
+    import __graft_entry__ as entry
+    from oracle import scan_oracle as so
+    pkg = entry.load_package()
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible")
+    dev = torch.device("cuda:0")
+
+    B, L, ED, N, dtname, seed, desc = WORKLOADS[args.workload]
+    dtype = getattr(torch, dtname)
+    inp = so.make_inputs(B, L, ED, N, seed=seed, dtype=dtype)
+    names = ("x", "delta", "A", "B", "C", "D")
+    gpu = [inp[k].to(dev).requires_grad_() for k in names]
+    dy = inp["dy"].to(dev)
+    torch.cuda.synchronize()
+
+    def step(events=None):
+        for a in gpu:
+            a.grad = None
+        if events:
+            events[0].record()
+        y = pkg.selective_scan_fn(*gpu)
+        if events:
+            events[1].record()
+        y.backward(dy)
+        if events:
+            events[2].record()
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms_per_step = wall / args.steps * 1e3
+
+    # per-entry-point GPU time from HIP events recorded on the launch stream
+    evs = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(args.steps)]
+    for e in evs:
+        step(e)
+    torch.cuda.synchronize()
+    fwd_ms = sum(e[0].elapsed_time(e[1]) for e in evs) / len(evs)
+    bwd_ms = sum(e[1].elapsed_time(e[2]) for e in evs) / len(evs)
+
+    s = 2 if dtype == torch.bfloat16 else 4
+    fwd_b, bwd_b = algorithmic_bytes(B, L, ED, N, s)
+    gbs = (fwd_b + bwd_b) / (ms_per_step * 1e-3) / 1e9
+    bwd_gbs = bwd_b / (bwd_ms * 1e-3) / 1e9
+    out = {
+        "metric": "selective-scan fwd+bwd GB/s (% HBM peak) + tokens/s, 1.4b layer L=4096",
+        "value": gbs, "unit": "GB/s",
+        "pct_hbm_peak": 100.0 * gbs / HBM_PEAK_GBS,
+        "tokens_per_s": B * L / (ms_per_step * 1e-3),
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step,
+        "fwd_ms": fwd_ms, "bwd_ms": bwd_ms,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32 state/accumulation, " + ("bf16" if s == 2 else "f32") + " I/O",
+        "data": "synthetic (seeded, S4D-real A, softplus delta; values resident in HBM)",
+        "config": {"workload": desc, "B": B, "L": L, "ED": ED, "N": N,
+                   "algorithmic_bytes_fwd": fwd_b, "algorithmic_bytes_bwd": bwd_b},
+        "roofline": {"bound": "hbm", "kernel": "mpa_sscan_bwd (sscan_bwd_kernel + sscan_bwd_finish_kernel)",
+                     "achieved": bwd_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": bwd_gbs / HBM_PEAK_GBS,
+                     "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload)},
+        "forward": {"kernel": "mpa_sscan_fwd (sscan_fwd_kernel)",
+                    "achieved": fwd_b / (fwd_ms * 1e-3) / 1e9, "unit": "GB/s",
+                    "frac": fwd_b / (fwd_ms * 1e-3) / 1e9 / HBM_PEAK_GBS},
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(args.workload, torch, so)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

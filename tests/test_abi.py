@@ -1,0 +1,70 @@
+"""The C-ABI library loads and exports every symbol include/mambapy_amd.h declares, and
+rejects malformed calls with status codes (no GPU needed: nothing is launched)."""
+import ctypes
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "mambapy_amd.h")
+
+
+def _declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(mpa_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_declares_the_expected_entry_points():
+    names = _declared_functions()
+    for n in ("mpa_sscan_fwd", "mpa_sscan_bwd", "mpa_pscan_fwd", "mpa_pscan_bwd", "mpa_ssm_step",
+              "mpa_sscan_ckpt_elems", "mpa_sscan_bwd_workspace_bytes", "mpa_version", "mpa_arch"):
+        assert n in names
+
+
+def test_library_exports_every_declared_symbol(pkg):
+    lib = pkg._lib.load()
+    for n in _declared_functions():
+        assert hasattr(lib, n), f"{n} is declared in the header but not exported"
+    assert set(pkg._lib.EXPORTS) == set(_declared_functions())
+    assert lib.mpa_arch() == b"gfx950"
+    assert lib.mpa_version() == 100
+
+
+def test_status_codes_without_launch(pkg):
+    L = pkg._lib
+    lib = L.load()
+    s = L.SscanShape()
+    assert lib.mpa_sscan_fwd(None, *([None] * 13)) == 1          # MPA_ERR_NULL_POINTER
+    s.batch, s.seqlen, s.dim, s.dstate = 1, 0, 8, 16
+    assert lib.mpa_sscan_fwd(ctypes.byref(s), *([None] * 13)) == 2  # bad shape
+    s.seqlen, s.dstate = 8, 1000
+    assert lib.mpa_sscan_fwd(ctypes.byref(s), *([None] * 13)) == 2  # d_state too large
+    s.dstate, s.io_dtype = 16, 7
+    assert lib.mpa_sscan_fwd(ctypes.byref(s), *([None] * 13)) == 3  # bad dtype
+    s.io_dtype = 0
+    assert lib.mpa_sscan_fwd(ctypes.byref(s), *([None] * 13)) == 1  # null data pointers
+    assert lib.mpa_sscan_ckpt_elems(ctypes.byref(s)) == 1 * 1 * 16 * 8
+    assert lib.mpa_sscan_bwd_workspace_bytes(ctypes.byref(s)) > 0
+    assert lib.mpa_status_string(6) == b"workspace too small"
+    p = L.PscanShape()
+    assert lib.mpa_pscan_fwd(ctypes.byref(p), None, None, None, None) == 2
+
+
+def test_missing_library_is_a_loud_import_error(pkg, monkeypatch):
+    L = pkg._lib
+    monkeypatch.setattr(L, "_lib", None)
+    monkeypatch.setattr(L, "LIB_PATH", os.path.join(ROOT, "does", "not", "exist.so"))
+    with pytest.raises(ImportError, match="no CPU or PyTorch fallback"):
+        L.load()
+
+
+def test_cpu_tensors_are_rejected(pkg):
+    import torch
+    x = torch.zeros(1, 4, 8)
+    with pytest.raises(RuntimeError, match="ROCm device"):
+        pkg.selective_scan(x, x, torch.zeros(8, 16), torch.zeros(1, 4, 16), torch.zeros(1, 4, 16),
+                           torch.zeros(8))
+    with pytest.raises(RuntimeError, match="ROCm device"):
+        pkg.pscan(torch.zeros(1, 4, 8, 16), torch.zeros(1, 4, 8, 16))
