@@ -90,14 +90,20 @@ const char* mpa_status_string(int status);
  *            gradient is needed.
  *   h_last   optional (batch, dim, dstate) float32: state after the last step, in the
  *            layout of the decode cache `h` (mamba.py:335, 341).
+ *   workspace  scratch of mpa_sscan_fwd_workspace_bytes() bytes.
  */
 int mpa_sscan_fwd(const mpa_sscan_shape* s, const void* x, const void* delta, const float* A,
                   const void* B, const void* C, const float* D, const void* z,
                   const float* delta_bias, const float* h0, void* y, float* h_ckpt,
-                  float* h_last, void* stream);
+                  float* h_last, void* workspace, size_t workspace_bytes, void* stream);
 
 /* Number of float32 elements of the h_ckpt buffer for this shape. */
 int64_t mpa_sscan_ckpt_elems(const mpa_sscan_shape* s);
+
+/* Bytes of the scratch `workspace` of mpa_sscan_fwd (256-byte aligned; holds B and C
+ * repacked as float32 in the order the scan waves read them; contents are dead after the
+ * call). */
+size_t mpa_sscan_fwd_workspace_bytes(const mpa_sscan_shape* s);
 
 /* ---- fused selective scan, backward -----------------------------------------------------
  * Replaces what autograd records for mamba.py:284-293 plus PScan.backward

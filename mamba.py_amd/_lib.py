@@ -15,7 +15,7 @@ MPA_CKPT_STEPS = 16
 MPA_MAX_DSTATE = 256
 
 EXPORTS = ("mpa_version", "mpa_arch", "mpa_status_string", "mpa_sscan_fwd",
-           "mpa_sscan_ckpt_elems", "mpa_sscan_bwd", "mpa_sscan_bwd_workspace_bytes",
+           "mpa_sscan_ckpt_elems", "mpa_sscan_fwd_workspace_bytes", "mpa_sscan_bwd", "mpa_sscan_bwd_workspace_bytes",
            "mpa_pscan_fwd", "mpa_pscan_bwd", "mpa_ssm_step")
 
 
@@ -55,7 +55,9 @@ def load():
     lib.mpa_status_string.restype = ctypes.c_char_p
     lib.mpa_status_string.argtypes = [ctypes.c_int]
     sp = ctypes.POINTER(SscanShape)
-    lib.mpa_sscan_fwd.argtypes = [sp] + [vp] * 13
+    lib.mpa_sscan_fwd.argtypes = [sp] + [vp] * 13 + [sz, vp]
+    lib.mpa_sscan_fwd_workspace_bytes.argtypes = [sp]
+    lib.mpa_sscan_fwd_workspace_bytes.restype = sz
     lib.mpa_sscan_ckpt_elems.argtypes = [sp]
     lib.mpa_sscan_ckpt_elems.restype = i64
     lib.mpa_sscan_bwd.argtypes = [sp] + [vp] * 20 + [sz, vp]

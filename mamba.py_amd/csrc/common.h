@@ -76,6 +76,10 @@ inline size_t dtype_size(int dt) { return dt == MPA_BF16 ? 2 : 4; }
 int pick_states_per_lane(int64_t batch, int64_t dim, int64_t dstate, int ns_max, const char* env);
 int padded_states(int64_t n);
 int validate_shape(const mpa_sscan_shape* s);
+// B and C repacked as float32 for scalar loads (see pack_bc_kernel in sscan_fwd.hip)
+size_t bcpack_floats(const mpa_sscan_shape* s);
+int launch_pack_bc(const mpa_sscan_shape* s, const void* B, const void* C, float* out, int ns,
+                   hipStream_t st);
 
 // Kernels may use more LDS than the 64 KB a static __shared__ array can hold (gfx950 has
 // 160 KB per CU), so they take dynamic LDS; the limit is raised once per kernel.

@@ -542,7 +542,8 @@ extern "C" int mpa_sscan_bwd(const mpa_sscan_shape* s, const void* x, const void
     p.out_tmajor = (s->g_sd != 1 && s->g_sl == 1) ? 1 : 0;
 
     const int np = padded_states(s->dstate);
-    const int ns = pick_states_per_lane(s->batch, s->dim, s->dstate, 4, "MPA_BWD_NS");
+    int ns = pick_states_per_lane(s->batch, s->dim, s->dstate, 4, "MPA_BWD_NS");
+    if (ns < 0) ns = 4;
     const int nw = np / ns;
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (s->io_dtype == MPA_F32)

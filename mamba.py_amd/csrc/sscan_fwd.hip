@@ -1,20 +1,26 @@
 // Fused selective-scan forward for gfx950: discretise -> scan -> readout in one pass.
 //
 // Work decomposition.  The recurrence h[t] = a[t]*h[t-1] + bx[t] is serial in t and
-// independent per (batch, channel, state).  A workgroup owns 64 channels of one batch row;
-// its NW waves split the d_state axis: wave w keeps NS states (n = w*NS .. w*NS+NS-1) of the
-// 64 channels in registers, one channel per lane, and walks the sequence in time order.
-// Per state and step the VALU work is one multiply for the exponent, one v_exp_f32, one
-// multiply a*h, one fma for +u*B and one fma for the readout; nothing else scales with N.
+// independent per (batch, channel, state); with N = 16 there is nothing to contract, so the
+// kernel is bound by fp32 VALU issue (one v_exp_f32 and four multiply/fma per state and
+// step), not by HBM.  Everything is organised to keep the VALU fed:
 //
-// Per tile of kTile steps:
-//   A. the whole workgroup converts the (kTile x 64) slices of delta and x to float32 in LDS
-//      (delta, u = delta*x, x), and the (kTile x N) slices of B and C; the global loads of
-//      the NEXT tile are issued before the arithmetic of this one (register prefetch);
-//   B. every wave runs its NS recurrences and writes a partial readout sum_n C*h to LDS;
-//   C. the workgroup sums the NW partials, adds D*x, applies the optional gate and stores y.
-// Both channel-contiguous and time-contiguous (B,ED,L memory) operands are read and written
-// coalesced: the thread -> (step, channel) map of phases A and C follows the unit stride.
+//  * A workgroup owns 64 channels of one batch row.  NW "scan" waves split the d_state axis:
+//    wave w keeps NS states (n = w*NS ..) of the 64 channels in registers, one channel per
+//    lane, and walks the sequence in tiles of kTile steps.
+//  * Four "service" waves do everything that is per (step, channel) rather than per state,
+//    one tile ahead / behind the scan waves: they load x, delta (z) from HBM, convert them,
+//    apply softplus, form u = delta*x and D*x, and publish float32 tiles in LDS; one tile
+//    later they sum the NW partial readouts, apply the gate and store y.  Scan and service
+//    waves meet at ONE workgroup barrier per tile, so HBM latency, conversions and the
+//    cross-wave reduction overlap with the recurrence arithmetic instead of preceding it.
+//  * B and C are wave-uniform (they do not depend on the channel).  A small pre-pass packs
+//    them as float32 in the order each scan wave consumes them, and the scan waves fetch
+//    them with scalar loads into SGPRs: no LDS traffic, no vector registers, no conversions
+//    in the loop.
+//  * Both channel-contiguous and time-contiguous ((B,ED,L) memory) operands are read and
+//    written coalesced: a service thread owns 4 consecutive steps of one channel, and the
+//    thread -> (channel, step group) map follows the unit-stride axis.
 #include "common.h"
 
 namespace mpa {
@@ -22,13 +28,12 @@ namespace mpa {
 struct FwdParams {
     const void* x;
     const void* delta;
-    const void* Bm;
-    const void* C;
     const void* z;
     const float* A;
     const float* D;
     const float* dbias;
     const float* h0;
+    const float* bcpack;  // packed B/C, see pack_bc_kernel
     void* y;
     float* ckpt;
     float* hlast;
@@ -39,173 +44,282 @@ struct FwdParams {
     int64_t u_sb, u_sl, u_sd;
     int64_t d_sb, d_sl, d_sd;
     int64_t y_sb, y_sl, y_sd;
-    int64_t bc_sb, bc_sl;
 };
 
-constexpr int kPitch = kWave + 1;  // LDS row pitch (floats): conflict-free for both maps
+// ---------------------------------------------------------------------------------------------
+// B/C pre-pass.  Output layout, float32:
+//     [batch][tile][wave][sub-tile][B | C][kSS steps][NS states]
+// i.e. the values one scan wave needs for one sub-tile of kSS steps are contiguous (the scan
+// waves fetch them one sub-tile ahead of use).  Steps beyond the sequence end and states
+// beyond d_state are written as zeros.
+// ---------------------------------------------------------------------------------------------
+template <typename IO>
+__global__ void __launch_bounds__(256) pack_bc_kernel(const void* Bm, const void* C, float* out,
+                                                      int L, int N, int NS, int NW, int kSS,
+                                                      int nchunks, int64_t bc_sb, int64_t bc_sl) {
+    const int NP = NS * NW;
+    const int64_t per_b = (int64_t)nchunks * 2 * kTile * NP;
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= per_b) return;
+    const int b = blockIdx.y;
+    // decompose the OUTPUT index
+    int r = (int)(i % (2 * kTile * NP));
+    const int c = (int)(i / (2 * kTile * NP));
+    const int w = r / (2 * kTile * NS);
+    r %= 2 * kTile * NS;
+    const int sub = r / (2 * kSS * NS);
+    r %= 2 * kSS * NS;
+    const int which = r / (kSS * NS);
+    r %= kSS * NS;
+    const int tt = sub * kSS + r / NS, s = r % NS;
+    const int t = c * kTile + tt, n = w * NS + s;
+    float v = 0.0f;
+    if (t < L && n < N)
+        v = load_as_float<IO>(which ? C : Bm, b * bc_sb + (int64_t)t * bc_sl + n);
+    out[b * per_b + i] = v;
+}
+
+constexpr int kCP = kTile + 4;  // pitch (floats) of a [channel][step] LDS tile: rows stay
+                                // 16-byte aligned and 16-byte accesses of 16 lanes hit 64
+                                // distinct banks
+constexpr int kService = 4;     // service waves per workgroup (256 items of 4 steps per tile)
+
+template <int NS, int NW>
+struct FwdLds {
+    // delta, u double-buffered (written two tiles ahead of use, read one tile ahead); D*x and
+    // the gate in four buffers (written two tiles ahead, read one tile behind); readout
+    // partials double-buffered per scan wave
+    static constexpr size_t floats = (size_t)(2 * 2 + 2 * 4 + 2 * NW) * kWave * kCP;
+};
+
+typedef float f16v __attribute__((ext_vector_type(16)));
+
+// B/C reach the scan waves in sub-tiles of kSS steps; two sub-tiles (the one in use and the
+// one in flight) must fit the scalar register file, so a sub-tile holds 32 floats (64 at 32
+// states per lane).
+template <int NS>
+struct BcPack {
+    static constexpr int kSS = NS >= 16 ? 1 : 16 / NS;
+};
+
+// COUNT consecutive floats through the scalar cache into SGPRs (the address is wave-uniform)
+template <int COUNT>
+__device__ __forceinline__ void scalar_load(const float* src, float (&dst)[COUNT]) {
+    static_assert(COUNT % 16 == 0, "scalar_load moves multiples of 16 floats");
+    const uintptr_t a = reinterpret_cast<uintptr_t>(src);
+#pragma unroll
+    for (int j = 0; j < COUNT / 16; ++j) {
+        const f16v v = *reinterpret_cast<const __attribute__((address_space(4))) f16v*>(a + 64 * j);
+#pragma unroll
+        for (int k = 0; k < 16; ++k) dst[16 * j + k] = v[k];
+    }
+}
 
 template <typename IO, int NS, int NW>
-__global__ void __launch_bounds__(NW* kWave) sscan_fwd_kernel(const FwdParams p) {
-    constexpr int NT = NW * kWave;
-    constexpr int NP = NS * NW;                    // padded state count
-    constexpr int EPT = (kTile * kWave + NT - 1) / NT;  // (step, channel) elements per thread
-    constexpr int BPT = (kTile * NP + NT - 1) / NT;     // B/C elements per thread
+__global__ void __launch_bounds__((NW + kService) * kWave) sscan_fwd_kernel(const FwdParams p) {
+    constexpr int NQ = kTile / 4;  // step groups (of 4) per tile
+    static_assert(kService * kWave == kWave * NQ, "one service thread per (channel, step group)");
 
-    extern __shared__ float smem[];
-    typedef float Tile[kTile][kPitch];
-    typedef float TileN[kTile][NP];
-    Tile* sDelta = reinterpret_cast<Tile*>(smem);                 // [2]
-    Tile* sU = sDelta + 2;                                        // [2]
-    Tile* sX = sU + 2;                                            // [2]
-    Tile* sY = sX + 2;                                            // [NW]
-    TileN* sB = reinterpret_cast<TileN*>(sY + NW);                // [2]
-    TileN* sC = sB + 2;                                           // [2]
+    extern __shared__ float4 smem4[];
+    typedef float CTile[kWave][kCP];  // [channel][step]
+    CTile* sDl = reinterpret_cast<CTile*>(smem4);  // [2]
+    CTile* sU = sDl + 2;                           // [2]
+    CTile* sDx = sU + 2;                           // [4] D*x
+    CTile* sG = sDx + 4;                           // [4] gate silu(z) (only with z)
+    CTile* sY = sG + 4;                            // [2][NW]
 
-    const int tid = threadIdx.x;
-    const int lane = tid & (kWave - 1);
+    const int lane = threadIdx.x & (kWave - 1);
     const int w = wave_id();
     const int b = blockIdx.y;
     const int d0 = blockIdx.x * kWave;
+    const int ntiles = p.nchunks;
+    const bool has_z = p.z != nullptr;
+
+    if (w >= NW) {
+        // =============================== service waves ===============================
+        const int item = (w - NW) * kWave + lane;  // 0 .. 255
+        const int cmax = min(kWave, p.ED - d0) - 1;
+        // input side: which (channel, step group) this thread loads and stages
+        const int ci = p.in_tmajor ? item / NQ : item % kWave;
+        const int qi = p.in_tmajor ? item % NQ : item / kWave;
+        // output side: which (channel, step group) this thread reduces and stores
+        const int co = p.out_tmajor ? item / NQ : item % kWave;
+        const int qo = p.out_tmajor ? item % NQ : item / kWave;
+        const bool ci_ok = ci <= cmax, co_ok = co <= cmax;
+        const int cic = min(ci, cmax);
+        const IO* const xg = static_cast<const IO*>(p.x) + (b * p.u_sb + (int64_t)(d0 + cic) * p.u_sd);
+        const IO* const dg = static_cast<const IO*>(p.delta) + (b * p.d_sb + (int64_t)(d0 + cic) * p.d_sd);
+        const IO* const zg = static_cast<const IO*>(p.z) + (b * p.u_sb + (int64_t)(d0 + cic) * p.u_sd);
+        IO* const yg = static_cast<IO*>(p.y) + (b * p.y_sb + (int64_t)(d0 + min(co, cmax)) * p.y_sd);
+        const float Dv = p.D[d0 + cic];
+        const float bias = p.dbias ? p.dbias[d0 + cic] : 0.0f;
+
+        IO rx[4], rd[4], rz[4];
+        auto load_tile = [&](int k) {
+            const int t0 = k * kTile + 4 * qi;
+            const int tlast = p.L - 1;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int64_t t = min(t0 + j, tlast);  // clamped: stays in bounds, no branch
+                rx[j] = xg[t * p.u_sl];
+                rd[j] = dg[t * p.d_sl];
+                if (has_z) rz[j] = zg[t * p.u_sl];
+            }
+        };
+        auto stage_tile = [&](int k) {
+            const int t0 = k * kTile + 4 * qi;
+            float dl[4], uu[4], dx[4], gg[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const bool ok = ci_ok && t0 + j < p.L;
+                const float xv = ok ? to_float(rx[j]) : 0.0f;
+                float dv = to_float(rd[j]);
+                if (p.softplus) dv = softplus_f(dv + bias);
+                dv = ok ? dv : 0.0f;  // padding: delta = 0, u = 0 leaves the state unchanged
+                dl[j] = dv;
+                uu[j] = dv * xv;
+                dx[j] = Dv * xv;
+                gg[j] = 0.0f;
+                if (has_z) {
+                    const float zv = to_float(rz[j]);
+                    gg[j] = zv * sigmoid_f(zv);
+                }
+            }
+            *reinterpret_cast<float4*>(&sDl[k & 1][ci][4 * qi]) = make_float4(dl[0], dl[1], dl[2], dl[3]);
+            *reinterpret_cast<float4*>(&sU[k & 1][ci][4 * qi]) = make_float4(uu[0], uu[1], uu[2], uu[3]);
+            *reinterpret_cast<float4*>(&sDx[k & 3][ci][4 * qi]) = make_float4(dx[0], dx[1], dx[2], dx[3]);
+            if (has_z)
+                *reinterpret_cast<float4*>(&sG[k & 3][ci][4 * qi]) = make_float4(gg[0], gg[1], gg[2], gg[3]);
+        };
+        auto reduce_store = [&](int k) {
+            float4 s = *reinterpret_cast<const float4*>(&sDx[k & 3][co][4 * qo]);
+#pragma unroll
+            for (int ww = 0; ww < NW; ++ww) {
+                const float4 v = *reinterpret_cast<const float4*>(&sY[(k & 1) * NW + ww][co][4 * qo]);
+                s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
+            }
+            if (has_z) {
+                const float4 g = *reinterpret_cast<const float4*>(&sG[k & 3][co][4 * qo]);
+                s.x *= g.x; s.y *= g.y; s.z *= g.z; s.w *= g.w;
+            }
+            const float sv[4] = {s.x, s.y, s.z, s.w};
+            const int t0 = k * kTile + 4 * qo;
+            if (co_ok) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    if (t0 + j < p.L) yg[(int64_t)(t0 + j) * p.y_sl] = from_float<IO>(sv[j]);
+            }
+        };
+
+        // the service waves run two tiles ahead of the scan waves on the input side and one
+        // tile behind on the output side
+        load_tile(0);
+        stage_tile(0);
+        if (ntiles > 1) {
+            load_tile(1);
+            stage_tile(1);
+        }
+        if (ntiles > 2) load_tile(2);
+        __syncthreads();  // tiles 0 and 1 are published
+        __syncthreads();  // the scan waves hold tile 0 in registers: its buffer may be reused
+        for (int k = 0; k < ntiles; ++k) {
+            if (k >= 1) reduce_store(k - 1);
+            if (k + 2 < ntiles) {
+                stage_tile(k + 2);
+                if (k + 3 < ntiles) load_tile(k + 3);
+            }
+            __syncthreads();
+        }
+        reduce_store(ntiles - 1);
+        return;
+    }
+
+    // ================================= scan waves =================================
     const int d = d0 + lane;
     const bool dvalid = d < p.ED;
-
     float A2[NS], h[NS];
 #pragma unroll
     for (int i = 0; i < NS; ++i) {
         const int n = w * NS + i;
         const bool ok = dvalid && n < p.N;
-        A2[i] = ok ? p.A[(int64_t)d * p.N + n] * kLog2e : 0.0f;
-        h[i] = (ok && p.h0) ? p.h0[((int64_t)b * p.ED + d) * p.N + n] : 0.0f;
+        const int64_t dn = (int64_t)min(d, p.ED - 1) * p.N + min(n, p.N - 1);
+        const float av = p.A[dn];
+        const float hv = p.h0 ? p.h0[(int64_t)b * p.ED * p.N + dn] : 0.0f;
+        A2[i] = ok ? av * kLog2e : 0.0f;
+        h[i] = ok ? hv : 0.0f;
     }
+    // packed B/C of this (batch, wave): sub-tile j of tile k at + (k*NW*NSUB + j) * kSub
+    constexpr int kSS = BcPack<NS>::kSS;        // steps per sub-tile
+    constexpr int NSUB = kTile / kSS;           // sub-tiles per tile
+    constexpr int kSub = 2 * kSS * NS;          // floats per sub-tile: B then C
+    const float* bc = p.bcpack + ((int64_t)b * ntiles * NW + w) * (NSUB * kSub);
+    const int64_t bc_tile = (int64_t)NW * NSUB * kSub;
 
-    // register staging of the next tile
-    float rX[EPT], rDl[EPT], rB[BPT], rC[BPT];
-
-    auto elem_map = [&](int idx, bool tmajor, int& tt, int& cc) {
-        if (tmajor) {
-            tt = idx % kTile;
-            cc = idx / kTile;
-        } else {
-            tt = idx / kWave;
-            cc = idx % kWave;
+    auto read_tile = [&](int k, float (&dl)[kTile], float (&uu)[kTile]) {
+#pragma unroll
+        for (int q = 0; q < NQ; ++q) {
+            const float4 v = *reinterpret_cast<const float4*>(&sDl[k & 1][lane][4 * q]);
+            const float4 u4 = *reinterpret_cast<const float4*>(&sU[k & 1][lane][4 * q]);
+            dl[4 * q] = v.x; dl[4 * q + 1] = v.y; dl[4 * q + 2] = v.z; dl[4 * q + 3] = v.w;
+            uu[4 * q] = u4.x; uu[4 * q + 1] = u4.y; uu[4 * q + 2] = u4.z; uu[4 * q + 3] = u4.w;
         }
     };
 
-    auto prefetch = [&](int t0) {
-        const int tl = min(kTile, p.L - t0);
-#pragma unroll
-        for (int k = 0; k < EPT; ++k) {
-            const int idx = tid + k * NT;
-            int tt, cc;
-            elem_map(idx, p.in_tmajor, tt, cc);
-            float xv = 0.0f, dv = 0.0f;
-            if (idx < kTile * kWave && tt < tl && d0 + cc < p.ED) {
-                const int64_t t = t0 + tt;
-                xv = load_as_float<IO>(p.x, b * p.u_sb + t * p.u_sl + (int64_t)(d0 + cc) * p.u_sd);
-                dv = load_as_float<IO>(p.delta, b * p.d_sb + t * p.d_sl + (int64_t)(d0 + cc) * p.d_sd);
-            }
-            rX[k] = xv;
-            rDl[k] = dv;
-        }
-#pragma unroll
-        for (int k = 0; k < BPT; ++k) {
-            const int idx = tid + k * NT;
-            const int tt = idx / NP, n = idx % NP;
-            float bv = 0.0f, cv = 0.0f;
-            if (idx < kTile * NP && tt < tl && n < p.N) {
-                const int64_t off = b * p.bc_sb + (int64_t)(t0 + tt) * p.bc_sl + n;
-                bv = load_as_float<IO>(p.Bm, off);
-                cv = load_as_float<IO>(p.C, off);
-            }
-            rB[k] = bv;
-            rC[k] = cv;
-        }
-    };
-
-    // the softplus is applied here, not in prefetch(), so that the loads stay in flight
-    // during the arithmetic of the previous tile; padded elements keep delta = 0
-    auto stage = [&](int buf, int t0) {
-        const int tl = min(kTile, p.L - t0);
-#pragma unroll
-        for (int k = 0; k < EPT; ++k) {
-            const int idx = tid + k * NT;
-            int tt, cc;
-            elem_map(idx, p.in_tmajor, tt, cc);
-            if (idx < kTile * kWave) {
-                if (p.softplus && tt < tl && d0 + cc < p.ED)
-                    rDl[k] = softplus_f(rDl[k] + (p.dbias ? p.dbias[d0 + cc] : 0.0f));
-                sDelta[buf][tt][cc] = rDl[k];
-                sU[buf][tt][cc] = rDl[k] * rX[k];
-                sX[buf][tt][cc] = rX[k];
-            }
-        }
-#pragma unroll
-        for (int k = 0; k < BPT; ++k) {
-            const int idx = tid + k * NT;
-            if (idx < kTile * NP) {
-                sB[buf][idx / NP][idx % NP] = rB[k];
-                sC[buf][idx / NP][idx % NP] = rC[k];
-            }
-        }
-    };
-
-    prefetch(0);
-    int buf = 0;
-    for (int t0 = 0, c = 0; t0 < p.L; t0 += kTile, ++c, buf ^= 1) {
-        const int tl = min(kTile, p.L - t0);
-        stage(buf, t0);
-        __syncthreads();
-        if (t0 + kTile < p.L) prefetch(t0 + kTile);
-
-        // phase B: steps beyond the sequence end were staged as delta = 0, u = 0, which
-        // leaves h unchanged (a = 2^0 = 1), so the loop needs no tail handling
+    // Software pipeline of one scan wave.  In interval k (between two barriers) it computes
+    // tile k from registers that were filled during interval k-1, fetches delta/u of tile
+    // k+1 from LDS (published by the service waves two intervals ahead) and B/C one sub-tile
+    // ahead through the scalar cache, so no load latency sits between two dependent steps.
+    // Padded steps were staged as delta = 0, u = 0 (a = 2^0 = 1: h unchanged) and padded
+    // states have A2 = 0, B = C = 0, so there is no tail handling.
+    float bcb[2][kSub];  // wave-uniform: live in SGPRs; sub-tile j of a tile uses bcb[j & 1]
+    auto tile_compute = [&](int k, const float (&dl)[kTile], const float (&uu)[kTile]) {
+        const float* bck = bc + (int64_t)k * bc_tile;
+        float acc[4];
 #pragma unroll
         for (int tt = 0; tt < kTile; ++tt) {
-            const float dv = sDelta[buf][tt][lane];
-            const float uv = sU[buf][tt][lane];
-            float acc = 0.0f;
+            const int sub = tt / kSS, ts = tt % kSS;
+            if (ts == 0) {
+                // fetch the next sub-tile (the first one of the next tile after the last)
+                if (sub + 1 < NSUB)
+                    scalar_load<kSub>(bck + (sub + 1) * kSub, bcb[(sub + 1) & 1]);
+                else if (k + 1 < ntiles)
+                    scalar_load<kSub>(bck + bc_tile, bcb[0]);
+            }
+            const float(&cur)[kSub] = bcb[sub & 1];
+            float sum = 0.0f;
 #pragma unroll
             for (int i = 0; i < NS; ++i) {
-                const float a = fast_exp2(dv * A2[i]);
-                const float bv = sB[buf][tt][w * NS + i];
-                const float cv = sC[buf][tt][w * NS + i];
-                h[i] = __builtin_fmaf(uv, bv, a * h[i]);
-                acc = __builtin_fmaf(cv, h[i], acc);
+                const float a = fast_exp2(dl[tt] * A2[i]);
+                h[i] = __builtin_fmaf(uu[tt], cur[ts * NS + i], a * h[i]);
+                sum = __builtin_fmaf(cur[kSS * NS + ts * NS + i], h[i], sum);
             }
-            sY[w][tt][lane] = acc;
+            acc[tt & 3] = sum;
+            if ((tt & 3) == 3)
+                *reinterpret_cast<float4*>(&sY[(k & 1) * NW + w][lane][tt - 3]) =
+                    make_float4(acc[0], acc[1], acc[2], acc[3]);
         }
-        if (p.ckpt && dvalid) {
+        if (p.ckpt && dvalid && k + 1 < ntiles) {
 #pragma unroll
             for (int i = 0; i < NS; ++i) {
                 const int n = w * NS + i;
-                if (n < p.N)
-                    p.ckpt[(((int64_t)b * p.nchunks + c) * p.N + n) * p.ED + d] = h[i];
+                if (n < p.N) p.ckpt[(((int64_t)b * ntiles + k) * p.N + n) * p.ED + d] = h[i];
             }
         }
-        __syncthreads();
+    };
 
-        // phase C
-#pragma unroll
-        for (int k = 0; k < EPT; ++k) {
-            const int idx = tid + k * NT;
-            int tt, cc;
-            elem_map(idx, p.out_tmajor, tt, cc);
-            if (idx < kTile * kWave && tt < tl && d0 + cc < p.ED) {
-                float s = 0.0f;
-#pragma unroll
-                for (int ww = 0; ww < NW; ++ww) s += sY[ww][tt][cc];
-                s = __builtin_fmaf(p.D[d0 + cc], sX[buf][tt][cc], s);
-                const int64_t t = t0 + tt;
-                if (p.z) {
-                    const float zv =
-                        load_as_float<IO>(p.z, b * p.u_sb + t * p.u_sl + (int64_t)(d0 + cc) * p.u_sd);
-                    s *= zv * sigmoid_f(zv);
-                }
-                store_from_float<IO>(p.y, b * p.y_sb + t * p.y_sl + (int64_t)(d0 + cc) * p.y_sd, s);
-            }
-        }
-        // the next stage() writes the other input buffer; sY is rewritten only after the
-        // barrier that follows it, so no third barrier is needed here
+    float dlA[kTile], uuA[kTile], dlB[kTile], uuB[kTile];
+    scalar_load<kSub>(bc, bcb[0]);
+    __syncthreads();
+    read_tile(0, dlA, uuA);
+    __syncthreads();
+    for (int k = 0; k < ntiles; k += 2) {
+        if (k + 1 < ntiles) read_tile(k + 1, dlB, uuB);
+        tile_compute(k, dlA, uuA);
+        __syncthreads();
+        if (k + 1 >= ntiles) break;
+        if (k + 2 < ntiles) read_tile(k + 2, dlA, uuA);
+        tile_compute(k + 1, dlB, uuB);
+        __syncthreads();
     }
 
     if (p.hlast && dvalid) {
@@ -220,8 +334,8 @@ __global__ void __launch_bounds__(NW* kWave) sscan_fwd_kernel(const FwdParams p)
 template <typename IO, int NS, int NW>
 static int launch_fwd(const FwdParams& p, hipStream_t stream) {
     dim3 grid((p.ED + kWave - 1) / kWave, p.batch);
-    dim3 block(NW * kWave);
-    constexpr size_t lds = sizeof(float) * ((6 + NW) * kTile * kPitch + 4 * kTile * NS * NW);
+    dim3 block((NW + kService) * kWave);
+    constexpr size_t lds = sizeof(float) * FwdLds<NS, NW>::floats;
     static const int attr_rc = allow_dynamic_lds(sscan_fwd_kernel<IO, NS, NW>, lds);
     if (attr_rc != MPA_OK) return attr_rc;
     hipLaunchKernelGGL((sscan_fwd_kernel<IO, NS, NW>), grid, block, lds, stream, p);
@@ -232,13 +346,75 @@ template <typename IO>
 static int dispatch_fwd(const FwdParams& p, int ns, int nw, hipStream_t stream) {
 #define MPA_CASE(NS_, NW_) \
     if (ns == NS_ && nw == NW_) return launch_fwd<IO, NS_, NW_>(p, stream);
-    MPA_CASE(1, 16) MPA_CASE(2, 8) MPA_CASE(4, 4) MPA_CASE(8, 2) MPA_CASE(16, 1)
-    MPA_CASE(2, 16) MPA_CASE(4, 8) MPA_CASE(8, 4) MPA_CASE(16, 2)
-    MPA_CASE(4, 16) MPA_CASE(8, 8) MPA_CASE(16, 4)
-    MPA_CASE(8, 16) MPA_CASE(16, 8)
-    MPA_CASE(16, 16)
+    MPA_CASE(2, 8) MPA_CASE(4, 4) MPA_CASE(8, 2) MPA_CASE(16, 1)
+    MPA_CASE(4, 8) MPA_CASE(8, 4) MPA_CASE(16, 2) MPA_CASE(32, 1)
+    MPA_CASE(8, 8) MPA_CASE(16, 4) MPA_CASE(32, 2)
+    MPA_CASE(16, 8) MPA_CASE(32, 4)
+    MPA_CASE(32, 8)
 #undef MPA_CASE
     return MPA_ERR_BAD_SHAPE;
+}
+
+int validate_shape(const mpa_sscan_shape* s) {
+    if (!s) return MPA_ERR_NULL_POINTER;
+    if (s->batch <= 0 || s->seqlen <= 0 || s->dim <= 0 || s->dstate <= 0) return MPA_ERR_BAD_SHAPE;
+    if (s->dstate > MPA_MAX_DSTATE || s->batch > 65535) return MPA_ERR_BAD_SHAPE;
+    if (s->seqlen > (int64_t)1 << 30 || s->dim > (int64_t)1 << 30) return MPA_ERR_BAD_SHAPE;
+    if (s->io_dtype != MPA_F32 && s->io_dtype != MPA_BF16) return MPA_ERR_BAD_DTYPE;
+    const int64_t st[] = {s->u_sb, s->u_sl, s->u_sd, s->d_sb, s->d_sl, s->d_sd, s->y_sb, s->y_sl,
+                          s->y_sd, s->g_sb, s->g_sl, s->g_sd, s->bc_sb, s->bc_sl, s->dbc_sb, s->dbc_sl};
+    for (int64_t v : st)
+        if (v < 0) return MPA_ERR_BAD_STRIDE;
+    return MPA_OK;
+}
+
+int padded_states(int64_t n) {
+    int np = 16;
+    while (np < n) np *= 2;
+    return np;
+}
+
+// States per lane (NS) for a launch.  The only parallel axes are batch*dim/64 workgroups and
+// d_state/NS scan waves inside each; a workgroup holds at most 8 scan waves.  Fewer states per
+// lane mean more waves (better latency hiding) but more LDS traffic per state; ask for about
+// two scan waves per SIMD over the chip's 1024 SIMDs when the problem offers them.
+int pick_states_per_lane(int64_t batch, int64_t dim, int64_t dstate, int ns_cap, const char* env) {
+    const int np = padded_states(dstate);
+    const int ns_min = np / 8 > 2 ? np / 8 : 2;
+    const int ns_max = ns_cap < np ? ns_cap : np;
+    if (ns_max < ns_min) return -1;
+    if (env) {
+        const char* v = getenv(env);
+        if (v) {
+            const int ns = atoi(v);
+            if (ns >= ns_min && ns <= ns_max && (ns & (ns - 1)) == 0) return ns;
+        }
+    }
+    const int64_t groups = batch * ((dim + kWave - 1) / kWave);
+    int ns = ns_max;
+    while (ns > ns_min && groups * (np / ns) < 2048) ns /= 2;
+    return ns;
+}
+
+size_t bcpack_floats(const mpa_sscan_shape* s) {
+    const size_t nchunks = (size_t)(s->seqlen + kTile - 1) / kTile;
+    return (size_t)s->batch * nchunks * 2 * kTile * padded_states(s->dstate);
+}
+
+int launch_pack_bc(const mpa_sscan_shape* s, const void* B, const void* C, float* out, int ns,
+                   hipStream_t st) {
+    const int np = padded_states(s->dstate);
+    const int nchunks = (int)((s->seqlen + kTile - 1) / kTile);
+    const int64_t per_b = (int64_t)nchunks * 2 * kTile * np;
+    const int kss = ns >= 16 ? 1 : 16 / ns;  // BcPack<NS>::kSS
+    dim3 grid((unsigned)((per_b + 255) / 256), (unsigned)s->batch);
+    if (s->io_dtype == MPA_F32)
+        hipLaunchKernelGGL(pack_bc_kernel<float>, grid, dim3(256), 0, st, B, C, out, (int)s->seqlen,
+                           (int)s->dstate, ns, np / ns, kss, nchunks, s->bc_sb, s->bc_sl);
+    else
+        hipLaunchKernelGGL(pack_bc_kernel<bf16_t>, grid, dim3(256), 0, st, B, C, out, (int)s->seqlen,
+                           (int)s->dstate, ns, np / ns, kss, nchunks, s->bc_sb, s->bc_sl);
+    return check_launch();
 }
 
 }  // namespace mpa
@@ -251,72 +427,48 @@ extern "C" int64_t mpa_sscan_ckpt_elems(const mpa_sscan_shape* s) {
     return s->batch * nchunks * s->dstate * s->dim;
 }
 
-namespace mpa {
-int validate_shape(const mpa_sscan_shape* s) {
-    if (!s) return MPA_ERR_NULL_POINTER;
-    if (s->batch <= 0 || s->seqlen <= 0 || s->dim <= 0 || s->dstate <= 0) return MPA_ERR_BAD_SHAPE;
-    if (s->dstate > MPA_MAX_DSTATE || s->batch > 65535) return MPA_ERR_BAD_SHAPE;
-    if (s->seqlen > (int64_t)1 << 30 || s->dim > (int64_t)1 << 30) return MPA_ERR_BAD_SHAPE;
-    if (s->io_dtype != MPA_F32 && s->io_dtype != MPA_BF16) return MPA_ERR_BAD_DTYPE;
-    return MPA_OK;
+extern "C" size_t mpa_sscan_fwd_workspace_bytes(const mpa_sscan_shape* s) {
+    if (validate_shape(s) != MPA_OK) return 0;
+    return (bcpack_floats(s) * sizeof(float) + 255) / 256 * 256;
 }
-
-int padded_states(int64_t n) {
-    int np = 16;
-    while (np < n) np *= 2;
-    return np;
-}
-
-int pick_states_per_lane(int64_t batch, int64_t dim, int64_t dstate, int ns_max, const char* env) {
-    const int np = padded_states(dstate);
-    const int ns_min = np / 16;  // at most 16 waves per workgroup
-    if (env) {
-        const char* v = getenv(env);
-        if (v) {
-            const int ns = atoi(v);
-            if (ns >= ns_min && ns <= ns_max && ns <= np && (ns & (ns - 1)) == 0) return ns;
-        }
-    }
-    // waves in flight = batch * ceil(dim/64) * np/ns; ask for two per SIMD (2048) if the
-    // problem has them, otherwise expose all the parallelism there is
-    const int64_t groups = batch * ((dim + kWave - 1) / kWave);
-    int ns = ns_max < np ? ns_max : np;
-    while (ns > ns_min && groups * (np / ns) < 2048) ns /= 2;
-    return ns < ns_min ? ns_min : ns;
-}
-}  // namespace mpa
 
 extern "C" int mpa_sscan_fwd(const mpa_sscan_shape* s, const void* x, const void* delta,
                              const float* A, const void* B, const void* C, const float* D,
                              const void* z, const float* delta_bias, const float* h0, void* y,
-                             float* h_ckpt, float* h_last, void* stream) {
+                             float* h_ckpt, float* h_last, void* workspace,
+                             size_t workspace_bytes, void* stream) {
     int rc = validate_shape(s);
     if (rc != MPA_OK) return rc;
-    if (!x || !delta || !A || !B || !C || !D || !y) return MPA_ERR_NULL_POINTER;
+    if (!x || !delta || !A || !B || !C || !D || !y || !workspace) return MPA_ERR_NULL_POINTER;
     const bool softplus = (s->flags & MPA_SSCAN_DELTA_SOFTPLUS) != 0;
     if (!softplus && delta_bias) return MPA_ERR_BAD_SHAPE;
     const size_t es = dtype_size(s->io_dtype);
     if (!aligned_to(x, es) || !aligned_to(delta, es) || !aligned_to(B, es) || !aligned_to(C, es) ||
-        !aligned_to(y, es) || (z && !aligned_to(z, es)) || !aligned_to(A, 4) || !aligned_to(D, 4))
+        !aligned_to(y, es) || (z && !aligned_to(z, es)) || !aligned_to(A, 4) || !aligned_to(D, 4) ||
+        !aligned_to(workspace, 256))
         return MPA_ERR_MISALIGNED;
+    if (workspace_bytes < mpa_sscan_fwd_workspace_bytes(s)) return MPA_ERR_WORKSPACE;
+
+    const int np = padded_states(s->dstate);
+    const int ns = pick_states_per_lane(s->batch, s->dim, s->dstate, 32, "MPA_FWD_NS");
+    if (ns < 0) return MPA_ERR_BAD_SHAPE;
+    const int nw = np / ns;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    rc = launch_pack_bc(s, B, C, static_cast<float*>(workspace), ns, st);
+    if (rc != MPA_OK) return rc;
 
     FwdParams p{};
-    p.x = x; p.delta = delta; p.Bm = B; p.C = C; p.z = z; p.A = A; p.D = D;
-    p.dbias = delta_bias; p.h0 = h0; p.y = y; p.ckpt = h_ckpt; p.hlast = h_last;
+    p.x = x; p.delta = delta; p.z = z; p.A = A; p.D = D;
+    p.dbias = delta_bias; p.h0 = h0; p.bcpack = static_cast<const float*>(workspace);
+    p.y = y; p.ckpt = h_ckpt; p.hlast = h_last;
     p.batch = (int)s->batch; p.L = (int)s->seqlen; p.ED = (int)s->dim; p.N = (int)s->dstate;
     p.nchunks = (p.L + kTile - 1) / kTile;
     p.softplus = softplus ? 1 : 0;
     p.u_sb = s->u_sb; p.u_sl = s->u_sl; p.u_sd = s->u_sd;
     p.d_sb = s->d_sb; p.d_sl = s->d_sl; p.d_sd = s->d_sd;
     p.y_sb = s->y_sb; p.y_sl = s->y_sl; p.y_sd = s->y_sd;
-    p.bc_sb = s->bc_sb; p.bc_sl = s->bc_sl;
     p.in_tmajor = (s->u_sd != 1 && s->u_sl == 1) ? 1 : 0;
     p.out_tmajor = (s->y_sd != 1 && s->y_sl == 1) ? 1 : 0;
-
-    const int np = padded_states(s->dstate);
-    const int ns = pick_states_per_lane(s->batch, s->dim, s->dstate, 16, "MPA_FWD_NS");
-    const int nw = np / ns;
-    hipStream_t st = static_cast<hipStream_t>(stream);
     if (s->io_dtype == MPA_F32) return dispatch_fwd<float>(p, ns, nw, st);
     return dispatch_fwd<bf16_t>(p, ns, nw, st);
 }

@@ -109,10 +109,12 @@ class SelectiveScanFn(torch.autograd.Function):
                                device=x.device)
         h_last = torch.empty((Bsz, ED, N), dtype=torch.float32, device=x.device) \
             if return_last_state else None
+        nbytes = lib.mpa_sscan_fwd_workspace_bytes(ctypes.byref(shape))
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=x.device)
         with torch.cuda.device(x.device):
             rc = lib.mpa_sscan_fwd(ctypes.byref(shape), _ptr(x_), _ptr(delta_), _ptr(A_), _ptr(B_),
                                    _ptr(C_), _ptr(D_), _ptr(z_), _ptr(bias_), _ptr(h0_), _ptr(y),
-                                   _ptr(ckpt), _ptr(h_last), _stream(x.device))
+                                   _ptr(ckpt), _ptr(h_last), _ptr(ws), nbytes, _stream(x.device))
         _lib.check(rc, "mpa_sscan_fwd")
         ctx.save_for_backward(x_, delta_, A_, B_, C_, D_, z_, bias_, h0_, ckpt)
         ctx.flags = flags
