@@ -29,17 +29,11 @@ template <>
 __device__ __forceinline__ float from_float<float>(float v) {
     return v;
 }
-// round-to-nearest-even; NaN stays NaN (quiet bit forced)
+// round-to-nearest-even on the hardware converter (v_cvt_pk_bf16_f32)
 template <>
 __device__ __forceinline__ bf16_t from_float<bf16_t>(float v) {
-    uint32_t u = __float_as_uint(v);
-    uint32_t r;
-    if ((u & 0x7fffffffu) > 0x7f800000u) {
-        r = (u >> 16) | 0x40u;
-    } else {
-        r = (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
-    }
-    return bf16_t{static_cast<uint16_t>(r)};
+    const __bf16 r = static_cast<__bf16>(v);
+    return bf16_t{__builtin_bit_cast(uint16_t, r)};
 }
 
 template <typename T>

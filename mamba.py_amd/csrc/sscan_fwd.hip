@@ -115,7 +115,7 @@ __device__ __forceinline__ void scalar_load(const float* src, float (&dst)[COUNT
     }
 }
 
-template <typename IO, int NS, int NW>
+template <typename IO, int NS, int NW, bool HAS_Z>
 __global__ void __launch_bounds__((NW + kService) * kWave) sscan_fwd_kernel(const FwdParams p) {
     constexpr int NQ = kTile / 4;  // step groups (of 4) per tile
     static_assert(kService * kWave == kWave * NQ, "one service thread per (channel, step group)");
@@ -133,104 +133,153 @@ __global__ void __launch_bounds__((NW + kService) * kWave) sscan_fwd_kernel(cons
     const int b = blockIdx.y;
     const int d0 = blockIdx.x * kWave;
     const int ntiles = p.nchunks;
-    const bool has_z = p.z != nullptr;
+    constexpr bool has_z = HAS_Z;
 
     if (w >= NW) {
         // =============================== service waves ===============================
-        const int item = (w - NW) * kWave + lane;  // 0 .. 255
-        const int cmax = min(kWave, p.ED - d0) - 1;
-        // input side: which (channel, step group) this thread loads and stages
-        const int ci = p.in_tmajor ? item / NQ : item % kWave;
-        const int qi = p.in_tmajor ? item % NQ : item / kWave;
-        // output side: which (channel, step group) this thread reduces and stores
-        const int co = p.out_tmajor ? item / NQ : item % kWave;
-        const int qo = p.out_tmajor ? item % NQ : item / kWave;
-        const bool ci_ok = ci <= cmax, co_ok = co <= cmax;
-        const int cic = min(ci, cmax);
-        const IO* const xg = static_cast<const IO*>(p.x) + (b * p.u_sb + (int64_t)(d0 + cic) * p.u_sd);
-        const IO* const dg = static_cast<const IO*>(p.delta) + (b * p.d_sb + (int64_t)(d0 + cic) * p.d_sd);
-        const IO* const zg = static_cast<const IO*>(p.z) + (b * p.u_sb + (int64_t)(d0 + cic) * p.u_sd);
-        IO* const yg = static_cast<IO*>(p.y) + (b * p.y_sb + (int64_t)(d0 + min(co, cmax)) * p.y_sd);
-        const float Dv = p.D[d0 + cic];
-        const float bias = p.dbias ? p.dbias[d0 + cic] : 0.0f;
-
-        IO rx[4], rd[4], rz[4];
-        auto load_tile = [&](int k) {
-            const int t0 = k * kTile + 4 * qi;
-            const int tlast = p.L - 1;
+        // Two loader waves and two reducer waves, two items of (channel, 4 steps) per thread.
+        // The roles are split across waves because loads and stores share one in-order
+        // counter per wave: a wave that stores y would wait for those stores to drain every
+        // time it waits for its next input tile.
+        const int sw = w - NW;                       // 0,1: loaders   2,3: reducers
+        const int cmax = min(kWave, p.ED - d0) - 1;  // last valid channel of the group
+        if (sw < 2) {
+            // ------------------------------- loaders -------------------------------
+            int ci[2], qi[2];
+            bool ci_ok[2];
+            uint32_t cx[2], cd[2];
+            float Dv[2], bias[2];
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const int64_t t = min(t0 + j, tlast);  // clamped: stays in bounds, no branch
-                rx[j] = xg[t * p.u_sl];
-                rd[j] = dg[t * p.d_sl];
-                if (has_z) rz[j] = zg[t * p.u_sl];
+            for (int r = 0; r < 2; ++r) {
+                const int item = sw * kWave + lane + r * 2 * kWave;  // 0 .. 255
+                ci[r] = p.in_tmajor ? item / NQ : item % kWave;
+                qi[r] = p.in_tmajor ? item % NQ : item / kWave;
+                ci_ok[r] = ci[r] <= cmax;
+                const int cic = min(ci[r], cmax);
+                cx[r] = (uint32_t)cic * (uint32_t)p.u_sd;
+                cd[r] = (uint32_t)cic * (uint32_t)p.d_sd;
+                Dv[r] = p.D[d0 + cic];
+                bias[r] = p.dbias ? p.dbias[d0 + cic] : 0.0f;
             }
-        };
-        auto stage_tile = [&](int k) {
-            const int t0 = k * kTile + 4 * qi;
-            float dl[4], uu[4], dx[4], gg[4];
+            // wave-uniform tile origins (scalar registers) + per-thread 32-bit element
+            // offsets: one global_load per element, no 64-bit address arithmetic in the loop
+            const IO* const xg = static_cast<const IO*>(p.x) + (b * p.u_sb + (int64_t)d0 * p.u_sd);
+            const IO* const dg = static_cast<const IO*>(p.delta) + (b * p.d_sb + (int64_t)d0 * p.d_sd);
+            const IO* const zg = static_cast<const IO*>(p.z) + (b * p.u_sb + (int64_t)d0 * p.u_sd);
+
+            IO rx[2][4], rd[2][4], rz[2][4];
+            auto load_tile = [&](int k) {
+                // steps beyond the sequence end are clamped to the last one: the loads stay in
+                // bounds and free of branches (a branch here would force a wait on the data)
+                const int tmax = min(kTile, p.L - k * kTile) - 1;
+                const IO* xk = xg + (int64_t)k * kTile * p.u_sl;
+                const IO* dk = dg + (int64_t)k * kTile * p.d_sl;
+                const IO* zk = zg + (int64_t)k * kTile * p.u_sl;
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const bool ok = ci_ok && t0 + j < p.L;
-                const float xv = ok ? to_float(rx[j]) : 0.0f;
-                float dv = to_float(rd[j]);
-                if (p.softplus) dv = softplus_f(dv + bias);
-                dv = ok ? dv : 0.0f;  // padding: delta = 0, u = 0 leaves the state unchanged
-                dl[j] = dv;
-                uu[j] = dv * xv;
-                dx[j] = Dv * xv;
-                gg[j] = 0.0f;
-                if (has_z) {
-                    const float zv = to_float(rz[j]);
-                    gg[j] = zv * sigmoid_f(zv);
+                for (int r = 0; r < 2; ++r) {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        const uint32_t tc = (uint32_t)min(4 * qi[r] + j, tmax);
+                        rx[r][j] = xk[tc * (uint32_t)p.u_sl + cx[r]];
+                        rd[r][j] = dk[tc * (uint32_t)p.d_sl + cd[r]];
+                        if (has_z) rz[r][j] = zk[tc * (uint32_t)p.u_sl + cx[r]];
+                    }
                 }
-            }
-            *reinterpret_cast<float4*>(&sDl[k & 1][ci][4 * qi]) = make_float4(dl[0], dl[1], dl[2], dl[3]);
-            *reinterpret_cast<float4*>(&sU[k & 1][ci][4 * qi]) = make_float4(uu[0], uu[1], uu[2], uu[3]);
-            *reinterpret_cast<float4*>(&sDx[k & 3][ci][4 * qi]) = make_float4(dx[0], dx[1], dx[2], dx[3]);
-            if (has_z)
-                *reinterpret_cast<float4*>(&sG[k & 3][ci][4 * qi]) = make_float4(gg[0], gg[1], gg[2], gg[3]);
-        };
-        auto reduce_store = [&](int k) {
-            float4 s = *reinterpret_cast<const float4*>(&sDx[k & 3][co][4 * qo]);
+            };
+            auto stage_tile = [&](int k) {
 #pragma unroll
-            for (int ww = 0; ww < NW; ++ww) {
-                const float4 v = *reinterpret_cast<const float4*>(&sY[(k & 1) * NW + ww][co][4 * qo]);
-                s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
-            }
-            if (has_z) {
-                const float4 g = *reinterpret_cast<const float4*>(&sG[k & 3][co][4 * qo]);
-                s.x *= g.x; s.y *= g.y; s.z *= g.z; s.w *= g.w;
-            }
-            const float sv[4] = {s.x, s.y, s.z, s.w};
-            const int t0 = k * kTile + 4 * qo;
-            if (co_ok) {
+                for (int r = 0; r < 2; ++r) {
+                    const int t0 = k * kTile + 4 * qi[r];
+                    float dl[4], uu[4], dx[4], gg[4];
 #pragma unroll
-                for (int j = 0; j < 4; ++j)
-                    if (t0 + j < p.L) yg[(int64_t)(t0 + j) * p.y_sl] = from_float<IO>(sv[j]);
+                    for (int j = 0; j < 4; ++j) {
+                        const bool ok = ci_ok[r] && t0 + j < p.L;
+                        const float xv = ok ? to_float(rx[r][j]) : 0.0f;
+                        float dv = to_float(rd[r][j]);
+                        if (p.softplus) dv = softplus_f(dv + bias[r]);
+                        dv = ok ? dv : 0.0f;  // padding: delta = 0, u = 0 keeps the state
+                        dl[j] = dv;
+                        uu[j] = dv * xv;
+                        dx[j] = Dv[r] * xv;
+                        gg[j] = 0.0f;
+                        if (has_z) {
+                            const float zv = to_float(rz[r][j]);
+                            gg[j] = zv * sigmoid_f(zv);
+                        }
+                    }
+                    const int c = ci[r], q4 = 4 * qi[r];
+                    *reinterpret_cast<float4*>(&sDl[k & 1][c][q4]) = make_float4(dl[0], dl[1], dl[2], dl[3]);
+                    *reinterpret_cast<float4*>(&sU[k & 1][c][q4]) = make_float4(uu[0], uu[1], uu[2], uu[3]);
+                    *reinterpret_cast<float4*>(&sDx[k & 3][c][q4]) = make_float4(dx[0], dx[1], dx[2], dx[3]);
+                    if (has_z)
+                        *reinterpret_cast<float4*>(&sG[k & 3][c][q4]) =
+                            make_float4(gg[0], gg[1], gg[2], gg[3]);
+                }
+            };
+            // the loaders run two tiles ahead of the scan waves
+            load_tile(0);
+            stage_tile(0);
+            if (ntiles > 1) {
+                load_tile(1);
+                stage_tile(1);
             }
-        };
-
-        // the service waves run two tiles ahead of the scan waves on the input side and one
-        // tile behind on the output side
-        load_tile(0);
-        stage_tile(0);
-        if (ntiles > 1) {
-            load_tile(1);
-            stage_tile(1);
-        }
-        if (ntiles > 2) load_tile(2);
-        __syncthreads();  // tiles 0 and 1 are published
-        __syncthreads();  // the scan waves hold tile 0 in registers: its buffer may be reused
-        for (int k = 0; k < ntiles; ++k) {
-            if (k >= 1) reduce_store(k - 1);
-            if (k + 2 < ntiles) {
-                stage_tile(k + 2);
+            if (ntiles > 2) load_tile(2);
+            __syncthreads();  // tiles 0 and 1 are published
+            __syncthreads();  // the scan waves hold tile 0 in registers: its buffer is free
+            for (int k = 0; k < ntiles; ++k) {
+                if (k + 2 < ntiles) stage_tile(k + 2);
                 if (k + 3 < ntiles) load_tile(k + 3);
+                __syncthreads();
             }
+        } else {
+            // ------------------------------- reducers -------------------------------
+            int co[2], qo[2];
+            bool co_ok[2];
+            uint32_t cy[2];
+#pragma unroll
+            for (int r = 0; r < 2; ++r) {
+                const int item = (sw - 2) * kWave + lane + r * 2 * kWave;
+                co[r] = p.out_tmajor ? item / NQ : item % kWave;
+                qo[r] = p.out_tmajor ? item % NQ : item / kWave;
+                co_ok[r] = co[r] <= cmax;
+                cy[r] = (uint32_t)min(co[r], cmax) * (uint32_t)p.y_sd;
+            }
+            IO* const yg = static_cast<IO*>(p.y) + (b * p.y_sb + (int64_t)d0 * p.y_sd);
+            auto reduce_store = [&](int k) {
+                IO* yk = yg + (int64_t)k * kTile * p.y_sl;
+#pragma unroll
+                for (int r = 0; r < 2; ++r) {
+                    const int c = co[r], q4 = 4 * qo[r];
+                    float4 s = *reinterpret_cast<const float4*>(&sDx[k & 3][c][q4]);
+#pragma unroll
+                    for (int ww = 0; ww < NW; ++ww) {
+                        const float4 v =
+                            *reinterpret_cast<const float4*>(&sY[(k & 1) * NW + ww][c][q4]);
+                        s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
+                    }
+                    if (has_z) {
+                        const float4 g = *reinterpret_cast<const float4*>(&sG[k & 3][c][q4]);
+                        s.x *= g.x; s.y *= g.y; s.z *= g.z; s.w *= g.w;
+                    }
+                    const float sv[4] = {s.x, s.y, s.z, s.w};
+                    const int t0 = k * kTile + q4;
+                    if (co_ok[r]) {
+#pragma unroll
+                        for (int j = 0; j < 4; ++j)
+                            if (t0 + j < p.L)
+                                yk[(uint32_t)(q4 + j) * (uint32_t)p.y_sl + cy[r]] = from_float<IO>(sv[j]);
+                    }
+                }
+            };
+            // the reducers run one tile behind the scan waves
             __syncthreads();
+            __syncthreads();
+            for (int k = 0; k < ntiles; ++k) {
+                if (k >= 1) reduce_store(k - 1);
+                __syncthreads();
+            }
+            reduce_store(ntiles - 1);
         }
-        reduce_store(ntiles - 1);
         return;
     }
 
@@ -272,12 +321,21 @@ __global__ void __launch_bounds__((NW + kService) * kWave) sscan_fwd_kernel(cons
     // Padded steps were staged as delta = 0, u = 0 (a = 2^0 = 1: h unchanged) and padded
     // states have A2 = 0, B = C = 0, so there is no tail handling.
     float bcb[2][kSub];  // wave-uniform: live in SGPRs; sub-tile j of a tile uses bcb[j & 1]
-    auto tile_compute = [&](int k, const float (&dl)[kTile], const float (&uu)[kTile]) {
+    auto tile_compute = [&](int k, const float (&dl)[kTile], const float (&uu)[kTile],
+                            float (&dl_next)[kTile], float (&uu_next)[kTile]) {
         const float* bck = bc + (int64_t)k * bc_tile;
         float acc[4];
 #pragma unroll
         for (int tt = 0; tt < kTile; ++tt) {
             const int sub = tt / kSS, ts = tt % kSS;
+            if (tt == kSS) {
+                // LDS prefetch of the next tile, placed after the first sub-tile: the scalar
+                // loads share their counter with LDS, so the wait that precedes the first use
+                // of B/C in a tile must not find these reads outstanding
+                __builtin_amdgcn_sched_barrier(0);
+                if (k + 1 < ntiles) read_tile(k + 1, dl_next, uu_next);
+                __builtin_amdgcn_sched_barrier(0);
+            }
             if (ts == 0) {
                 // fetch the next sub-tile (the first one of the next tile after the last)
                 if (sub + 1 < NSUB)
@@ -313,12 +371,10 @@ __global__ void __launch_bounds__((NW + kService) * kWave) sscan_fwd_kernel(cons
     read_tile(0, dlA, uuA);
     __syncthreads();
     for (int k = 0; k < ntiles; k += 2) {
-        if (k + 1 < ntiles) read_tile(k + 1, dlB, uuB);
-        tile_compute(k, dlA, uuA);
+        tile_compute(k, dlA, uuA, dlB, uuB);
         __syncthreads();
         if (k + 1 >= ntiles) break;
-        if (k + 2 < ntiles) read_tile(k + 2, dlA, uuA);
-        tile_compute(k + 1, dlB, uuB);
+        tile_compute(k + 1, dlB, uuB, dlA, uuA);
         __syncthreads();
     }
 
@@ -331,21 +387,23 @@ __global__ void __launch_bounds__((NW + kService) * kWave) sscan_fwd_kernel(cons
     }
 }
 
-template <typename IO, int NS, int NW>
+template <typename IO, int NS, int NW, bool HAS_Z>
 static int launch_fwd(const FwdParams& p, hipStream_t stream) {
     dim3 grid((p.ED + kWave - 1) / kWave, p.batch);
     dim3 block((NW + kService) * kWave);
     constexpr size_t lds = sizeof(float) * FwdLds<NS, NW>::floats;
-    static const int attr_rc = allow_dynamic_lds(sscan_fwd_kernel<IO, NS, NW>, lds);
+    static const int attr_rc = allow_dynamic_lds(sscan_fwd_kernel<IO, NS, NW, HAS_Z>, lds);
     if (attr_rc != MPA_OK) return attr_rc;
-    hipLaunchKernelGGL((sscan_fwd_kernel<IO, NS, NW>), grid, block, lds, stream, p);
+    hipLaunchKernelGGL((sscan_fwd_kernel<IO, NS, NW, HAS_Z>), grid, block, lds, stream, p);
     return check_launch();
 }
 
 template <typename IO>
 static int dispatch_fwd(const FwdParams& p, int ns, int nw, hipStream_t stream) {
-#define MPA_CASE(NS_, NW_) \
-    if (ns == NS_ && nw == NW_) return launch_fwd<IO, NS_, NW_>(p, stream);
+#define MPA_CASE(NS_, NW_)                                                        \
+    if (ns == NS_ && nw == NW_)                                                   \
+        return p.z ? launch_fwd<IO, NS_, NW_, true>(p, stream)                    \
+                   : launch_fwd<IO, NS_, NW_, false>(p, stream);
     MPA_CASE(2, 8) MPA_CASE(4, 4) MPA_CASE(8, 2) MPA_CASE(16, 1)
     MPA_CASE(4, 8) MPA_CASE(8, 4) MPA_CASE(16, 2) MPA_CASE(32, 1)
     MPA_CASE(8, 8) MPA_CASE(16, 4) MPA_CASE(32, 2)
@@ -365,6 +423,11 @@ int validate_shape(const mpa_sscan_shape* s) {
                           s->y_sd, s->g_sb, s->g_sl, s->g_sd, s->bc_sb, s->bc_sl, s->dbc_sb, s->dbc_sl};
     for (int64_t v : st)
         if (v < 0) return MPA_ERR_BAD_STRIDE;
+    // one (kTile steps x 64 channels) tile is addressed with 32-bit element offsets
+    const int64_t tile[][2] = {{s->u_sl, s->u_sd}, {s->d_sl, s->d_sd}, {s->y_sl, s->y_sd},
+                               {s->g_sl, s->g_sd}};
+    for (const auto& v : tile)
+        if (v[0] * kTile + v[1] * kWave >= ((int64_t)1 << 31)) return MPA_ERR_BAD_STRIDE;
     return MPA_OK;
 }
 
