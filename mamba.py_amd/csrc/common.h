@@ -59,6 +59,29 @@ __device__ __forceinline__ int wave_id() {
     return __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x) >> 6);
 }
 
+typedef float f16v __attribute__((ext_vector_type(16)));
+
+// B/C reach the scan waves in sub-tiles of kSS steps; two sub-tiles (the one in use and the
+// one in flight) must fit the scalar register file, so a sub-tile holds 32 floats (64 at 32
+// states per lane).
+template <int NS>
+struct BcPack {
+    static constexpr int kSS = NS >= 16 ? 1 : 16 / NS;
+};
+
+// COUNT consecutive floats through the scalar cache into SGPRs (the address is wave-uniform)
+template <int COUNT>
+__device__ __forceinline__ void scalar_load(const float* src, float (&dst)[COUNT]) {
+    static_assert(COUNT % 16 == 0, "scalar_load moves multiples of 16 floats");
+    const uintptr_t a = reinterpret_cast<uintptr_t>(src);
+#pragma unroll
+    for (int j = 0; j < COUNT / 16; ++j) {
+        const f16v v = *reinterpret_cast<const __attribute__((address_space(4))) f16v*>(a + 64 * j);
+#pragma unroll
+        for (int k = 0; k < 16; ++k) dst[16 * j + k] = v[k];
+    }
+}
+
 inline int check_launch() { return hipGetLastError() == hipSuccess ? MPA_OK : MPA_ERR_LAUNCH; }
 
 inline bool aligned_to(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }

@@ -1,0 +1,44 @@
+// Parameters shared by the two backward kernels of the fused selective scan.
+#pragma once
+
+#include "common.h"
+
+namespace mpa {
+
+struct BwdParams {
+    const void* x;
+    const void* delta;
+    const void* Bm;
+    const void* C;
+    const void* z;
+    const void* dy;
+    const float* A;
+    const float* D;
+    const float* dbias;
+    const float* h0;
+    const float* ckpt;
+    void* dx;
+    void* ddelta;
+    void* dz;
+    float* partB;   // [CG][batch][L][N]
+    float* partC;   // [CG][batch][L][N]
+    float* partA;   // [batch][ED][N]
+    float* partD;   // [batch][ED]
+    float* partDb;  // [batch][ED]  (ddelta_bias)
+    int batch, L, ED, N, nchunks;
+    int softplus;
+    int in_tmajor, dy_tmajor, out_tmajor;
+    int64_t u_sb, u_sl, u_sd;
+    int64_t d_sb, d_sl, d_sd;
+    int64_t y_sb, y_sl, y_sd;
+    int64_t g_sb, g_sl, g_sd;
+    int64_t bc_sb, bc_sl;
+};
+
+// Fast path (no gate): scan / loader / reducer waves, see sscan_bwd_fast.hip.  Returns
+// MPA_ERR_BAD_SHAPE when the shape is outside what it was instantiated for.
+int launch_bwd_fast(const BwdParams& p, const float* bcpack, int ns, int nw, int io_dtype,
+                    hipStream_t stream);
+bool bwd_fast_supported(int ns, int nw);
+
+}  // namespace mpa

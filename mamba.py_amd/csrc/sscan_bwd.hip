@@ -17,39 +17,9 @@
 // readout); over the 64 channels of a wave by a wave-private LDS transposition every four
 // steps; over channel groups, batch and time by deterministic partial buffers that a small
 // second kernel sums (no floating-point atomics: results are bitwise reproducible).
-#include "common.h"
+#include "sscan_bwd.h"
 
 namespace mpa {
-
-struct BwdParams {
-    const void* x;
-    const void* delta;
-    const void* Bm;
-    const void* C;
-    const void* z;
-    const void* dy;
-    const float* A;
-    const float* D;
-    const float* dbias;
-    const float* h0;
-    const float* ckpt;
-    void* dx;
-    void* ddelta;
-    void* dz;
-    float* partB;   // [CG][batch][L][N]
-    float* partC;   // [CG][batch][L][N]
-    float* partA;   // [batch][ED][N]
-    float* partD;   // [batch][ED]
-    float* partDb;  // [batch][ED]  (ddelta_bias)
-    int batch, L, ED, N, nchunks;
-    int softplus;
-    int in_tmajor, dy_tmajor, out_tmajor;
-    int64_t u_sb, u_sl, u_sd;
-    int64_t d_sb, d_sl, d_sd;
-    int64_t y_sb, y_sl, y_sd;
-    int64_t g_sb, g_sl, g_sd;
-    int64_t bc_sb, bc_sl;
-};
 
 constexpr int kPitchB = kWave + 1;
 constexpr int kRedPitch = kWave + 4;  // keeps 16-byte row alignment, conflict-free b128 reads
@@ -448,7 +418,7 @@ __global__ void __launch_bounds__(256) sscan_bwd_finish_kernel(
 }
 
 struct BwdWorkspace {
-    size_t offB, offC, offA, offD, offDb, total;
+    size_t offB, offC, offA, offD, offDb, offPack, total;
 };
 
 static BwdWorkspace bwd_workspace(const mpa_sscan_shape* s) {
@@ -463,7 +433,8 @@ static BwdWorkspace bwd_workspace(const mpa_sscan_shape* s) {
     w.offA = w.offC + up(cg * bln);
     w.offD = w.offA + up(ben);
     w.offDb = w.offD + up(be);
-    w.total = (w.offDb + up(be)) * sizeof(float);
+    w.offPack = w.offDb + up(be);
+    w.total = (w.offPack + up(bcpack_floats(s))) * sizeof(float);
     return w;
 }
 
@@ -546,7 +517,14 @@ extern "C" int mpa_sscan_bwd(const mpa_sscan_shape* s, const void* x, const void
     if (ns < 0) ns = 4;
     const int nw = np / ns;
     hipStream_t st = static_cast<hipStream_t>(stream);
-    if (s->io_dtype == MPA_F32)
+    const char* force_general = getenv("MPA_BWD_GENERAL");
+    if (!z && bwd_fast_supported(ns, nw) && !(force_general && force_general[0] == '1')) {
+        // fast path: B and C repacked as float32 for scalar loads, then the scan / loader /
+        // reducer kernel
+        float* pack = wsf + ws.offPack;
+        rc = launch_pack_bc(s, B, C, pack, ns, st);
+        if (rc == MPA_OK) rc = launch_bwd_fast(p, pack, ns, nw, s->io_dtype, st);
+    } else if (s->io_dtype == MPA_F32)
         rc = z ? dispatch_bwd<float, true>(p, ns, nw, st) : dispatch_bwd<float, false>(p, ns, nw, st);
     else
         rc = z ? dispatch_bwd<bf16_t, true>(p, ns, nw, st)

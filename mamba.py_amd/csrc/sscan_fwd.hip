@@ -92,29 +92,6 @@ struct FwdLds {
     static constexpr size_t floats = (size_t)(2 * 2 + 2 * 4 + 2 * NW) * kWave * kCP;
 };
 
-typedef float f16v __attribute__((ext_vector_type(16)));
-
-// B/C reach the scan waves in sub-tiles of kSS steps; two sub-tiles (the one in use and the
-// one in flight) must fit the scalar register file, so a sub-tile holds 32 floats (64 at 32
-// states per lane).
-template <int NS>
-struct BcPack {
-    static constexpr int kSS = NS >= 16 ? 1 : 16 / NS;
-};
-
-// COUNT consecutive floats through the scalar cache into SGPRs (the address is wave-uniform)
-template <int COUNT>
-__device__ __forceinline__ void scalar_load(const float* src, float (&dst)[COUNT]) {
-    static_assert(COUNT % 16 == 0, "scalar_load moves multiples of 16 floats");
-    const uintptr_t a = reinterpret_cast<uintptr_t>(src);
-#pragma unroll
-    for (int j = 0; j < COUNT / 16; ++j) {
-        const f16v v = *reinterpret_cast<const __attribute__((address_space(4))) f16v*>(a + 64 * j);
-#pragma unroll
-        for (int k = 0; k < 16; ++k) dst[16 * j + k] = v[k];
-    }
-}
-
 template <typename IO, int NS, int NW, bool HAS_Z>
 __global__ void __launch_bounds__((NW + kService) * kWave) sscan_fwd_kernel(const FwdParams p) {
     constexpr int NQ = kTile / 4;  // step groups (of 4) per tile
@@ -328,21 +305,6 @@ __global__ void __launch_bounds__((NW + kService) * kWave) sscan_fwd_kernel(cons
 #pragma unroll
         for (int tt = 0; tt < kTile; ++tt) {
             const int sub = tt / kSS, ts = tt % kSS;
-            if (tt == kSS) {
-                // LDS prefetch of the next tile, placed after the first sub-tile: the scalar
-                // loads share their counter with LDS, so the wait that precedes the first use
-                // of B/C in a tile must not find these reads outstanding
-                __builtin_amdgcn_sched_barrier(0);
-                if (k + 1 < ntiles) read_tile(k + 1, dl_next, uu_next);
-                __builtin_amdgcn_sched_barrier(0);
-            }
-            if (ts == 0) {
-                // fetch the next sub-tile (the first one of the next tile after the last)
-                if (sub + 1 < NSUB)
-                    scalar_load<kSub>(bck + (sub + 1) * kSub, bcb[(sub + 1) & 1]);
-                else if (k + 1 < ntiles)
-                    scalar_load<kSub>(bck + bc_tile, bcb[0]);
-            }
             const float(&cur)[kSub] = bcb[sub & 1];
             float sum = 0.0f;
 #pragma unroll
@@ -355,6 +317,22 @@ __global__ void __launch_bounds__((NW + kService) * kWave) sscan_fwd_kernel(cons
             if ((tt & 3) == 3)
                 *reinterpret_cast<float4*>(&sY[(k & 1) * NW + w][lane][tt - 3]) =
                     make_float4(acc[0], acc[1], acc[2], acc[3]);
+            if (ts == 0) {
+                // Prefetches are issued right AFTER the first step of a sub-tile has consumed
+                // its B/C: scalar loads return out of order and share their counter with LDS,
+                // so the wait that precedes the first use of a sub-tile drains everything in
+                // flight.  Placed here, that wait only ever finds loads issued a whole
+                // sub-tile earlier.
+                // (after the last tile the prefetches re-read valid memory and are ignored:
+                // no branch, so that the compiler cannot sink the arithmetic below them)
+                __builtin_amdgcn_sched_barrier(0);
+                if (sub + 1 < NSUB)
+                    scalar_load<kSub>(bck + (sub + 1) * kSub, bcb[(sub + 1) & 1]);
+                else
+                    scalar_load<kSub>(bc + (int64_t)min(k + 1, ntiles - 1) * bc_tile, bcb[0]);
+                if (sub == 0) read_tile(k + 1, dl_next, uu_next);
+                __builtin_amdgcn_sched_barrier(0);
+            }
         }
         if (p.ckpt && dvalid && k + 1 < ntiles) {
 #pragma unroll
