@@ -10,7 +10,7 @@
 //         d(delta*A) = g*a*h[t-1]   -> dA += .*delta ;  ddelta += .*A
 //         sum_n g*B                 -> dx = delta*. ;   ddelta += x*.
 //         g*u (u = delta*x), dy*h   -> dB, dC, summed over the 64 channels of the wave by a
-//                                      wave-private LDS transposition every RS steps.
+//                                      wave by an in-register reduce-scatter (rs_stage).
 //     B and C come through scalar loads from the float32 pack the pre-pass wrote.
 //   * two loader waves fetch x, delta, dy two tiles ahead, convert, apply softplus and
 //     publish delta, u, dy, x and D*dy as float32 LDS tiles; they also accumulate dD.
@@ -27,7 +27,7 @@
 namespace mpa {
 
 constexpr int kTileF = kWave * kTile;  // floats per LDS tile
-constexpr int kRedPitchF = kWave + 4;  // pitch of the channel-reduction rows (16-byte aligned)
+
 
 // float index of the 16-byte column q (4 steps) of channel ch inside a swizzled tile
 __device__ __forceinline__ int tile_off(int ch, int q) { return ch * kTile + 4 * (q ^ ((ch >> 2) & 3)); }
@@ -39,20 +39,48 @@ __device__ __forceinline__ void tile_st(float* tile, int ch, int q, float a, flo
     *reinterpret_cast<float4*>(tile + tile_off(ch, q)) = make_float4(a, b, c, d);
 }
 
-__device__ __forceinline__ void wave_lds_fence() {
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+// ---- in-register reduce-scatter over the 64 lanes of a wave ------------------------------
+// 64 values per lane are summed over all lanes in six halving stages; after stage s only
+// half of the registers remain, and a lane keeps the value whose index bit s equals the
+// matching lane bit, so that at the end lane l holds the complete sum of value number l and
+// each value cost (32+16+8+4+2+1)/64 adds plus the data movement, all on the VALU (no LDS
+// round trip sits in the dependency chain of the reverse sweep).
+//   stage 1: v_permlane32_swap  (lane bit 5)     stage 4: DPP row_half_mirror (lane bit 2)
+//   stage 2: v_permlane16_swap  (lane bit 4)     stage 5: DPP quad_perm 3210  (lane bit 1)
+//   stage 3: DPP row_mirror     (lane bit 3)     stage 6: DPP quad_perm 1032  (lane bit 0)
+// `lo` is the value with index bit 0 (kept by lanes whose bit is clear), `hi` the other one.
+__device__ __forceinline__ float rs_swap32(float lo, float hi) {
+    const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(lo), __float_as_uint(hi), false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+__device__ __forceinline__ float rs_swap16(float lo, float hi) {
+    const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(lo), __float_as_uint(hi), false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+template <int CTRL>
+__device__ __forceinline__ float rs_dpp(float lo, float hi, bool lane_bit) {
+    const float keep = lane_bit ? hi : lo;
+    const float send = lane_bit ? lo : hi;
+    const float got = __uint_as_float(
+        __builtin_amdgcn_update_dpp(0u, __float_as_uint(send), CTRL, 0xf, 0xf, false));
+    return keep + got;
+}
+// stage number (1..6) -> combine
+template <int STAGE>
+__device__ __forceinline__ float rs_stage(float lo, float hi, int lane) {
+    if constexpr (STAGE == 1) return rs_swap32(lo, hi);
+    else if constexpr (STAGE == 2) return rs_swap16(lo, hi);
+    else if constexpr (STAGE == 3) return rs_dpp<0x140>(lo, hi, (lane & 8) != 0);
+    else if constexpr (STAGE == 4) return rs_dpp<0x141>(lo, hi, (lane & 4) != 0);
+    else if constexpr (STAGE == 5) return rs_dpp<0x1B>(lo, hi, (lane & 2) != 0);
+    else return rs_dpp<0xB1>(lo, hi, (lane & 1) != 0);
 }
 
 template <int NS, int NW>
 struct BwdFastLds {
     static constexpr int NP = NS * NW;
-    static constexpr int RS = 2;                     // steps between two channel reductions
-    static constexpr int kRows = RS * 2 * NS;        // rows of a wave's reduction buffer
     static constexpr size_t kInputs = 4 * 4 + 2;     // delta, x, D*dy, dy: four buffers; u: two
-    static constexpr size_t floats = (kInputs + 2 * NW) * kTileF + (size_t)NW * kRows * kRedPitchF +
-                                     2 * kTile * 2 * NP + 2 * 4 * kWave;
+    static constexpr size_t floats = (kInputs + 2 * NW) * kTileF + 2 * kTile * 2 * NP + 2 * 4 * kWave;
 };
 
 template <typename IO, int NS, int NW>
@@ -60,14 +88,13 @@ __global__ void __launch_bounds__((NW + 4) * kWave)
     sscan_bwd_fast_kernel(const BwdParams p, const float* __restrict__ bcpack) {
     constexpr int NP = NS * NW;
     constexpr int NQ = kTile / 4;
-    constexpr int RS = BwdFastLds<NS, NW>::RS;
-    constexpr int kRows = BwdFastLds<NS, NW>::kRows;
-    constexpr int LPR = kWave / kRows;          // lanes sharing one reduction row
+    // channel reduction of dB/dC: 64 values (2 * NS per step, kBatch steps) per reduce-scatter
+    constexpr int kStepBits = NS == 2 ? 2 : 3;  // stages spent inside one step: log2(2*NS)
+    constexpr int kBatch = 64 / (2 * NS);       // steps per batch
+    static_assert(NS == 2 || NS == 4, "reduce-scatter layout written for 2 or 4 states per lane");
     constexpr int kSS = BcPack<NS>::kSS;        // steps per B/C sub-tile
     constexpr int NSUB = kTile / kSS;
     constexpr int kSub = 2 * kSS * NS;          // floats per sub-tile: B then C
-    static_assert(kRows <= kWave && kWave % kRows == 0, "reduction rows must tile one wave");
-    static_assert(kSS % RS == 0 || RS % kSS == 0, "sub-tiles and reduction batches must nest");
 
     extern __shared__ float4 smem4[];
     float* const smem = reinterpret_cast<float*>(smem4);
@@ -78,8 +105,7 @@ __global__ void __launch_bounds__((NW + 4) * kWave)
     float* const sU = sDy + 4 * kTileF;           // [2] u = delta*x
     float* const sP1 = sU + 2 * kTileF;           // [NW] sum_n g*B
     float* const sP2 = sP1 + NW * kTileF;         // [NW] sum_n g*a*h[t-1]*A*log2(e)
-    float* const sR = sP2 + NW * kTileF;          // [NW][kRows][kRedPitchF]
-    float* const sRed = sR + NW * kRows * kRedPitchF;  // [2][kTile][2][NP] dB | dC tile sums
+    float* const sRed = sP2 + NW * kTileF;        // [2][kTile][2][NP] dB | dC tile sums
     float* const sDD = sRed + 2 * kTile * 2 * NP;      // [2][4][kWave] dD, ddelta_bias partials
 
     const int lane = threadIdx.x & (kWave - 1);
@@ -315,7 +341,6 @@ __global__ void __launch_bounds__((NW + 4) * kWave)
     };
     const float* bc = bcpack + ((int64_t)b * ntiles * NW + w) * (NSUB * kSub);
     const int64_t bc_tile = (int64_t)NW * NSUB * kSub;
-    float* const myR = sR + w * kRows * kRedPitchF;
 
     auto read_fwd_inputs = [&](int k, float (&dl)[kTile], float (&uu)[kTile]) {
 #pragma unroll
@@ -342,7 +367,7 @@ __global__ void __launch_bounds__((NW + 4) * kWave)
         for (int i = 0; i < NS; ++i) h[i] = hnext[i];
 
         // ---- 1. recompute the tile forward, keeping a and a*h[t-1] ----
-        float aS[kTile][NS], tS[kTile][NS], dyr[kTile];
+        float aS[kTile][NS], tS[kTile][NS], dyq[2][4];
 #pragma unroll
         for (int tt = 0; tt < kTile; ++tt) {
             const int sub = tt / kSS, ts = tt % kSS;
@@ -365,12 +390,10 @@ __global__ void __launch_bounds__((NW + 4) * kWave)
                     scalar_load<kSub>(bck + (NSUB - 1) * kSub, bcb[NSUB & 1]);
                 if (sub == 0) load_state(k + 1, hnext);
                 if (sub == NSUB - 1) {
-                    // dy of the tile, needed from the first step of the reverse sweep
-#pragma unroll
-                    for (int q = 0; q < NQ; ++q) {
-                        const float4 v = tile_ld(sDy + (k & 3) * kTileF, lane, q);
-                        dyr[4 * q] = v.x; dyr[4 * q + 1] = v.y; dyr[4 * q + 2] = v.z; dyr[4 * q + 3] = v.w;
-                    }
+                    // dy of the last four steps, needed when the reverse sweep starts
+                    const float4 v = tile_ld(sDy + (k & 3) * kTileF, lane, NQ - 1);
+                    dyq[(NQ - 1) & 1][0] = v.x; dyq[(NQ - 1) & 1][1] = v.y;
+                    dyq[(NQ - 1) & 1][2] = v.z; dyq[(NQ - 1) & 1][3] = v.w;
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
@@ -378,14 +401,21 @@ __global__ void __launch_bounds__((NW + 4) * kWave)
 
         // ---- 2. reverse sweep ----
         float gBv[kTile], ddv[kTile];
+        float pend[4];
 #pragma unroll
         for (int tt = kTile - 1; tt >= 0; --tt) {
             const int sub = tt / kSS, ts = tt % kSS;
             const int fetch = NSUB + (NSUB - 1 - sub);  // fetch number of this sub-tile
             const float(&cur)[kSub] = bcb[fetch & 1];
-            const float dyv = dyr[tt];
+            if ((tt & 3) == 3 && tt >= 4) {
+                // dy of the next (earlier) four steps, one group ahead of use
+                const int qn = (tt >> 2) - 1;
+                const float4 v = tile_ld(sDy + (k & 3) * kTileF, lane, qn);
+                dyq[qn & 1][0] = v.x; dyq[qn & 1][1] = v.y; dyq[qn & 1][2] = v.z; dyq[qn & 1][3] = v.w;
+            }
+            const float dyv = dyq[(tt >> 2) & 1][tt & 3];
             float gB = 0.0f, dd = 0.0f;
-            const int slot = tt % RS;
+            float pB[NS], pC[NS];
 #pragma unroll
             for (int i = 0; i < NS; ++i) {
                 const float bv = cur[ts * NS + i];
@@ -397,8 +427,8 @@ __global__ void __launch_bounds__((NW + 4) * kWave)
                 dd = __builtin_fmaf(gha, A2[i], dd);
                 gB = __builtin_fmaf(g, bv, gB);
                 ag[i] = aS[tt][i] * g;
-                myR[(slot * 2 * NS + i) * kRedPitchF + lane] = g * uu[tt];
-                myR[(slot * 2 * NS + NS + i) * kRedPitchF + lane] = dyv * hh;
+                pB[i] = g * uu[tt];
+                pC[i] = dyv * hh;
             }
             gBv[tt] = gB;
             ddv[tt] = dd;
@@ -419,24 +449,50 @@ __global__ void __launch_bounds__((NW + 4) * kWave)
                 read_fwd_inputs(k + 1, dl_next, uu_next);
                 __builtin_amdgcn_sched_barrier(0);
             }
-            if (slot == 0) {
-                // channel reduction of the last RS steps: row = (step, dB|dC, state); LPR
-                // lanes share a row and each sums kWave/LPR consecutive channels
-                wave_lds_fence();
-                const int row = lane / LPR, part = lane % LPR;
-                const float4* src = reinterpret_cast<const float4*>(myR + row * kRedPitchF + part * (kWave / LPR));
-                float s = 0.0f;
-#pragma unroll
-                for (int j = 0; j < kWave / LPR / 4; ++j) {
-                    const float4 v = src[j];
-                    s += (v.x + v.y) + (v.z + v.w);
+            // ---- channel reduction of this step's dB / dC products (see rs_stage) ----
+            // value index bits, from stage 1 up: dB|dC, the state index, then the step index
+            // inside the batch; steps arrive in descending order, so a step with a set index
+            // bit waits in `pend` for its partner with the bit clear
+            {
+                float r;
+                if constexpr (NS == 2) {
+                    r = rs_stage<2>(rs_stage<1>(pB[0], pC[0], lane), rs_stage<1>(pB[1], pC[1], lane), lane);
+                } else {
+                    const float a0 = rs_stage<1>(pB[0], pC[0], lane), a1 = rs_stage<1>(pB[1], pC[1], lane);
+                    const float a2 = rs_stage<1>(pB[2], pC[2], lane), a3 = rs_stage<1>(pB[3], pC[3], lane);
+                    r = rs_stage<3>(rs_stage<2>(a0, a2, lane), rs_stage<2>(a1, a3, lane), lane);
                 }
-#pragma unroll
-                for (int m = 1; m < LPR; m *= 2) s += __shfl_xor(s, m, kWave);
-                const int rs = row / (2 * NS), o = row % (2 * NS);
-                if (part == 0)
-                    sRed[(k & 1) * (kTile * 2 * NP) + ((tt + rs) * 2 + (o >= NS ? 1 : 0)) * NP + w * NS + (o % NS)] = s;
-                wave_lds_fence();
+                const int sb = tt % kBatch;  // step inside the batch
+                if (sb & 1) {
+                    pend[0] = r;
+                } else {
+                    r = rs_stage<kStepBits + 1>(r, pend[0], lane);
+                    if (sb & 2) {
+                        pend[1] = r;
+                    } else {
+                        r = rs_stage<kStepBits + 2>(r, pend[1], lane);
+                        if (sb & 4) {
+                            pend[2] = r;
+                        } else {
+                            r = rs_stage<kStepBits + 3>(r, pend[2], lane);
+                            if constexpr (kBatch == 16) {
+                                if (sb & 8) {
+                                    pend[3] = r;
+                                } else {
+                                    r = rs_stage<6>(r, pend[3], lane);
+                                }
+                            }
+                            if (sb == 0) {
+                                // lane l holds value number l: decode (step, dB|dC, state)
+                                const int which = lane >> 5;
+                                const int st = NS == 2 ? (lane >> 4) & 1 : (((lane >> 4) & 1) << 1) | ((lane >> 3) & 1);
+                                const int stp = NS == 2 ? (lane & 1) << 3 | (lane & 2) << 1 | (lane & 4) >> 1 | (lane & 8) >> 3
+                                                        : (lane & 1) << 2 | (lane & 2) | (lane & 4) >> 2;
+                                sRed[(k & 1) * (kTile * 2 * NP) + ((tt + stp) * 2 + which) * NP + w * NS + st] = r;
+                            }
+                        }
+                    }
+                }
             }
         }
         __syncthreads();  // B1(k): the reducers are done with the partials of tile k-1
