@@ -1,0 +1,258 @@
+"""Callers of the selective-scan hot path, restated on top of the gfx950 kernels.
+
+These classes mirror the reference's public surface (constructor arguments, method names,
+tensor shapes and `state_dict` keys) so that a model built or trained with mambapy loads
+here and the other way round:
+    MambaConfig, MambaBlock, ResidualBlock, Mamba, RMSNorm      mambapy/mamba.py:31-433
+They are the harness around the kernels, not the product: projections, the depthwise
+convolution and the norms stay on PyTorch-ROCm library calls; the scan, its backward and the
+decode-step state update run in libmambapy_amd.so.
+"""
+import math
+from dataclasses import dataclass
+from typing import Optional, Tuple, Union
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+from .scan import selective_scan, selective_scan_fn, ssm_step
+
+
+@dataclass
+class MambaConfig:
+    """Same fields and derived values as mambapy/mamba.py:31-67 (d_inner = expand_factor *
+    d_model, dt_rank = ceil(d_model / 16) when 'auto').  `pscan` / `use_cuda` are accepted for
+    compatibility; both select the fused HIP scan here.  `fused_softplus` folds
+    softplus(delta + dt_proj.bias) into the scan kernel (the reference does so only on its
+    `use_cuda` path, mamba.py:259-260)."""
+    d_model: int
+    n_layers: int
+    dt_rank: Union[int, str] = "auto"
+    d_state: int = 16
+    expand_factor: int = 2
+    d_conv: int = 4
+
+    dt_min: float = 0.001
+    dt_max: float = 0.1
+    dt_init: str = "random"
+    dt_scale: float = 1.0
+    dt_init_floor: float = 1e-4
+
+    rms_norm_eps: float = 1e-5
+    base_std: float = 0.02
+
+    bias: bool = False
+    conv_bias: bool = True
+    inner_layernorms: bool = False
+
+    mup: bool = False
+    mup_base_width: float = 128
+
+    pscan: bool = True
+    use_cuda: bool = False
+    fused_softplus: bool = True
+
+    def __post_init__(self):
+        self.d_inner = self.expand_factor * self.d_model
+        if self.dt_rank == "auto":
+            self.dt_rank = math.ceil(self.d_model / 16)
+        if self.mup:
+            self.mup_width_mult = self.d_model / self.mup_base_width
+
+
+class RMSNorm(nn.Module):
+    """x * rsqrt(mean(x^2) + eps) [* weight]  (mambapy/mamba.py:416-433; no gain under muP)."""
+
+    def __init__(self, d_model: int, eps: float = 1e-5, use_mup: bool = False):
+        super().__init__()
+        self.eps = eps
+        self.use_mup = use_mup
+        if not use_mup:
+            self.weight = nn.Parameter(torch.ones(d_model))
+
+    def forward(self, x):
+        y = x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + self.eps)
+        return y if self.use_mup else y * self.weight
+
+
+class MambaBlock(nn.Module):
+    """The mixer of mambapy/mamba.py:127-414 with the scan replaced by the HIP kernels.
+
+    Parameters (state_dict keys): in_proj.weight, conv1d.weight (ED,1,d_conv), conv1d.bias,
+    x_proj.weight, dt_proj.weight, dt_proj.bias, A_log (ED,N), D (ED), out_proj.weight.
+    """
+
+    def __init__(self, config: MambaConfig):
+        super().__init__()
+        self.config = config
+        ED, N, R = config.d_inner, config.d_state, config.dt_rank
+        self.in_proj = nn.Linear(config.d_model, 2 * ED, bias=config.bias)
+        self.conv1d = nn.Conv1d(ED, ED, kernel_size=config.d_conv, groups=ED,
+                                padding=config.d_conv - 1, bias=config.conv_bias)
+        self.x_proj = nn.Linear(ED, R + 2 * N, bias=False)
+        self.dt_proj = nn.Linear(R, ED, bias=True)
+        self.out_proj = nn.Linear(ED, config.d_model, bias=config.bias)
+
+        # initial values as in mamba.py:147-172: dt_proj.weight uniform or constant,
+        # dt_proj.bias = inverse softplus of a log-uniform step in [dt_min, dt_max],
+        # A = -(1..N) per channel stored as log (S4D-real), D = 1
+        bound = R ** -0.5 * config.dt_scale
+        if config.dt_init == "constant":
+            nn.init.constant_(self.dt_proj.weight, bound)
+        elif config.dt_init == "random":
+            nn.init.uniform_(self.dt_proj.weight, -bound, bound)
+        else:
+            raise NotImplementedError(f"dt_init={config.dt_init!r}")
+        lo, hi = math.log(config.dt_min), math.log(config.dt_max)
+        dt = torch.exp(torch.rand(ED) * (hi - lo) + lo).clamp(min=config.dt_init_floor)
+        with torch.no_grad():
+            self.dt_proj.bias.copy_(dt + torch.log(-torch.expm1(-dt)))
+        self.A_log = nn.Parameter(torch.log(torch.arange(1, N + 1, dtype=torch.float32)).repeat(ED, 1))
+        self.A_log._no_weight_decay = True
+        self.D = nn.Parameter(torch.ones(ED))
+        self.D._no_weight_decay = True
+
+        if config.inner_layernorms:
+            self.dt_layernorm = RMSNorm(R, config.rms_norm_eps, config.mup)
+            self.B_layernorm = RMSNorm(N, config.rms_norm_eps, config.mup)
+            self.C_layernorm = RMSNorm(N, config.rms_norm_eps, config.mup)
+        else:
+            self.dt_layernorm = self.B_layernorm = self.C_layernorm = None
+
+    # -- helpers -------------------------------------------------------------------------
+    def _split_projection(self, dbc):
+        R, N = self.config.dt_rank, self.config.d_state
+        dlow, Bm, C = torch.split(dbc, [R, N, N], dim=-1)
+        if self.dt_layernorm is not None:
+            dlow, Bm, C = self.dt_layernorm(dlow), self.B_layernorm(Bm), self.C_layernorm(C)
+        return dlow, Bm, C
+
+    def _A(self):
+        return -torch.exp(self.A_log.float())
+
+    # -- training / prefill ---------------------------------------------------------------
+    def forward(self, x, cache: Optional[Tuple] = None, return_cache: bool = False):
+        """x : (B, L, D) -> (B, L, D).  With return_cache=True also returns the decode cache
+        (h (B,ED,N) float32, inputs (B,ED,d_conv-1)) after the last position, so that
+        generation can continue with step() instead of re-running the sequence."""
+        L = x.shape[1]
+        xz = self.in_proj(x)
+        xin, z = xz.chunk(2, dim=-1)
+        # causal depthwise convolution along time, kept in (B, ED, L) memory: the scan kernel
+        # reads this layout directly
+        xc = self.conv1d(xin.transpose(1, 2))[:, :, :L]
+        xs = F.silu(xc).transpose(1, 2)                      # (B, L, ED), unit stride along L
+        if return_cache:
+            y, h_last = self.ssm(xs, z, return_last_state=True)
+        else:
+            y = self.ssm(xs, z)
+        out = self.out_proj(y * F.silu(z))
+        if not return_cache:
+            return out
+        K = self.config.d_conv - 1
+        pre = xin.transpose(1, 2)
+        if L >= K:
+            window = pre[:, :, L - K:].contiguous()
+        else:
+            window = F.pad(pre, (K - L, 0)).contiguous()
+        return out, (h_last, window)
+
+    def ssm(self, x, z=None, return_last_state: bool = False):
+        """(B, L, ED) -> (B, L, ED): projections to (delta, B, C), then the fused scan
+        (mambapy/mamba.py:236-272)."""
+        A, D = self._A(), self.D.float()
+        dlow, Bm, C = self._split_projection(self.x_proj(x))
+        delta = (self.dt_proj.weight @ dlow.transpose(1, 2)).transpose(1, 2)   # (B, L, ED) view
+        if self.config.fused_softplus:
+            return selective_scan_fn(x, delta, A, Bm, C, D, delta_bias=self.dt_proj.bias,
+                                     delta_softplus=True, return_last_state=return_last_state)
+        delta = F.softplus(delta + self.dt_proj.bias)
+        return selective_scan_fn(x, delta, A, Bm, C, D, return_last_state=return_last_state)
+
+    def selective_scan(self, x, delta, A, B, C, D):
+        """Same call as MambaBlock.selective_scan (mambapy/mamba.py:274-295)."""
+        return selective_scan(x, delta, A, B, C, D)
+
+    def selective_scan_seq(self, x, delta, A, B, C, D):
+        """The reference keeps a sequential twin (mamba.py:297-327); both names run the same
+        kernel here."""
+        return selective_scan(x, delta, A, B, C, D)
+
+    # -- decode -----------------------------------------------------------------------------
+    def step(self, x, cache):
+        """x : (B, D), cache = (h (B,ED,N) or None, inputs (B,ED,d_conv-1)) ->
+        (y (B, D), new cache); mambapy/mamba.py:351-382.  The old cache tuple stays valid."""
+        h, inputs = cache
+        xz = self.in_proj(x)
+        xin, z = xz.chunk(2, dim=1)
+        window = torch.cat([inputs, xin.unsqueeze(2)], dim=2)            # (B, ED, d_conv)
+        xc = (window * self.conv1d.weight[:, 0, :]).sum(-1)
+        if self.conv1d.bias is not None:
+            xc = xc + self.conv1d.bias
+        xs = F.silu(xc)
+        y, h = self.ssm_step(xs, h, z=z)
+        out = self.out_proj(y)
+        return out, (h, window[:, :, 1:])
+
+    def ssm_step(self, x, h, z=None):
+        """x : (B, ED), h : (B, ED, N) or None -> (y, h'); mambapy/mamba.py:384-414.  With z
+        the gate y*silu(z) is applied inside the kernel."""
+        dlow, Bm, C = self._split_projection(self.x_proj(x))
+        raw = F.linear(dlow, self.dt_proj.weight)                        # bias added in-kernel
+        y, h_new = ssm_step(x, raw, self._A(), Bm, C, self.D.float(), h, z=z,
+                            delta_bias=self.dt_proj.bias, delta_softplus=True)
+        return y, h_new
+
+
+class ResidualBlock(nn.Module):
+    """mixer(norm(x)) + x  (mambapy/mamba.py:99-125); keys: mixer.*, norm.weight."""
+
+    def __init__(self, config: MambaConfig):
+        super().__init__()
+        self.mixer = MambaBlock(config)
+        self.norm = RMSNorm(config.d_model, config.rms_norm_eps, config.mup)
+
+    def forward(self, x, return_cache: bool = False):
+        if return_cache:
+            y, cache = self.mixer(self.norm(x), return_cache=True)
+            return y + x, cache
+        return self.mixer(self.norm(x)) + x
+
+    def step(self, x, cache):
+        y, cache = self.mixer.step(self.norm(x), cache)
+        return y + x, cache
+
+
+class Mamba(nn.Module):
+    """Stack of residual blocks (mambapy/mamba.py:69-97); keys: layers.{i}.*"""
+
+    def __init__(self, config: MambaConfig):
+        super().__init__()
+        self.config = config
+        self.layers = nn.ModuleList([ResidualBlock(config) for _ in range(config.n_layers)])
+
+    def forward(self, x, return_caches: bool = False):
+        if not return_caches:
+            for layer in self.layers:
+                x = layer(x)
+            return x
+        caches = []
+        for layer in self.layers:
+            x, c = layer(x, return_cache=True)
+            caches.append(c)
+        return x, caches
+
+    def step(self, x, caches):
+        for i, layer in enumerate(self.layers):
+            x, caches[i] = layer.step(x, caches[i])
+        return x, caches
+
+    def empty_caches(self, batch: int, device=None, dtype=None):
+        """Fresh decode caches: h = None (zero state), zero conv window (mamba.py:344-346)."""
+        cfg = self.config
+        p = self.layers[0].mixer.in_proj.weight
+        device = device or p.device
+        dtype = dtype or p.dtype
+        return [(None, torch.zeros(batch, cfg.d_inner, cfg.d_conv - 1, device=device, dtype=dtype))
+                for _ in self.layers]
