@@ -84,6 +84,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="also run a plain 256 MiB device copy (reference point that scales the "
+                         "FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU (one process, one MI355X); "
@@ -116,6 +119,13 @@ def main():
         y.backward(dy)
         if events:
             events[2].record()
+
+    if args.copy_probe:
+        src = torch.empty(256 * 1024 * 1024, dtype=torch.uint8, device=dev).zero_()
+        for _ in range(3):
+            dst = src.clone()
+        torch.cuda.synchronize()
+        del src, dst
 
     for _ in range(args.warmup):
         step()

@@ -13,12 +13,11 @@
 //                                      wave by an in-register reduce-scatter (rs_stage).
 //     B and C come through scalar loads from the float32 pack the pre-pass wrote.
 //   * two loader waves fetch x, delta, dy two tiles ahead, convert, apply softplus and
-//     publish delta, u, dy, x and D*dy as float32 LDS tiles; they also accumulate dD.
+//     publish delta, u, dy and x as float32 LDS tiles; they also accumulate dD.
 //   * two reducer waves, one tile behind, sum the partial sum_n over the scan waves, finish
 //     dx and ddelta (softplus chain rule included), store them, and forward the per-tile
 //     dB/dC sums to the per-channel-group partial buffers.
-// Tiles in LDS are [64 channels][16 steps] float32 with an XOR swizzle of the 16-byte column
-// so that pitch-16 rows are conflict-free for 16-byte accesses.
+// Tiles in LDS are [64 channels][16 steps] float32 at a pitch of 20 floats.
 // Reductions over channel groups, batch and time go through deterministic partial buffers
 // summed by sscan_bwd_finish_kernel (no floating-point atomics: results are bitwise
 // reproducible).
@@ -26,11 +25,13 @@
 
 namespace mpa {
 
-constexpr int kTileF = kWave * kTile;  // floats per LDS tile
+constexpr int kPitchT = kTile + 4;         // row pitch (floats) of a [channel][step] LDS tile: rows stay
+                                          // 16-byte aligned and 16-byte accesses are conflict-free
+constexpr int kTileF = kWave * kPitchT;   // floats per LDS tile
 
 
-// float index of the 16-byte column q (4 steps) of channel ch inside a swizzled tile
-__device__ __forceinline__ int tile_off(int ch, int q) { return ch * kTile + 4 * (q ^ ((ch >> 2) & 3)); }
+// float index of the 16-byte column q (4 steps) of channel ch inside a tile
+__device__ __forceinline__ int tile_off(int ch, int q) { return ch * kPitchT + 4 * q; }
 
 __device__ __forceinline__ float4 tile_ld(const float* tile, int ch, int q) {
     return *reinterpret_cast<const float4*>(tile + tile_off(ch, q));
@@ -79,7 +80,7 @@ __device__ __forceinline__ float rs_stage(float lo, float hi, int lane) {
 template <int NS, int NW>
 struct BwdFastLds {
     static constexpr int NP = NS * NW;
-    static constexpr size_t kInputs = 4 * 4 + 2;     // delta, x, D*dy, dy: four buffers; u: two
+    static constexpr size_t kInputs = 3 * 4 + 2;     // delta, x, dy: four buffers each; u: two
     static constexpr size_t floats = (kInputs + 2 * NW) * kTileF + 2 * kTile * 2 * NP + 2 * 4 * kWave;
 };
 
@@ -100,8 +101,7 @@ __global__ void __launch_bounds__((NW + 4) * kWave)
     float* const smem = reinterpret_cast<float*>(smem4);
     float* const sDl = smem;                      // [4] delta (after softplus)
     float* const sX = sDl + 4 * kTileF;           // [4] x
-    float* const sDdy = sX + 4 * kTileF;          // [4] D*dy
-    float* const sDy = sDdy + 4 * kTileF;         // [4] dy
+    float* const sDy = sX + 4 * kTileF;           // [4] dy
     float* const sU = sDy + 4 * kTileF;           // [2] u = delta*x
     float* const sP1 = sU + 2 * kTileF;           // [NW] sum_n g*B
     float* const sP2 = sP1 + NW * kTileF;         // [NW] sum_n g*a*h[t-1]*A*log2(e)
@@ -125,6 +125,7 @@ __global__ void __launch_bounds__((NW + 4) * kWave)
         int co[2], qo[2];
         bool co_ok[2];
         uint32_t cgo[2];
+        float Dr[2];
         float dDb[2] = {0.0f, 0.0f};
 #pragma unroll
         for (int r = 0; r < 2; ++r) {
@@ -133,6 +134,7 @@ __global__ void __launch_bounds__((NW + 4) * kWave)
             qo[r] = p.out_tmajor ? item % NQ : item / kWave;
             co_ok[r] = co[r] <= cmax;
             cgo[r] = (uint32_t)min(co[r], cmax) * (uint32_t)p.g_sd;
+            Dr[r] = p.D[d0 + min(co[r], cmax)];
         }
         IO* const dxg = static_cast<IO*>(p.dx) + (b * p.g_sb + (int64_t)d0 * p.g_sd);
         IO* const ddg = static_cast<IO*>(p.ddelta) + (b * p.g_sb + (int64_t)d0 * p.g_sd);
@@ -155,14 +157,14 @@ __global__ void __launch_bounds__((NW + 4) * kWave)
                 }
                 const float4 dl = tile_ld(sDl + (k & 3) * kTileF, ch, q);
                 const float4 xv = tile_ld(sX + (k & 3) * kTileF, ch, q);
-                const float4 ddy = tile_ld(sDdy + (k & 3) * kTileF, ch, q);
+                const float4 ddy = tile_ld(sDy + (k & 3) * kTileF, ch, q);
                 const float gBv[4] = {gB.x, gB.y, gB.z, gB.w}, ddv[4] = {dd.x, dd.y, dd.z, dd.w};
                 const float dlv[4] = {dl.x, dl.y, dl.z, dl.w}, xvv[4] = {xv.x, xv.y, xv.z, xv.w};
                 const float dyv[4] = {ddy.x, ddy.y, ddy.z, ddy.w};
                 const int t0 = c * kTile + 4 * q;
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
-                    const float dxv = __builtin_fmaf(dlv[j], gBv[j], dyv[j]);
+                    const float dxv = __builtin_fmaf(dlv[j], gBv[j], Dr[r] * dyv[j]);
                     float dv = __builtin_fmaf(xvv[j], gBv[j], ddv[j] * kLn2);
                     if (p.softplus) {
                         // d softplus(r)/dr = sigmoid(r) = 1 - exp(-softplus(r))
@@ -210,7 +212,7 @@ __global__ void __launch_bounds__((NW + 4) * kWave)
         int ci[2], qi[2];
         bool ci_ok[2];
         uint32_t cx[2], cd[2], cy[2];
-        float Dv[2], bias[2], dDacc[2] = {0.0f, 0.0f};
+        float bias[2], dDacc[2] = {0.0f, 0.0f};
 #pragma unroll
         for (int r = 0; r < 2; ++r) {
             const int item = sw * kWave + lane + r * 2 * kWave;
@@ -221,7 +223,6 @@ __global__ void __launch_bounds__((NW + 4) * kWave)
             cx[r] = (uint32_t)cic * (uint32_t)p.u_sd;
             cd[r] = (uint32_t)cic * (uint32_t)p.d_sd;
             cy[r] = (uint32_t)cic * (uint32_t)p.y_sd;
-            Dv[r] = p.D[d0 + cic];
             bias[r] = p.dbias ? p.dbias[d0 + cic] : 0.0f;
         }
         const IO* const xg = static_cast<const IO*>(p.x) + (b * p.u_sb + (int64_t)d0 * p.u_sd);
@@ -253,7 +254,7 @@ __global__ void __launch_bounds__((NW + 4) * kWave)
 #pragma unroll
             for (int r = 0; r < 2; ++r) {
                 const int t0 = c * kTile + 4 * qi[r];
-                float dl[4], uu[4], xx[4], yy[4], dd[4];
+                float dl[4], uu[4], xx[4], yy[4];
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
                     // padding (beyond the sequence or the channel count): delta = 0, u = 0,
@@ -268,7 +269,6 @@ __global__ void __launch_bounds__((NW + 4) * kWave)
                     uu[j] = dv * xv;
                     xx[j] = xv;
                     yy[j] = yv;
-                    dd[j] = Dv[r] * yv;
                     dDacc[r] = __builtin_fmaf(yv, xv, dDacc[r]);
                 }
                 const int ch = ci[r], q = qi[r], s4 = (k & 3) * kTileF;
@@ -276,7 +276,6 @@ __global__ void __launch_bounds__((NW + 4) * kWave)
                 tile_st(sU + (k & 1) * kTileF, ch, q, uu[0], uu[1], uu[2], uu[3]);
                 tile_st(sDy + s4, ch, q, yy[0], yy[1], yy[2], yy[3]);
                 tile_st(sX + s4, ch, q, xx[0], xx[1], xx[2], xx[3]);
-                tile_st(sDdy + s4, ch, q, dd[0], dd[1], dd[2], dd[3]);
             }
         };
 
