@@ -81,7 +81,7 @@ template <int NS, int NW>
 struct BwdFastLds {
     static constexpr int NP = NS * NW;
     static constexpr size_t kInputs = 3 * 4 + 2;     // delta, x, dy: four buffers each; u: two
-    static constexpr size_t floats = (kInputs + 2 * NW) * kTileF + 2 * kTile * 2 * NP + 2 * 4 * kWave;
+    static constexpr size_t floats = (kInputs + 2 * NW) * kTileF + 2 * kTile * 2 * NP + 2 * 4 * kWave + 4;
 };
 
 template <typename IO, int NS, int NW>
@@ -107,6 +107,8 @@ __global__ void __launch_bounds__((NW + 4) * kWave)
     float* const sP2 = sP1 + NW * kTileF;         // [NW] sum_n g*a*h[t-1]*A*log2(e)
     float* const sRed = sP2 + NW * kTileF;        // [2][kTile][2][NP] dB | dC tile sums
     float* const sDD = sRed + 2 * kTile * 2 * NP;      // [2][4][kWave] dD, ddelta_bias partials
+    // one word per reducer wave: index of the last tile whose partial sums it has consumed
+    int* const sConsumed = reinterpret_cast<int*>(sDD + 2 * 4 * kWave);
 
     const int lane = threadIdx.x & (kWave - 1);
     const int w = wave_id();
@@ -144,6 +146,7 @@ __global__ void __launch_bounds__((NW + 4) * kWave)
             const int c = chunk_of(k);
             IO* dxk = dxg + (int64_t)c * kTile * p.g_sl;
             IO* ddk = ddg + (int64_t)c * kTile * p.g_sl;
+            float4 gBs[2], dds[2];
 #pragma unroll
             for (int r = 0; r < 2; ++r) {
                 const int ch = co[r], q = qo[r];
@@ -155,6 +158,17 @@ __global__ void __launch_bounds__((NW + 4) * kWave)
                     gB.x += a.x; gB.y += a.y; gB.z += a.z; gB.w += a.w;
                     dd.x += e.x; dd.y += e.y; dd.z += e.z; dd.w += e.w;
                 }
+                gBs[r] = gB;
+                dds[r] = dd;
+            }
+            // the partial sums of tile k are in registers: the scan waves may overwrite them
+            // (the release orders this store after the LDS reads above)
+            if (lane == 0)
+                __hip_atomic_store(sConsumed + sw, k, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
+#pragma unroll
+            for (int r = 0; r < 2; ++r) {
+                const int ch = co[r], q = qo[r];
+                const float4 gB = gBs[r], dd = dds[r];
                 const float4 dl = tile_ld(sDl + (k & 3) * kTileF, ch, q);
                 const float4 xv = tile_ld(sX + (k & 3) * kTileF, ch, q);
                 const float4 ddy = tile_ld(sDy + (k & 3) * kTileF, ch, q);
@@ -190,12 +204,12 @@ __global__ void __launch_bounds__((NW + 4) * kWave)
             }
         };
 
+        if (lane == 0) sConsumed[sw] = -1;
         __syncthreads();
         __syncthreads();
         for (int k = 0; k < ntiles; ++k) {
             if (k >= 1) reduce_store(k - 1);
-            __syncthreads();  // B1(k)
-            __syncthreads();  // B2(k)
+            __syncthreads();  // end of interval k
         }
         reduce_store(ntiles - 1);
         if (p.softplus) {
@@ -291,8 +305,7 @@ __global__ void __launch_bounds__((NW + 4) * kWave)
         for (int k = 0; k < ntiles; ++k) {
             if (k + 2 < ntiles) stage_tile(k + 2);
             if (k + 3 < ntiles) load_tile(k + 3);
-            __syncthreads();  // B1(k)
-            __syncthreads();  // B2(k)
+            __syncthreads();  // end of interval k
         }
 #pragma unroll
         for (int r = 0; r < 2; ++r) sDD[qi[r] * kWave + ci[r]] = dDacc[r];
@@ -494,13 +507,23 @@ __global__ void __launch_bounds__((NW + 4) * kWave)
                 }
             }
         }
-        __syncthreads();  // B1(k): the reducers are done with the partials of tile k-1
+        // The partial sums go to single-buffered LDS tiles.  The reducers read tile k-1 at the
+        // start of this interval and publish that in sConsumed; by the end of the sweep that
+        // has long happened, so this wait normally falls through (bounded: a wave never
+        // spins forever).
+        if (k >= 1) {
+            int spins = 0;
+            while ((__hip_atomic_load(sConsumed, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP) < k - 1 ||
+                    __hip_atomic_load(sConsumed + 1, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP) < k - 1) &&
+                   ++spins < (1 << 20))
+                __builtin_amdgcn_s_sleep(1);
+        }
 #pragma unroll
         for (int q = 0; q < NQ; ++q) {
             tile_st(sP1 + w * kTileF, lane, q, gBv[4 * q], gBv[4 * q + 1], gBv[4 * q + 2], gBv[4 * q + 3]);
             tile_st(sP2 + w * kTileF, lane, q, ddv[4 * q], ddv[4 * q + 1], ddv[4 * q + 2], ddv[4 * q + 3]);
         }
-        __syncthreads();  // B2(k)
+        __syncthreads();  // end of interval k: partial sums and dB/dC sums of tile k are visible
     };
 
     float dlA[kTile], uuA[kTile], dlB[kTile], uuB[kTile];
