@@ -32,7 +32,7 @@ WORKLOADS = {
 # HBM bytes per launch of the backward entry point measured with rocprofv3 --pmc
 # (FETCH_SIZE + WRITE_SIZE, scaled by a copy kernel of known size); filled from the
 # summaries under profiles/.  None = not measured for that workload.
-MEASURED_TRAFFIC_BYTES = {}
+MEASURED_TRAFFIC_BYTES = {"c2": 1.2526e9}
 
 
 def algorithmic_bytes(B, L, ED, N, s):
