@@ -49,10 +49,19 @@ __device__ __forceinline__ void store_from_float(void* p, int64_t i, float v) {
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
 __device__ __forceinline__ float softplus_f(float v) {
-    // log(1 + e^v); linear above 20 like torch.nn.functional.softplus
-    return v > 20.0f ? v : log1pf(__expf(v));
+    // log(1 + e^v) = max(v, 0) + log1p(e^-|v|), free of branches on the hardware exp2 / log2
+    // units (a library log1p is ~110 instructions and a branch).  log1p(e), 0 < e <= 1: the
+    // cubic series below 2^-6 (truncation < 1e-6 relative), log2(1 + e) above (the rounding
+    // of 1 + e costs < 4e-6 relative).  Above v = 20 the second term vanishes in fp32, which is
+    // torch.nn.functional.softplus' linear branch.
+    const float e = fast_exp2(-fabsf(v) * kLog2e);
+    const float series = e * __builtin_fmaf(e, __builtin_fmaf(e, 0.33333334f, -0.5f), 1.0f);
+    const float lg = __builtin_amdgcn_logf(1.0f + e) * kLn2;
+    return fmaxf(v, 0.0f) + (e < 0.015625f ? series : lg);
 }
-__device__ __forceinline__ float sigmoid_f(float v) { return 1.0f / (1.0f + __expf(-v)); }
+__device__ __forceinline__ float sigmoid_f(float v) {
+    return __builtin_amdgcn_rcpf(1.0f + fast_exp2(-v * kLog2e));
+}
 
 __device__ __forceinline__ int wave_id() {
     // threadIdx.x / 64, told to the compiler as wave-uniform
@@ -82,6 +91,11 @@ __device__ __forceinline__ void scalar_load(const float* src, float (&dst)[COUNT
     }
 }
 
+// one float through the scalar cache (used to pull a 64-byte line into that cache)
+__device__ __forceinline__ float scalar_touch(const float* src) {
+    return *reinterpret_cast<const __attribute__((address_space(4))) float*>(reinterpret_cast<uintptr_t>(src));
+}
+
 inline int check_launch() { return hipGetLastError() == hipSuccess ? MPA_OK : MPA_ERR_LAUNCH; }
 
 inline bool aligned_to(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
@@ -96,7 +110,7 @@ int validate_shape(const mpa_sscan_shape* s);
 // B and C repacked as float32 for scalar loads (see pack_bc_kernel in sscan_fwd.hip)
 size_t bcpack_floats(const mpa_sscan_shape* s);
 int launch_pack_bc(const mpa_sscan_shape* s, const void* B, const void* C, float* out, int ns,
-                   hipStream_t st);
+                   int steps_per_subtile, hipStream_t st);
 
 // Kernels may use more LDS than the 64 KB a static __shared__ array can hold (gfx950 has
 // 160 KB per CU), so they take dynamic LDS; the limit is raised once per kernel.

@@ -522,7 +522,7 @@ extern "C" int mpa_sscan_bwd(const mpa_sscan_shape* s, const void* x, const void
         // fast path: B and C repacked as float32 for scalar loads, then the scan / loader /
         // reducer kernel
         float* pack = wsf + ws.offPack;
-        rc = launch_pack_bc(s, B, C, pack, ns, st);
+        rc = launch_pack_bc(s, B, C, pack, ns, ns >= 16 ? 1 : 16 / ns /* BcPack<NS>::kSS */, st);
         if (rc == MPA_OK) rc = launch_bwd_fast(p, pack, ns, nw, s->io_dtype, st);
     } else if (s->io_dtype == MPA_F32)
         rc = z ? dispatch_bwd<float, true>(p, ns, nw, st) : dispatch_bwd<float, false>(p, ns, nw, st);

@@ -79,10 +79,23 @@ __global__ void __launch_bounds__(256) pack_bc_kernel(const void* Bm, const void
     out[b * per_b + i] = v;
 }
 
+// Packed B/C of the forward kernel: sub-tiles of 16 floats (32 at 16 states per lane, 64 at
+// 32), and as many of them resident in scalar registers as 64 registers hold.  A scalar load
+// that hits L2 takes 200+ clocks (500+ on a miss) while a scan step takes ~25, so a sub-tile is
+// requested three sub-tiles before its first use.
+template <int NS>
+struct FwdPack {
+    static constexpr int kSS = NS >= 8 ? 1 : 8 / NS;       // steps per sub-tile
+    static constexpr int kSub = 2 * kSS * NS;              // floats per sub-tile
+    static constexpr int kRing = kSub <= 16 ? 4 : 2;       // resident sub-tiles
+};
+
 constexpr int kCP = kTile + 4;  // pitch (floats) of a [channel][step] LDS tile: rows stay
                                 // 16-byte aligned and 16-byte accesses of 16 lanes hit 64
                                 // distinct banks
-constexpr int kService = 4;     // service waves per workgroup (256 items of 4 steps per tile)
+constexpr int kLoaders = 4;     // loader waves per workgroup (one item of (channel, 4 steps) per thread)
+constexpr int kReducers = 4;    // reducer waves per workgroup (one item per thread)
+constexpr int kService = kLoaders + kReducers;
 
 template <int NS, int NW>
 struct FwdLds {
@@ -95,7 +108,7 @@ struct FwdLds {
 template <typename IO, int NS, int NW, bool HAS_Z>
 __global__ void __launch_bounds__((NW + kService) * kWave) sscan_fwd_kernel(const FwdParams p) {
     constexpr int NQ = kTile / 4;  // step groups (of 4) per tile
-    static_assert(kService * kWave == kWave * NQ, "one service thread per (channel, step group)");
+    static_assert(kLoaders == NQ && kReducers == NQ, "a tile has 64 * NQ items of (channel, 4 steps)");
 
     extern __shared__ float4 smem4[];
     typedef float CTile[kWave][kCP];  // [channel][step]
@@ -114,138 +127,173 @@ __global__ void __launch_bounds__((NW + kService) * kWave) sscan_fwd_kernel(cons
 
     if (w >= NW) {
         // =============================== service waves ===============================
-        // Two loader waves and two reducer waves, two items of (channel, 4 steps) per thread.
+        // Four loader waves and four reducer waves, one item of (channel, 4 steps) per thread.
         // The roles are split across waves because loads and stores share one in-order
         // counter per wave: a wave that stores y would wait for those stores to drain every
-        // time it waits for its next input tile.
-        const int sw = w - NW;                       // 0,1: loaders   2,3: reducers
+        // time it waits for its next input tile.  A lone wave issues an instruction only every
+        // 6-10 clocks and pays tens of clocks for every branch, so the per-tile code of these
+        // waves is kept short (offsets precomputed, one uniform branch for the ragged edge)
+        // and spread over four waves per role.
+        const int sw = w - NW;                       // 0..3: loaders   4..7: reducers
         const int cmax = min(kWave, p.ED - d0) - 1;  // last valid channel of the group
-        if (sw < 2) {
+        const int item = (sw & 3) * kWave + lane;    // 0 .. 255
+        if (sw < kLoaders) {
             // ------------------------------- loaders -------------------------------
-            int ci[2], qi[2];
-            bool ci_ok[2];
-            uint32_t cx[2], cd[2];
-            float Dv[2], bias[2];
-#pragma unroll
-            for (int r = 0; r < 2; ++r) {
-                const int item = sw * kWave + lane + r * 2 * kWave;  // 0 .. 255
-                ci[r] = p.in_tmajor ? item / NQ : item % kWave;
-                qi[r] = p.in_tmajor ? item % NQ : item / kWave;
-                ci_ok[r] = ci[r] <= cmax;
-                const int cic = min(ci[r], cmax);
-                cx[r] = (uint32_t)cic * (uint32_t)p.u_sd;
-                cd[r] = (uint32_t)cic * (uint32_t)p.d_sd;
-                Dv[r] = p.D[d0 + cic];
-                bias[r] = p.dbias ? p.dbias[d0 + cic] : 0.0f;
-            }
+            const int ci = p.in_tmajor ? item / NQ : item % kWave;
+            const int qi = p.in_tmajor ? item % NQ : item / kWave;
+            const bool ci_ok = ci <= cmax;
+            const int cic = min(ci, cmax);
+            const float Dv = p.D[d0 + cic];
+            const float bias = p.dbias ? p.dbias[d0 + cic] : 0.0f;
             // wave-uniform tile origins (scalar registers) + per-thread 32-bit element
-            // offsets: one global_load per element, no 64-bit address arithmetic in the loop
+            // offsets that do not change from tile to tile: one global_load per element and no
+            // address arithmetic in the loop
             const IO* const xg = static_cast<const IO*>(p.x) + (b * p.u_sb + (int64_t)d0 * p.u_sd);
             const IO* const dg = static_cast<const IO*>(p.delta) + (b * p.d_sb + (int64_t)d0 * p.d_sd);
             const IO* const zg = static_cast<const IO*>(p.z) + (b * p.u_sb + (int64_t)d0 * p.u_sd);
+            uint32_t offx[4], offd[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                offx[j] = (uint32_t)(4 * qi + j) * (uint32_t)p.u_sl + (uint32_t)cic * (uint32_t)p.u_sd;
+                offd[j] = (uint32_t)(4 * qi + j) * (uint32_t)p.d_sl + (uint32_t)cic * (uint32_t)p.d_sd;
+            }
+            const bool group_full = cmax == kWave - 1;
 
-            IO rx[2][4], rd[2][4], rz[2][4];
-            auto load_tile = [&](int k) {
-                // steps beyond the sequence end are clamped to the last one: the loads stay in
-                // bounds and free of branches (a branch here would force a wait on the data)
-                const int tmax = min(kTile, p.L - k * kTile) - 1;
+            // Raw values of three tiles in flight: HBM latency under load is longer than one
+            // tile interval, so a tile is requested five intervals before the scan waves use
+            // it and staged (converted, published in LDS) three intervals after the request.
+            // The scan waves fetch packed B/C through the scalar cache.  All workgroups of a
+            // batch row walk the sequence in step, so without help every one of those scalar
+            // loads would wait for the same trip to memory; each loader thread therefore
+            // touches 16 bytes of the pack five tiles ahead, which brings the lines into L2.
+            constexpr int kPackVec = 2 * kTile * NS * NW / 4;  // float4 per tile of the pack
+            const float4* const warm =
+                reinterpret_cast<const float4*>(p.bcpack) + (int64_t)b * ntiles * kPackVec + min(item, kPackVec - 1);
+            struct Raw { IO x[4], d[4], z[4]; float4 warm; };
+            auto load_tile = [&](int kk, Raw& raw) {
+                // tiles and steps beyond the sequence end are clamped to the last one, so the
+                // loads stay in bounds; only the offsets depend on the (uniform) branch, the
+                // loads themselves are unconditional (a branch around them would force a wait
+                // on their data)
+                const int k = min(kk, ntiles - 1);
                 const IO* xk = xg + (int64_t)k * kTile * p.u_sl;
                 const IO* dk = dg + (int64_t)k * kTile * p.d_sl;
                 const IO* zk = zg + (int64_t)k * kTile * p.u_sl;
+                uint32_t ox[4], od[4];
 #pragma unroll
-                for (int r = 0; r < 2; ++r) {
+                for (int j = 0; j < 4; ++j) {
+                    ox[j] = offx[j];
+                    od[j] = offd[j];
+                }
+                if ((k + 1) * kTile > p.L) {
+                    const int tmax = p.L - k * kTile - 1;
 #pragma unroll
                     for (int j = 0; j < 4; ++j) {
-                        const uint32_t tc = (uint32_t)min(4 * qi[r] + j, tmax);
-                        rx[r][j] = xk[tc * (uint32_t)p.u_sl + cx[r]];
-                        rd[r][j] = dk[tc * (uint32_t)p.d_sl + cd[r]];
-                        if (has_z) rz[r][j] = zk[tc * (uint32_t)p.u_sl + cx[r]];
+                        const uint32_t tc = (uint32_t)min(4 * qi + j, tmax);
+                        ox[j] = tc * (uint32_t)p.u_sl + (uint32_t)cic * (uint32_t)p.u_sd;
+                        od[j] = tc * (uint32_t)p.d_sl + (uint32_t)cic * (uint32_t)p.d_sd;
                     }
                 }
-            };
-            auto stage_tile = [&](int k) {
 #pragma unroll
-                for (int r = 0; r < 2; ++r) {
-                    const int t0 = k * kTile + 4 * qi[r];
-                    float dl[4], uu[4], dx[4], gg[4];
+                for (int j = 0; j < 4; ++j) {
+                    raw.x[j] = xk[ox[j]];
+                    raw.d[j] = dk[od[j]];
+                    if (has_z) raw.z[j] = zk[ox[j]];
+                }
+                raw.warm = warm[(int64_t)k * kPackVec];
+            };
+            auto stage_tile = [&](int k, const Raw& raw) {
+                asm volatile("" ::"v"(raw.warm.x), "v"(raw.warm.w));  // keeps the touch alive
+                float xv[4], dv[4], gg[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    xv[j] = to_float(raw.x[j]);
+                    dv[j] = to_float(raw.d[j]);
+                }
+                if (p.softplus) {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) dv[j] = softplus_f(dv[j] + bias);
+                }
+                if (!group_full || (k + 1) * kTile > p.L) {
+                    // ragged edge: delta = 0, u = 0 keeps the state of padded steps/channels
+                    const int t0 = k * kTile + 4 * qi;
 #pragma unroll
                     for (int j = 0; j < 4; ++j) {
-                        const bool ok = ci_ok[r] && t0 + j < p.L;
-                        const float xv = ok ? to_float(rx[r][j]) : 0.0f;
-                        float dv = to_float(rd[r][j]);
-                        if (p.softplus) dv = softplus_f(dv + bias[r]);
-                        dv = ok ? dv : 0.0f;  // padding: delta = 0, u = 0 keeps the state
-                        dl[j] = dv;
-                        uu[j] = dv * xv;
-                        dx[j] = Dv[r] * xv;
-                        gg[j] = 0.0f;
-                        if (has_z) {
-                            const float zv = to_float(rz[r][j]);
-                            gg[j] = zv * sigmoid_f(zv);
-                        }
+                        const bool ok = ci_ok && t0 + j < p.L;
+                        xv[j] = ok ? xv[j] : 0.0f;
+                        dv[j] = ok ? dv[j] : 0.0f;
                     }
-                    const int c = ci[r], q4 = 4 * qi[r];
-                    *reinterpret_cast<float4*>(&sDl[k & 1][c][q4]) = make_float4(dl[0], dl[1], dl[2], dl[3]);
-                    *reinterpret_cast<float4*>(&sU[k & 1][c][q4]) = make_float4(uu[0], uu[1], uu[2], uu[3]);
-                    *reinterpret_cast<float4*>(&sDx[k & 3][c][q4]) = make_float4(dx[0], dx[1], dx[2], dx[3]);
-                    if (has_z)
-                        *reinterpret_cast<float4*>(&sG[k & 3][c][q4]) =
-                            make_float4(gg[0], gg[1], gg[2], gg[3]);
+                }
+                const int q4 = 4 * qi;
+                *reinterpret_cast<float4*>(&sDl[k & 1][ci][q4]) = make_float4(dv[0], dv[1], dv[2], dv[3]);
+                *reinterpret_cast<float4*>(&sU[k & 1][ci][q4]) =
+                    make_float4(dv[0] * xv[0], dv[1] * xv[1], dv[2] * xv[2], dv[3] * xv[3]);
+                *reinterpret_cast<float4*>(&sDx[k & 3][ci][q4]) =
+                    make_float4(Dv * xv[0], Dv * xv[1], Dv * xv[2], Dv * xv[3]);
+                if (has_z) {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        const float zv = to_float(raw.z[j]);
+                        gg[j] = zv * sigmoid_f(zv);
+                    }
+                    *reinterpret_cast<float4*>(&sG[k & 3][ci][q4]) = make_float4(gg[0], gg[1], gg[2], gg[3]);
                 }
             };
-            // the loaders run two tiles ahead of the scan waves
-            load_tile(0);
-            stage_tile(0);
-            if (ntiles > 1) {
-                load_tile(1);
-                stage_tile(1);
-            }
-            if (ntiles > 2) load_tile(2);
+            // tile j travels in register set j % 3; staging runs two tiles ahead of the scan
+            Raw ra, rb, rc;
+            load_tile(0, ra);
+            load_tile(1, rb);
+            load_tile(2, rc);
+            stage_tile(0, ra);
+            load_tile(3, ra);
+            if (ntiles > 1) stage_tile(1, rb);
+            load_tile(4, rb);
             __syncthreads();  // tiles 0 and 1 are published
             __syncthreads();  // the scan waves hold tile 0 in registers: its buffer is free
-            for (int k = 0; k < ntiles; ++k) {
-                if (k + 2 < ntiles) stage_tile(k + 2);
-                if (k + 3 < ntiles) load_tile(k + 3);
+            for (int k = 0; k < ntiles; k += 3) {
+                if (k + 2 < ntiles) stage_tile(k + 2, rc);
+                load_tile(k + 5, rc);
+                __syncthreads();
+                if (k + 1 >= ntiles) break;
+                if (k + 3 < ntiles) stage_tile(k + 3, ra);
+                load_tile(k + 6, ra);
+                __syncthreads();
+                if (k + 2 >= ntiles) break;
+                if (k + 4 < ntiles) stage_tile(k + 4, rb);
+                load_tile(k + 7, rb);
                 __syncthreads();
             }
         } else {
             // ------------------------------- reducers -------------------------------
-            int co[2], qo[2];
-            bool co_ok[2];
-            uint32_t cy[2];
+            const int co = p.out_tmajor ? item / NQ : item % kWave;
+            const int qo = p.out_tmajor ? item % NQ : item / kWave;
+            const bool co_ok = co <= cmax;
+            const int q4 = 4 * qo;
+            uint32_t offy[4];
 #pragma unroll
-            for (int r = 0; r < 2; ++r) {
-                const int item = (sw - 2) * kWave + lane + r * 2 * kWave;
-                co[r] = p.out_tmajor ? item / NQ : item % kWave;
-                qo[r] = p.out_tmajor ? item % NQ : item / kWave;
-                co_ok[r] = co[r] <= cmax;
-                cy[r] = (uint32_t)min(co[r], cmax) * (uint32_t)p.y_sd;
-            }
+            for (int j = 0; j < 4; ++j)
+                offy[j] = (uint32_t)(q4 + j) * (uint32_t)p.y_sl + (uint32_t)min(co, cmax) * (uint32_t)p.y_sd;
             IO* const yg = static_cast<IO*>(p.y) + (b * p.y_sb + (int64_t)d0 * p.y_sd);
             auto reduce_store = [&](int k) {
                 IO* yk = yg + (int64_t)k * kTile * p.y_sl;
+                float4 s = *reinterpret_cast<const float4*>(&sDx[k & 3][co][q4]);
 #pragma unroll
-                for (int r = 0; r < 2; ++r) {
-                    const int c = co[r], q4 = 4 * qo[r];
-                    float4 s = *reinterpret_cast<const float4*>(&sDx[k & 3][c][q4]);
+                for (int ww = 0; ww < NW; ++ww) {
+                    const float4 v = *reinterpret_cast<const float4*>(&sY[(k & 1) * NW + ww][co][q4]);
+                    s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
+                }
+                if (has_z) {
+                    const float4 g = *reinterpret_cast<const float4*>(&sG[k & 3][co][q4]);
+                    s.x *= g.x; s.y *= g.y; s.z *= g.z; s.w *= g.w;
+                }
+                const float sv[4] = {s.x, s.y, s.z, s.w};
+                const int t0 = k * kTile + q4;
+                if (co_ok && t0 + 3 < p.L) {
 #pragma unroll
-                    for (int ww = 0; ww < NW; ++ww) {
-                        const float4 v =
-                            *reinterpret_cast<const float4*>(&sY[(k & 1) * NW + ww][c][q4]);
-                        s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
-                    }
-                    if (has_z) {
-                        const float4 g = *reinterpret_cast<const float4*>(&sG[k & 3][c][q4]);
-                        s.x *= g.x; s.y *= g.y; s.z *= g.z; s.w *= g.w;
-                    }
-                    const float sv[4] = {s.x, s.y, s.z, s.w};
-                    const int t0 = k * kTile + q4;
-                    if (co_ok[r]) {
-#pragma unroll
-                        for (int j = 0; j < 4; ++j)
-                            if (t0 + j < p.L)
-                                yk[(uint32_t)(q4 + j) * (uint32_t)p.y_sl + cy[r]] = from_float<IO>(sv[j]);
-                    }
+                    for (int j = 0; j < 4; ++j) yk[offy[j]] = from_float<IO>(sv[j]);
+                } else if (co_ok) {
+                    for (int j = 0; j < 4; ++j)
+                        if (t0 + j < p.L) yk[offy[j]] = from_float<IO>(sv[j]);
                 }
             };
             // the reducers run one tile behind the scan waves
@@ -275,9 +323,11 @@ __global__ void __launch_bounds__((NW + kService) * kWave) sscan_fwd_kernel(cons
         h[i] = ok ? hv : 0.0f;
     }
     // packed B/C of this (batch, wave): sub-tile j of tile k at + (k*NW*NSUB + j) * kSub
-    constexpr int kSS = BcPack<NS>::kSS;        // steps per sub-tile
-    constexpr int NSUB = kTile / kSS;           // sub-tiles per tile
-    constexpr int kSub = 2 * kSS * NS;          // floats per sub-tile: B then C
+    constexpr int kSS = FwdPack<NS>::kSS;        // steps per sub-tile
+    constexpr int NSUB = kTile / kSS;            // sub-tiles per tile
+    constexpr int kSub = 2 * kSS * NS;           // floats per sub-tile: B then C
+    constexpr int kRing = FwdPack<NS>::kRing;    // sub-tiles resident in scalar registers
+    static_assert(NSUB % kRing == 0, "a sub-tile always lands in the same ring slot");
     const float* bc = p.bcpack + ((int64_t)b * ntiles * NW + w) * (NSUB * kSub);
     const int64_t bc_tile = (int64_t)NW * NSUB * kSub;
 
@@ -297,7 +347,7 @@ __global__ void __launch_bounds__((NW + kService) * kWave) sscan_fwd_kernel(cons
     // ahead through the scalar cache, so no load latency sits between two dependent steps.
     // Padded steps were staged as delta = 0, u = 0 (a = 2^0 = 1: h unchanged) and padded
     // states have A2 = 0, B = C = 0, so there is no tail handling.
-    float bcb[2][kSub];  // wave-uniform: live in SGPRs; sub-tile j of a tile uses bcb[j & 1]
+    float bcb[kRing][kSub];  // wave-uniform: live in SGPRs; sub-tile j of a tile uses slot j % kRing
     auto tile_compute = [&](int k, const float (&dl)[kTile], const float (&uu)[kTile],
                             float (&dl_next)[kTile], float (&uu_next)[kTile]) {
         const float* bck = bc + (int64_t)k * bc_tile;
@@ -305,7 +355,7 @@ __global__ void __launch_bounds__((NW + kService) * kWave) sscan_fwd_kernel(cons
 #pragma unroll
         for (int tt = 0; tt < kTile; ++tt) {
             const int sub = tt / kSS, ts = tt % kSS;
-            const float(&cur)[kSub] = bcb[sub & 1];
+            const float(&cur)[kSub] = bcb[sub % kRing];
             float sum = 0.0f;
 #pragma unroll
             for (int i = 0; i < NS; ++i) {
@@ -326,10 +376,12 @@ __global__ void __launch_bounds__((NW + kService) * kWave) sscan_fwd_kernel(cons
                 // (after the last tile the prefetches re-read valid memory and are ignored:
                 // no branch, so that the compiler cannot sink the arithmetic below them)
                 __builtin_amdgcn_sched_barrier(0);
-                if (sub + 1 < NSUB)
-                    scalar_load<kSub>(bck + (sub + 1) * kSub, bcb[(sub + 1) & 1]);
+                constexpr int kAhead = kRing - 1;  // the slot of the sub-tile just finished is free
+                if (sub + kAhead < NSUB)
+                    scalar_load<kSub>(bck + (sub + kAhead) * kSub, bcb[(sub + kAhead) % kRing]);
                 else
-                    scalar_load<kSub>(bc + (int64_t)min(k + 1, ntiles - 1) * bc_tile, bcb[0]);
+                    scalar_load<kSub>(bc + (int64_t)min(k + 1, ntiles - 1) * bc_tile + (sub + kAhead - NSUB) * kSub,
+                                      bcb[(sub + kAhead) % kRing]);
                 if (sub == 0) read_tile(k + 1, dl_next, uu_next);
                 __builtin_amdgcn_sched_barrier(0);
             }
@@ -344,7 +396,8 @@ __global__ void __launch_bounds__((NW + kService) * kWave) sscan_fwd_kernel(cons
     };
 
     float dlA[kTile], uuA[kTile], dlB[kTile], uuB[kTile];
-    scalar_load<kSub>(bc, bcb[0]);
+#pragma unroll
+    for (int j = 0; j < kRing - 1; ++j) scalar_load<kSub>(bc + j * kSub, bcb[j]);
     __syncthreads();
     read_tile(0, dlA, uuA);
     __syncthreads();
@@ -443,11 +496,10 @@ size_t bcpack_floats(const mpa_sscan_shape* s) {
 }
 
 int launch_pack_bc(const mpa_sscan_shape* s, const void* B, const void* C, float* out, int ns,
-                   hipStream_t st) {
+                   int kss, hipStream_t st) {
     const int np = padded_states(s->dstate);
     const int nchunks = (int)((s->seqlen + kTile - 1) / kTile);
     const int64_t per_b = (int64_t)nchunks * 2 * kTile * np;
-    const int kss = ns >= 16 ? 1 : 16 / ns;  // BcPack<NS>::kSS
     dim3 grid((unsigned)((per_b + 255) / 256), (unsigned)s->batch);
     if (s->io_dtype == MPA_F32)
         hipLaunchKernelGGL(pack_bc_kernel<float>, grid, dim3(256), 0, st, B, C, out, (int)s->seqlen,
@@ -495,7 +547,7 @@ extern "C" int mpa_sscan_fwd(const mpa_sscan_shape* s, const void* x, const void
     if (ns < 0) return MPA_ERR_BAD_SHAPE;
     const int nw = np / ns;
     hipStream_t st = static_cast<hipStream_t>(stream);
-    rc = launch_pack_bc(s, B, C, static_cast<float*>(workspace), ns, st);
+    rc = launch_pack_bc(s, B, C, static_cast<float*>(workspace), ns, ns >= 8 ? 1 : 8 / ns /* FwdPack<NS>::kSS */, st);
     if (rc != MPA_OK) return rc;
 
     FwdParams p{};
