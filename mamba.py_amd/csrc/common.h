@@ -91,9 +91,17 @@ __device__ __forceinline__ void scalar_load(const float* src, float (&dst)[COUNT
     }
 }
 
-// one float through the scalar cache (used to pull a 64-byte line into that cache)
-__device__ __forceinline__ float scalar_touch(const float* src) {
-    return *reinterpret_cast<const __attribute__((address_space(4))) float*>(reinterpret_cast<uintptr_t>(src));
+// acc + v[lane T of the reader's row of 16 lanes] * x in ONE instruction: the DPP control
+// row_newbcast broadcasts lane T of every row to the 16 lanes of that row on the way into the
+// multiplier.  A register that holds 16 wave-uniform values (one per lane of a row, the same
+// in all four rows) thus feeds 16 different FMAs without a move or a scalar register.
+template <int T>
+__device__ __forceinline__ float fmac_bcast(float acc, float v, float x) {
+    static_assert(T >= 0 && T < 16, "lane inside a row");
+    asm("v_fmac_f32_dpp %0, %1, %2 row_newbcast:%3 row_mask:0xf bank_mask:0xf"
+        : "+v"(acc)
+        : "v"(v), "v"(x), "n"(T));
+    return acc;
 }
 
 inline int check_launch() { return hipGetLastError() == hipSuccess ? MPA_OK : MPA_ERR_LAUNCH; }

@@ -33,7 +33,10 @@ struct FwdParams {
     const float* D;
     const float* dbias;
     const float* h0;
-    const float* bcpack;  // packed B/C, see pack_bc_kernel
+    const float* bcpack;  // packed B/C, see pack_bc_kernel (only at 16 or more states per lane)
+    const void* Bm;
+    const void* C;
+    int64_t bc_sb, bc_sl;
     void* y;
     float* ckpt;
     float* hlast;
@@ -97,13 +100,46 @@ constexpr int kLoaders = 4;     // loader waves per workgroup (one item of (chan
 constexpr int kReducers = 4;    // reducer waves per workgroup (one item per thread)
 constexpr int kService = kLoaders + kReducers;
 
+// Up to 8 states per lane B and C reach the scan waves through LDS and a register per state
+// whose 16 lanes of a row hold the 16 steps of a tile (see fmac_bcast); above that the register
+// and LDS cost is too high and they come packed through the scalar cache (FwdPack).
+template <int NS>
+constexpr bool kBcastBC = NS <= 8;
+
 template <int NS, int NW>
 struct FwdLds {
     // delta, u double-buffered (written two tiles ahead of use, read one tile ahead); D*x and
     // the gate in four buffers (written two tiles ahead, read one tile behind); readout
-    // partials double-buffered per scan wave
-    static constexpr size_t floats = (size_t)(2 * 2 + 2 * 4 + 2 * NW) * kWave * kCP;
+    // partials double-buffered per scan wave; B/C tiles [2][B|C][state][step] double-buffered
+    static constexpr size_t tiles = (size_t)(2 * 2 + 2 * 4 + 2 * NW) * kWave * kCP;
+    static constexpr size_t floats = tiles + (kBcastBC<NS> ? 2 * 2 * NS * NW * kTile : 0);
 };
+
+// One scan step / one group of four steps on the broadcast path: B and C of step TT come out of
+// lane TT of the registers vb[i] / vc[i] inside the FMA (fmac_bcast).
+template <int TT, int NS>
+__device__ __forceinline__ float scan_step_bcast(float dlv, float uuv, const float (&A2)[NS], float (&h)[NS],
+                                                 const float (&vb)[NS], const float (&vc)[NS]) {
+    float sum = 0.0f;
+#pragma unroll
+    for (int i = 0; i < NS; ++i) {
+        const float a = fast_exp2(dlv * A2[i]);
+        h[i] = fmac_bcast<TT>(a * h[i], vb[i], uuv);
+        sum = fmac_bcast<TT>(sum, vc[i], h[i]);
+    }
+    return sum;
+}
+template <int Q, int NS>
+__device__ __forceinline__ float4 scan_group_bcast(const float (&dl)[kTile], const float (&uu)[kTile],
+                                                   const float (&A2)[NS], float (&h)[NS],
+                                                   const float (&vb)[NS], const float (&vc)[NS]) {
+    float4 y;
+    y.x = scan_step_bcast<4 * Q + 0, NS>(dl[4 * Q + 0], uu[4 * Q + 0], A2, h, vb, vc);
+    y.y = scan_step_bcast<4 * Q + 1, NS>(dl[4 * Q + 1], uu[4 * Q + 1], A2, h, vb, vc);
+    y.z = scan_step_bcast<4 * Q + 2, NS>(dl[4 * Q + 2], uu[4 * Q + 2], A2, h, vb, vc);
+    y.w = scan_step_bcast<4 * Q + 3, NS>(dl[4 * Q + 3], uu[4 * Q + 3], A2, h, vb, vc);
+    return y;
+}
 
 template <typename IO, int NS, int NW, bool HAS_Z>
 __global__ void __launch_bounds__((NW + kService) * kWave) sscan_fwd_kernel(const FwdParams p) {
@@ -117,6 +153,9 @@ __global__ void __launch_bounds__((NW + kService) * kWave) sscan_fwd_kernel(cons
     CTile* sDx = sU + 2;                           // [4] D*x
     CTile* sG = sDx + 4;                           // [4] gate silu(z) (only with z)
     CTile* sY = sG + 4;                            // [2][NW]
+    float* const sBC = reinterpret_cast<float*>(sY + 2 * NW);  // [2][B|C][NP states][kTile steps]
+    constexpr int NP = NS * NW;
+    constexpr bool kBcast = kBcastBC<NS>;
 
     const int lane = threadIdx.x & (kWave - 1);
     const int w = wave_id();
@@ -158,6 +197,20 @@ __global__ void __launch_bounds__((NW + kService) * kWave) sscan_fwd_kernel(cons
                 offd[j] = (uint32_t)(4 * qi + j) * (uint32_t)p.d_sl + (uint32_t)cic * (uint32_t)p.d_sd;
             }
             const bool group_full = cmax == kWave - 1;
+            // B/C of a tile: kTile * NP elements each, kBcPer per loader thread, step fastest
+            constexpr int kBcPer = kBcast ? NP * kTile / (kLoaders * kWave) : 0;
+            static_assert(!kBcast || NP * kTile % (kLoaders * kWave) == 0, "whole elements per thread");
+            const IO* const Bg = static_cast<const IO*>(p.Bm) + b * p.bc_sb;
+            const IO* const Cg = static_cast<const IO*>(p.C) + b * p.bc_sb;
+            int bct[kBcPer > 0 ? kBcPer : 1], bcn[kBcPer > 0 ? kBcPer : 1];
+            uint32_t offbc[kBcPer > 0 ? kBcPer : 1];
+#pragma unroll
+            for (int r = 0; r < kBcPer; ++r) {
+                const int e = item + r * (kLoaders * kWave);
+                bct[r] = e % kTile;
+                bcn[r] = e / kTile;
+                offbc[r] = (uint32_t)bct[r] * (uint32_t)p.bc_sl + (uint32_t)min(bcn[r], p.N - 1);
+            }
 
             // Raw values of three tiles in flight: HBM latency under load is longer than one
             // tile interval, so a tile is requested five intervals before the scan waves use
@@ -168,8 +221,9 @@ __global__ void __launch_bounds__((NW + kService) * kWave) sscan_fwd_kernel(cons
             // touches 16 bytes of the pack five tiles ahead, which brings the lines into L2.
             constexpr int kPackVec = 2 * kTile * NS * NW / 4;  // float4 per tile of the pack
             const float4* const warm =
-                reinterpret_cast<const float4*>(p.bcpack) + (int64_t)b * ntiles * kPackVec + min(item, kPackVec - 1);
-            struct Raw { IO x[4], d[4], z[4]; float4 warm; };
+                kBcast ? nullptr
+                       : reinterpret_cast<const float4*>(p.bcpack) + (int64_t)b * ntiles * kPackVec + min(item, kPackVec - 1);
+            struct Raw { IO x[4], d[4], z[4], b[kBcPer > 0 ? kBcPer : 1], c[kBcPer > 0 ? kBcPer : 1]; float4 warm; };
             auto load_tile = [&](int kk, Raw& raw) {
                 // tiles and steps beyond the sequence end are clamped to the last one, so the
                 // loads stay in bounds; only the offsets depend on the (uniform) branch, the
@@ -179,12 +233,16 @@ __global__ void __launch_bounds__((NW + kService) * kWave) sscan_fwd_kernel(cons
                 const IO* xk = xg + (int64_t)k * kTile * p.u_sl;
                 const IO* dk = dg + (int64_t)k * kTile * p.d_sl;
                 const IO* zk = zg + (int64_t)k * kTile * p.u_sl;
-                uint32_t ox[4], od[4];
+                const IO* Bk = Bg + (int64_t)k * kTile * p.bc_sl;
+                const IO* Ck = Cg + (int64_t)k * kTile * p.bc_sl;
+                uint32_t ox[4], od[4], ob[kBcPer > 0 ? kBcPer : 1];
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
                     ox[j] = offx[j];
                     od[j] = offd[j];
                 }
+#pragma unroll
+                for (int r = 0; r < kBcPer; ++r) ob[r] = offbc[r];
                 if ((k + 1) * kTile > p.L) {
                     const int tmax = p.L - k * kTile - 1;
 #pragma unroll
@@ -193,6 +251,9 @@ __global__ void __launch_bounds__((NW + kService) * kWave) sscan_fwd_kernel(cons
                         ox[j] = tc * (uint32_t)p.u_sl + (uint32_t)cic * (uint32_t)p.u_sd;
                         od[j] = tc * (uint32_t)p.d_sl + (uint32_t)cic * (uint32_t)p.d_sd;
                     }
+#pragma unroll
+                    for (int r = 0; r < kBcPer; ++r)
+                        ob[r] = (uint32_t)min(bct[r], tmax) * (uint32_t)p.bc_sl + (uint32_t)min(bcn[r], p.N - 1);
                 }
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
@@ -200,10 +261,24 @@ __global__ void __launch_bounds__((NW + kService) * kWave) sscan_fwd_kernel(cons
                     raw.d[j] = dk[od[j]];
                     if (has_z) raw.z[j] = zk[ox[j]];
                 }
-                raw.warm = warm[(int64_t)k * kPackVec];
+#pragma unroll
+                for (int r = 0; r < kBcPer; ++r) {
+                    raw.b[r] = Bk[ob[r]];
+                    raw.c[r] = Ck[ob[r]];
+                }
+                if (!kBcast) raw.warm = warm[(int64_t)k * kPackVec];
             };
             auto stage_tile = [&](int k, const Raw& raw) {
-                asm volatile("" ::"v"(raw.warm.x), "v"(raw.warm.w));  // keeps the touch alive
+                if (!kBcast) asm volatile("" ::"v"(raw.warm.x), "v"(raw.warm.w));  // keeps the touch alive
+#pragma unroll
+                for (int r = 0; r < kBcPer; ++r) {
+                    // states beyond d_state: B = C = 0 (padded steps need no care: u = 0 there
+                    // and their y is never stored)
+                    const bool ok = bcn[r] < p.N;
+                    float* dst = sBC + (k & 1) * (2 * NP * kTile) + bcn[r] * kTile + bct[r];
+                    dst[0] = ok ? to_float(raw.b[r]) : 0.0f;
+                    dst[NP * kTile] = ok ? to_float(raw.c[r]) : 0.0f;
+                }
                 float xv[4], dv[4], gg[4];
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
@@ -322,70 +397,30 @@ __global__ void __launch_bounds__((NW + kService) * kWave) sscan_fwd_kernel(cons
         A2[i] = ok ? av * kLog2e : 0.0f;
         h[i] = ok ? hv : 0.0f;
     }
-    // packed B/C of this (batch, wave): sub-tile j of tile k at + (k*NW*NSUB + j) * kSub
-    constexpr int kSS = FwdPack<NS>::kSS;        // steps per sub-tile
-    constexpr int NSUB = kTile / kSS;            // sub-tiles per tile
-    constexpr int kSub = 2 * kSS * NS;           // floats per sub-tile: B then C
-    constexpr int kRing = FwdPack<NS>::kRing;    // sub-tiles resident in scalar registers
-    static_assert(NSUB % kRing == 0, "a sub-tile always lands in the same ring slot");
-    const float* bc = p.bcpack + ((int64_t)b * ntiles * NW + w) * (NSUB * kSub);
-    const int64_t bc_tile = (int64_t)NW * NSUB * kSub;
-
-    auto read_tile = [&](int k, float (&dl)[kTile], float (&uu)[kTile]) {
+    // registers of one tile: delta and u of the lane's channel and, on the broadcast path, one
+    // register per state for B and for C whose lane t of every row holds step t
+    struct TileRegs {
+        float dl[kTile], uu[kTile];
+        float vb[kBcast ? NS : 1], vc[kBcast ? NS : 1];
+    };
+    auto read_tile = [&](int k, TileRegs& r) {
 #pragma unroll
         for (int q = 0; q < NQ; ++q) {
             const float4 v = *reinterpret_cast<const float4*>(&sDl[k & 1][lane][4 * q]);
             const float4 u4 = *reinterpret_cast<const float4*>(&sU[k & 1][lane][4 * q]);
-            dl[4 * q] = v.x; dl[4 * q + 1] = v.y; dl[4 * q + 2] = v.z; dl[4 * q + 3] = v.w;
-            uu[4 * q] = u4.x; uu[4 * q + 1] = u4.y; uu[4 * q + 2] = u4.z; uu[4 * q + 3] = u4.w;
+            r.dl[4 * q] = v.x; r.dl[4 * q + 1] = v.y; r.dl[4 * q + 2] = v.z; r.dl[4 * q + 3] = v.w;
+            r.uu[4 * q] = u4.x; r.uu[4 * q + 1] = u4.y; r.uu[4 * q + 2] = u4.z; r.uu[4 * q + 3] = u4.w;
         }
-    };
-
-    // Software pipeline of one scan wave.  In interval k (between two barriers) it computes
-    // tile k from registers that were filled during interval k-1, fetches delta/u of tile
-    // k+1 from LDS (published by the service waves two intervals ahead) and B/C one sub-tile
-    // ahead through the scalar cache, so no load latency sits between two dependent steps.
-    // Padded steps were staged as delta = 0, u = 0 (a = 2^0 = 1: h unchanged) and padded
-    // states have A2 = 0, B = C = 0, so there is no tail handling.
-    float bcb[kRing][kSub];  // wave-uniform: live in SGPRs; sub-tile j of a tile uses slot j % kRing
-    auto tile_compute = [&](int k, const float (&dl)[kTile], const float (&uu)[kTile],
-                            float (&dl_next)[kTile], float (&uu_next)[kTile]) {
-        const float* bck = bc + (int64_t)k * bc_tile;
-        float acc[4];
-#pragma unroll
-        for (int tt = 0; tt < kTile; ++tt) {
-            const int sub = tt / kSS, ts = tt % kSS;
-            const float(&cur)[kSub] = bcb[sub % kRing];
-            float sum = 0.0f;
+        if constexpr (kBcast) {
+            const float* bck = sBC + (k & 1) * (2 * NP * kTile) + (w * NS) * kTile + (lane & (kTile - 1));
 #pragma unroll
             for (int i = 0; i < NS; ++i) {
-                const float a = fast_exp2(dl[tt] * A2[i]);
-                h[i] = __builtin_fmaf(uu[tt], cur[ts * NS + i], a * h[i]);
-                sum = __builtin_fmaf(cur[kSS * NS + ts * NS + i], h[i], sum);
-            }
-            acc[tt & 3] = sum;
-            if ((tt & 3) == 3)
-                *reinterpret_cast<float4*>(&sY[(k & 1) * NW + w][lane][tt - 3]) =
-                    make_float4(acc[0], acc[1], acc[2], acc[3]);
-            if (ts == 0) {
-                // Prefetches are issued right AFTER the first step of a sub-tile has consumed
-                // its B/C: scalar loads return out of order and share their counter with LDS,
-                // so the wait that precedes the first use of a sub-tile drains everything in
-                // flight.  Placed here, that wait only ever finds loads issued a whole
-                // sub-tile earlier.
-                // (after the last tile the prefetches re-read valid memory and are ignored:
-                // no branch, so that the compiler cannot sink the arithmetic below them)
-                __builtin_amdgcn_sched_barrier(0);
-                constexpr int kAhead = kRing - 1;  // the slot of the sub-tile just finished is free
-                if (sub + kAhead < NSUB)
-                    scalar_load<kSub>(bck + (sub + kAhead) * kSub, bcb[(sub + kAhead) % kRing]);
-                else
-                    scalar_load<kSub>(bc + (int64_t)min(k + 1, ntiles - 1) * bc_tile + (sub + kAhead - NSUB) * kSub,
-                                      bcb[(sub + kAhead) % kRing]);
-                if (sub == 0) read_tile(k + 1, dl_next, uu_next);
-                __builtin_amdgcn_sched_barrier(0);
+                r.vb[i] = bck[i * kTile];
+                r.vc[i] = bck[NP * kTile + i * kTile];
             }
         }
+    };
+    auto store_ckpt = [&](int k) {
         if (p.ckpt && dvalid && k + 1 < ntiles) {
 #pragma unroll
             for (int i = 0; i < NS; ++i) {
@@ -395,18 +430,96 @@ __global__ void __launch_bounds__((NW + kService) * kWave) sscan_fwd_kernel(cons
         }
     };
 
-    float dlA[kTile], uuA[kTile], dlB[kTile], uuB[kTile];
+    // Software pipeline of one scan wave.  In interval k (between two barriers) it computes
+    // tile k from registers that were filled during interval k-1 and fetches the inputs of
+    // tile k+1 from LDS (published by the loader waves two intervals ahead), so no load
+    // latency sits between two dependent steps.  Padded steps were staged as delta = 0, u = 0
+    // (a = 2^0 = 1: h unchanged) and padded states have A2 = 0, B = C = 0, so there is no tail
+    // handling.
+    TileRegs ra, rb;
+    if constexpr (kBcast) {
+        auto tile_compute = [&](int k, const TileRegs& cur, TileRegs& next) {
+            CTile& yt = sY[(k & 1) * NW + w];
+            *reinterpret_cast<float4*>(&yt[lane][0]) = scan_group_bcast<0, NS>(cur.dl, cur.uu, A2, h, cur.vb, cur.vc);
+            __builtin_amdgcn_sched_barrier(0);
+            read_tile(k + 1, next);
+            __builtin_amdgcn_sched_barrier(0);
+            *reinterpret_cast<float4*>(&yt[lane][4]) = scan_group_bcast<1, NS>(cur.dl, cur.uu, A2, h, cur.vb, cur.vc);
+            *reinterpret_cast<float4*>(&yt[lane][8]) = scan_group_bcast<2, NS>(cur.dl, cur.uu, A2, h, cur.vb, cur.vc);
+            *reinterpret_cast<float4*>(&yt[lane][12]) = scan_group_bcast<3, NS>(cur.dl, cur.uu, A2, h, cur.vb, cur.vc);
+            store_ckpt(k);
+        };
+        __syncthreads();
+        read_tile(0, ra);
+        __syncthreads();
+        for (int k = 0; k < ntiles; k += 2) {
+            tile_compute(k, ra, rb);
+            __syncthreads();
+            if (k + 1 >= ntiles) break;
+            tile_compute(k + 1, rb, ra);
+            __syncthreads();
+        }
+    } else {
+        // packed B/C of this (batch, wave): sub-tile j of tile k at + (k*NW*NSUB + j) * kSub,
+        // fetched through the scalar cache a few sub-tiles ahead of use
+        constexpr int kSS = FwdPack<NS>::kSS;        // steps per sub-tile
+        constexpr int NSUB = kTile / kSS;            // sub-tiles per tile
+        constexpr int kSub = 2 * kSS * NS;           // floats per sub-tile: B then C
+        constexpr int kRing = FwdPack<NS>::kRing;    // sub-tiles resident in scalar registers
+        static_assert(NSUB % kRing == 0, "a sub-tile always lands in the same ring slot");
+        const float* bc = p.bcpack + ((int64_t)b * ntiles * NW + w) * (NSUB * kSub);
+        const int64_t bc_tile = (int64_t)NW * NSUB * kSub;
+        float bcb[kRing][kSub];  // wave-uniform: live in SGPRs; sub-tile j of a tile uses slot j % kRing
+        auto tile_compute = [&](int k, const TileRegs& cur_t, TileRegs& next) {
+            const float* bck = bc + (int64_t)k * bc_tile;
+            float acc[4];
 #pragma unroll
-    for (int j = 0; j < kRing - 1; ++j) scalar_load<kSub>(bc + j * kSub, bcb[j]);
-    __syncthreads();
-    read_tile(0, dlA, uuA);
-    __syncthreads();
-    for (int k = 0; k < ntiles; k += 2) {
-        tile_compute(k, dlA, uuA, dlB, uuB);
+            for (int tt = 0; tt < kTile; ++tt) {
+                const int sub = tt / kSS, ts = tt % kSS;
+                const float(&cur)[kSub] = bcb[sub % kRing];
+                float sum = 0.0f;
+#pragma unroll
+                for (int i = 0; i < NS; ++i) {
+                    const float a = fast_exp2(cur_t.dl[tt] * A2[i]);
+                    h[i] = __builtin_fmaf(cur_t.uu[tt], cur[ts * NS + i], a * h[i]);
+                    sum = __builtin_fmaf(cur[kSS * NS + ts * NS + i], h[i], sum);
+                }
+                acc[tt & 3] = sum;
+                if ((tt & 3) == 3)
+                    *reinterpret_cast<float4*>(&sY[(k & 1) * NW + w][lane][tt - 3]) =
+                        make_float4(acc[0], acc[1], acc[2], acc[3]);
+                if (ts == 0) {
+                    // Prefetches are issued right AFTER the first step of a sub-tile has
+                    // consumed its B/C: scalar loads return out of order and share their
+                    // counter with LDS, so the wait that precedes the first use of a sub-tile
+                    // drains everything in flight.  (After the last tile the prefetches
+                    // re-read valid memory and are ignored: no branch, so that the compiler
+                    // cannot sink the arithmetic below them.)
+                    __builtin_amdgcn_sched_barrier(0);
+                    constexpr int kAhead = kRing - 1;  // the slot of the sub-tile just finished is free
+                    if (sub + kAhead < NSUB)
+                        scalar_load<kSub>(bck + (sub + kAhead) * kSub, bcb[(sub + kAhead) % kRing]);
+                    else
+                        scalar_load<kSub>(bc + (int64_t)min(k + 1, ntiles - 1) * bc_tile + (sub + kAhead - NSUB) * kSub,
+                                          bcb[(sub + kAhead) % kRing]);
+                    if (sub == 0) read_tile(k + 1, next);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
+            store_ckpt(k);
+        };
+#pragma unroll
+        for (int j = 0; j < kRing - 1; ++j) scalar_load<kSub>(bc + j * kSub, bcb[j]);
         __syncthreads();
-        if (k + 1 >= ntiles) break;
-        tile_compute(k + 1, dlB, uuB, dlA, uuA);
+        read_tile(0, ra);
         __syncthreads();
+        for (int k = 0; k < ntiles; k += 2) {
+            tile_compute(k, ra, rb);
+            __syncthreads();
+            if (k + 1 >= ntiles) break;
+            tile_compute(k + 1, rb, ra);
+            __syncthreads();
+        }
     }
 
     if (p.hlast && dvalid) {
@@ -547,12 +660,15 @@ extern "C" int mpa_sscan_fwd(const mpa_sscan_shape* s, const void* x, const void
     if (ns < 0) return MPA_ERR_BAD_SHAPE;
     const int nw = np / ns;
     hipStream_t st = static_cast<hipStream_t>(stream);
-    rc = launch_pack_bc(s, B, C, static_cast<float*>(workspace), ns, ns >= 8 ? 1 : 8 / ns /* FwdPack<NS>::kSS */, st);
-    if (rc != MPA_OK) return rc;
+    if (ns > 8) {  // !kBcastBC<NS>: B/C go through the scalar cache, repacked per scan wave
+        rc = launch_pack_bc(s, B, C, static_cast<float*>(workspace), ns, 1 /* FwdPack<NS>::kSS */, st);
+        if (rc != MPA_OK) return rc;
+    }
 
     FwdParams p{};
     p.x = x; p.delta = delta; p.z = z; p.A = A; p.D = D;
     p.dbias = delta_bias; p.h0 = h0; p.bcpack = static_cast<const float*>(workspace);
+    p.Bm = B; p.C = C; p.bc_sb = s->bc_sb; p.bc_sl = s->bc_sl;
     p.y = y; p.ckpt = h_ckpt; p.hlast = h_last;
     p.batch = (int)s->batch; p.L = (int)s->seqlen; p.ED = (int)s->dim; p.N = (int)s->dstate;
     p.nchunks = (p.L + kTile - 1) / kTile;
