@@ -63,6 +63,45 @@ __device__ __forceinline__ float sigmoid_f(float v) {
     return __builtin_amdgcn_rcpf(1.0f + fast_exp2(-v * kLog2e));
 }
 
+// Element at a 32-bit BYTE offset from a wave-uniform pointer, through the buffer instructions:
+// one instruction per access (scalar descriptor + 32-bit vector offset), no 64-bit address
+// arithmetic or address registers per lane.  The descriptor is raw (stride 0) with the maximum
+// range, i.e. the access is not bounds-checked; callers keep offsets inside their tensors.
+typedef __amdgpu_buffer_rsrc_t rsrc_t;
+__device__ __forceinline__ rsrc_t make_rsrc(const void* base) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, 0xffffffff, 0x00020000);
+}
+__device__ __forceinline__ float ld_off(const float* base, uint32_t byte_off) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(make_rsrc(base), byte_off, 0, 0));
+}
+__device__ __forceinline__ bf16_t ld_off(const bf16_t* base, uint32_t byte_off) {
+    return __builtin_bit_cast(bf16_t, __builtin_amdgcn_raw_buffer_load_b16(make_rsrc(base), byte_off, 0, 0));
+}
+__device__ __forceinline__ void st_off(float* base, uint32_t byte_off, float v) {
+    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, v), make_rsrc(base), byte_off, 0, 0);
+}
+__device__ __forceinline__ void st_off(bf16_t* base, uint32_t byte_off, bf16_t v) {
+    __builtin_amdgcn_raw_buffer_store_b16(__builtin_bit_cast(unsigned short, v), make_rsrc(base), byte_off, 0, 0);
+}
+typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ void st_off(float2* base, uint32_t byte_off, float2 v) {
+    __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(u32x2, v), make_rsrc(base), byte_off, 0, 0);
+}
+__device__ __forceinline__ void st_off(float4* base, uint32_t byte_off, float4 v) {
+    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v), make_rsrc(base), byte_off, 0, 0);
+}
+
+// Lane index recomputed on the spot (two VALU instructions).  Per-lane addresses that are used
+// once per tile are derived from this instead of a value computed before the loop: the
+// compiler would keep such a value alive across the whole tile and, under register pressure,
+// spill it to scratch memory, where every reload costs a round trip of several hundred clocks.
+__device__ __forceinline__ int lane_now() {
+    int l;
+    asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(l));
+    return l;
+}
+
 __device__ __forceinline__ int wave_id() {
     // threadIdx.x / 64, told to the compiler as wave-uniform
     return __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x) >> 6);

@@ -35,10 +35,9 @@ struct BwdParams {
     int64_t bc_sb, bc_sl;
 };
 
-// Fast path (no gate): scan / loader / reducer waves, see sscan_bwd_fast.hip.  Returns
+// Fast path (no gate): scan and service waves, see sscan_bwd_fast.hip.  Returns
 // MPA_ERR_BAD_SHAPE when the shape is outside what it was instantiated for.
-int launch_bwd_fast(const BwdParams& p, const float* bcpack, int ns, int nw, int io_dtype,
-                    hipStream_t stream);
+int launch_bwd_fast(const BwdParams& p, int ns, int nw, int io_dtype, hipStream_t stream);
 bool bwd_fast_supported(int ns, int nw);
 
 }  // namespace mpa

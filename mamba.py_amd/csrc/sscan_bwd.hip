@@ -418,7 +418,7 @@ __global__ void __launch_bounds__(256) sscan_bwd_finish_kernel(
 }
 
 struct BwdWorkspace {
-    size_t offB, offC, offA, offD, offDb, offPack, total;
+    size_t offB, offC, offA, offD, offDb, total;
 };
 
 static BwdWorkspace bwd_workspace(const mpa_sscan_shape* s) {
@@ -433,8 +433,7 @@ static BwdWorkspace bwd_workspace(const mpa_sscan_shape* s) {
     w.offA = w.offC + up(cg * bln);
     w.offD = w.offA + up(ben);
     w.offDb = w.offD + up(be);
-    w.offPack = w.offDb + up(be);
-    w.total = (w.offPack + up(bcpack_floats(s))) * sizeof(float);
+    w.total = (w.offDb + up(be)) * sizeof(float);
     return w;
 }
 
@@ -519,11 +518,7 @@ extern "C" int mpa_sscan_bwd(const mpa_sscan_shape* s, const void* x, const void
     hipStream_t st = static_cast<hipStream_t>(stream);
     const char* force_general = getenv("MPA_BWD_GENERAL");
     if (!z && bwd_fast_supported(ns, nw) && !(force_general && force_general[0] == '1')) {
-        // fast path: B and C repacked as float32 for scalar loads, then the scan / loader /
-        // reducer kernel
-        float* pack = wsf + ws.offPack;
-        rc = launch_pack_bc(s, B, C, pack, ns, ns >= 16 ? 1 : 16 / ns /* BcPack<NS>::kSS */, st);
-        if (rc == MPA_OK) rc = launch_bwd_fast(p, pack, ns, nw, s->io_dtype, st);
+        rc = launch_bwd_fast(p, ns, nw, s->io_dtype, st);
     } else if (s->io_dtype == MPA_F32)
         rc = z ? dispatch_bwd<float, true>(p, ns, nw, st) : dispatch_bwd<float, false>(p, ns, nw, st);
     else

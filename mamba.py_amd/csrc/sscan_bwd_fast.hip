@@ -1,7 +1,7 @@
 // Fused selective-scan backward for gfx950, fast path (no output gate).
 //
-// Same roles as the forward kernel.  A workgroup owns 64 channels of one batch row and walks
-// the sequence from the last tile of kTile steps to the first.
+// A workgroup owns 64 channels of one batch row and walks the sequence from the last tile of
+// kTile steps to the first.
 //   * NW scan waves split d_state (NS states per lane, one channel per lane).  Per tile a
 //     scan wave reloads the state at the tile start from the forward checkpoints, recomputes
 //     the kTile steps keeping a[t] and a[t]*h[t-1] in registers (the recurrence is never
@@ -9,18 +9,26 @@
 //         g[t] = dy[t]*C[t] + a[t+1]*g[t+1]
 //         d(delta*A) = g*a*h[t-1]   -> dA += .*delta ;  ddelta += .*A
 //         sum_n g*B                 -> dx = delta*. ;   ddelta += x*.
-//         g*u (u = delta*x), dy*h   -> dB, dC, summed over the 64 channels of the wave by a
-//                                      wave by an in-register reduce-scatter (rs_stage).
-//     B and C come through scalar loads from the float32 pack the pre-pass wrote.
-//   * two loader waves fetch x, delta, dy two tiles ahead, convert, apply softplus and
-//     publish delta, u, dy and x as float32 LDS tiles; they also accumulate dD.
-//   * two reducer waves, one tile behind, sum the partial sum_n over the scan waves, finish
-//     dx and ddelta (softplus chain rule included), store them, and forward the per-tile
-//     dB/dC sums to the per-channel-group partial buffers.
+//         g*u (u = delta*x), dy*h   -> dB, dC, summed over the 64 channels of the wave by an
+//                                      in-register reduce-scatter (rs_stage).
+//     B and C of a tile sit in one register per state whose lane t of every row of 16 lanes
+//     holds step t; the FMAs pick their step with a DPP row broadcast (fmac_bcast), so B and C
+//     cost neither scalar registers nor extra instructions.
+//   * four service waves, one item of (channel, 4 steps) per thread and tile, do everything
+//     else: they request x, delta, dy, B, C five tiles ahead (three tiles in flight), convert,
+//     apply softplus and publish delta, u, dy, x, B, C as float32 LDS tiles two tiles ahead
+//     (accumulating dD on the way); one tile behind the scan they sum the partial sum_n over
+//     the scan waves, finish dx and ddelta (softplus chain rule included), store them, and
+//     forward the per-tile dB/dC sums to the per-channel-group partial buffers.  Their
+//     per-tile code is short and has one uniform branch for the ragged edge: a lone wave
+//     issues an instruction only every ~6 clocks and pays tens of clocks per branch, and every
+//     instruction it issues takes a VALU slot away from the scan waves of its SIMD.
 // Tiles in LDS are [64 channels][16 steps] float32 at a pitch of 20 floats.
 // Reductions over channel groups, batch and time go through deterministic partial buffers
 // summed by sscan_bwd_finish_kernel (no floating-point atomics: results are bitwise
 // reproducible).
+#include <type_traits>
+
 #include "sscan_bwd.h"
 
 namespace mpa {
@@ -77,25 +85,38 @@ __device__ __forceinline__ float rs_stage(float lo, float hi, int lane) {
     else return rs_dpp<0xB1>(lo, hi, (lane & 1) != 0);
 }
 
+constexpr int kSvc = 4;  // service waves per workgroup
+
+// compile-time loop: f(std::integral_constant<int, I>) for I = 0 .. N-1
+template <int I, int N, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+    if constexpr (I < N) {
+        f(std::integral_constant<int, I>{});
+        static_for<I + 1, N>(f);
+    }
+}
+
 template <int NS, int NW>
 struct BwdFastLds {
     static constexpr int NP = NS * NW;
     static constexpr size_t kInputs = 3 * 4 + 2;     // delta, x, dy: four buffers each; u: two
-    static constexpr size_t floats = (kInputs + 2 * NW) * kTileF + 2 * kTile * 2 * NP + 2 * 4 * kWave + 4;
+    // + partial sums per scan wave, dB|dC tile sums [2][kTile][2][NP], B|C tiles
+    // [2][2][NP][kTile], consumption flags
+    static constexpr size_t floats =
+        (kInputs + 2 * NW) * kTileF + 2 * kTile * 2 * NP + 2 * 2 * NP * kTile + 4;
 };
 
 template <typename IO, int NS, int NW>
-__global__ void __launch_bounds__((NW + 4) * kWave)
-    sscan_bwd_fast_kernel(const BwdParams p, const float* __restrict__ bcpack) {
+__global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(const BwdParams p) {
     constexpr int NP = NS * NW;
     constexpr int NQ = kTile / 4;
+    static_assert(kSvc == NQ, "one service thread per (channel, 4 steps) item of a tile");
     // channel reduction of dB/dC: 64 values (2 * NS per step, kBatch steps) per reduce-scatter
     constexpr int kStepBits = NS == 2 ? 2 : 3;  // stages spent inside one step: log2(2*NS)
     constexpr int kBatch = 64 / (2 * NS);       // steps per batch
     static_assert(NS == 2 || NS == 4, "reduce-scatter layout written for 2 or 4 states per lane");
-    constexpr int kSS = BcPack<NS>::kSS;        // steps per B/C sub-tile
-    constexpr int NSUB = kTile / kSS;
-    constexpr int kSub = 2 * kSS * NS;          // floats per sub-tile: B then C
+    constexpr int kRedF = kTile * 2 * NP;       // floats of one dB|dC tile
+    constexpr int kBcF = 2 * NP * kTile;        // floats of one B|C tile
 
     extern __shared__ float4 smem4[];
     float* const smem = reinterpret_cast<float*>(smem4);
@@ -106,9 +127,9 @@ __global__ void __launch_bounds__((NW + 4) * kWave)
     float* const sP1 = sU + 2 * kTileF;           // [NW] sum_n g*B
     float* const sP2 = sP1 + NW * kTileF;         // [NW] sum_n g*a*h[t-1]*A*log2(e)
     float* const sRed = sP2 + NW * kTileF;        // [2][kTile][2][NP] dB | dC tile sums
-    float* const sDD = sRed + 2 * kTile * 2 * NP;      // [2][4][kWave] dD, ddelta_bias partials
-    // one word per reducer wave: index of the last tile whose partial sums it has consumed
-    int* const sConsumed = reinterpret_cast<int*>(sDD + 2 * 4 * kWave);
+    float* const sBC = sRed + 2 * kRedF;          // [2][B|C][NP][kTile]
+    // one word per service wave: index of the last tile whose partial sums it has consumed
+    int* const sConsumed = reinterpret_cast<int*>(sBC + 2 * kBcF);
 
     const int lane = threadIdx.x & (kWave - 1);
     const int w = wave_id();
@@ -117,198 +138,262 @@ __global__ void __launch_bounds__((NW + 4) * kWave)
     const int d0 = cg * kWave;
     const int ntiles = p.nchunks;
     const int cmax = min(kWave, p.ED - d0) - 1;  // last valid channel of the group
+    // dD / ddelta_bias partials [2][4][kWave]: written once at the very end, into the delta
+    // buffer that no tile uses any more
+    float* const sDD = sDl + (ntiles & 3) * kTileF;
 
     // tile index k counts from the END of the sequence: tile k covers chunk c = ntiles-1-k
     auto chunk_of = [&](int k) { return ntiles - 1 - k; };
 
-    if (w >= NW + 2) {
-        // ================================ reducers ================================
-        const int sw = w - NW - 2;
-        int co[2], qo[2];
-        bool co_ok[2];
-        uint32_t cgo[2];
-        float Dr[2];
-        float dDb[2] = {0.0f, 0.0f};
+    if (w >= NW) {
+        // ================================ service waves ================================
+        const int sw = w - NW;
+        const int item = sw * kWave + lane;  // 0 .. 255
+        constexpr uint32_t kES = sizeof(IO);
+        const bool group_full = cmax == kWave - 1;
+
+        // ---- input side: item -> (channel, step group), offsets that never change ----
+        const int ci = p.in_tmajor ? item / NQ : item % kWave;
+        const int qi = p.in_tmajor ? item % NQ : item / kWave;
+        const bool ci_ok = ci <= cmax;
+        const int cic = min(ci, cmax);
+        const float bias = p.dbias ? p.dbias[d0 + cic] : 0.0f;
+        const IO* const xg = static_cast<const IO*>(p.x) + (b * p.u_sb + (int64_t)d0 * p.u_sd);
+        const IO* const dg = static_cast<const IO*>(p.delta) + (b * p.d_sb + (int64_t)d0 * p.d_sd);
+        const IO* const yg = static_cast<const IO*>(p.dy) + (b * p.y_sb + (int64_t)d0 * p.y_sd);
+        const IO* const Bg = static_cast<const IO*>(p.Bm) + b * p.bc_sb;
+        const IO* const Cg = static_cast<const IO*>(p.C) + b * p.bc_sb;
+        uint32_t offx[4], offd[4], offy[4];
 #pragma unroll
-        for (int r = 0; r < 2; ++r) {
-            const int item = sw * kWave + lane + r * 2 * kWave;
-            co[r] = p.out_tmajor ? item / NQ : item % kWave;
-            qo[r] = p.out_tmajor ? item % NQ : item / kWave;
-            co_ok[r] = co[r] <= cmax;
-            cgo[r] = (uint32_t)min(co[r], cmax) * (uint32_t)p.g_sd;
-            Dr[r] = p.D[d0 + min(co[r], cmax)];
+        for (int j = 0; j < 4; ++j) {
+            // byte offsets (see ld_off)
+            offx[j] = ((uint32_t)(4 * qi + j) * (uint32_t)p.u_sl + (uint32_t)cic * (uint32_t)p.u_sd) * kES;
+            offd[j] = ((uint32_t)(4 * qi + j) * (uint32_t)p.d_sl + (uint32_t)cic * (uint32_t)p.d_sd) * kES;
+            offy[j] = ((uint32_t)(4 * qi + j) * (uint32_t)p.y_sl + (uint32_t)cic * (uint32_t)p.y_sd) * kES;
         }
+        // B/C of a tile: kTile * NP elements each, kBcPer per service thread, step fastest
+        constexpr int kBcPer = NP * kTile / (kSvc * kWave);
+        static_assert(NP * kTile % (kSvc * kWave) == 0, "whole elements per thread");
+        int bct[kBcPer], bcn[kBcPer];
+        uint32_t offbc[kBcPer];
+#pragma unroll
+        for (int r = 0; r < kBcPer; ++r) {
+            const int e = item + r * (kSvc * kWave);
+            bct[r] = e % kTile;
+            bcn[r] = e / kTile;
+            offbc[r] = ((uint32_t)bct[r] * (uint32_t)p.bc_sl + (uint32_t)min(bcn[r], p.N - 1)) * kES;
+        }
+
+        // ---- output side: item -> (channel, step group) ----
+        const int co = p.out_tmajor ? item / NQ : item % kWave;
+        const int qo = p.out_tmajor ? item % NQ : item / kWave;
+        const bool co_ok = co <= cmax;
+        const float Dr = p.D[d0 + min(co, cmax)];
+        uint32_t offg[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            offg[j] = ((uint32_t)(4 * qo + j) * (uint32_t)p.g_sl + (uint32_t)min(co, cmax) * (uint32_t)p.g_sd) * kES;
         IO* const dxg = static_cast<IO*>(p.dx) + (b * p.g_sb + (int64_t)d0 * p.g_sd);
         IO* const ddg = static_cast<IO*>(p.ddelta) + (b * p.g_sb + (int64_t)d0 * p.g_sd);
-        const int rtid = sw * kWave + lane;  // 0..127: dB/dC forwarding
+        // dB/dC forwarding: kFw consecutive states of one (step, dB|dC) per thread
+        constexpr int kFw = kRedF / (kSvc * kWave);
+        static_assert(kRedF % (kSvc * kWave) == 0 && NP % kFw == 0 && (kFw == 2 || kFw == 4), "forwarding layout");
+        // (even service waves forward dB, odd ones dC, so that the destination is wave-uniform)
+        const int fw_which = sw & 1;
+        const int fw_i = ((sw >> 1) * kWave + lane) * kFw;  // index inside the [kTile][NP] half
+        const int fw_tt = fw_i / NP, fw_n = fw_i % NP;
+        const int fw_e = (fw_tt * 2 + fw_which) * NP + fw_n;  // index inside the dB|dC tile in LDS
+        float* const fw_base = (fw_which ? p.partC : p.partB) + ((int64_t)cg * p.batch + b) * p.L * p.N;
+        const uint32_t fw_off = ((uint32_t)fw_tt * (uint32_t)p.N + (uint32_t)fw_n) * 4u;
+        const bool fw_vec = p.N == NP;  // rows of the partial buffers are then aligned for vector stores
 
-        auto reduce_store = [&](int k) {
+        float dDacc = 0.0f, dDb = 0.0f;
+
+        // Raw values of three tiles in flight (see the forward kernel: HBM latency under load
+        // is longer than one tile interval)
+        struct Raw { IO x[4], d[4], y[4], b[kBcPer], c[kBcPer]; };
+        auto load_tile = [&](int kk, Raw& raw) {
+            // tiles and steps beyond the sequence are clamped, so the loads stay in bounds;
+            // only the offsets depend on the (uniform) branch, the loads are unconditional
+            const int k = min(kk, ntiles - 1);
             const int c = chunk_of(k);
-            IO* dxk = dxg + (int64_t)c * kTile * p.g_sl;
-            IO* ddk = ddg + (int64_t)c * kTile * p.g_sl;
-            float4 gBs[2], dds[2];
+            const IO* xk = xg + (int64_t)c * kTile * p.u_sl;
+            const IO* dk = dg + (int64_t)c * kTile * p.d_sl;
+            const IO* yk = yg + (int64_t)c * kTile * p.y_sl;
+            const IO* Bk = Bg + (int64_t)c * kTile * p.bc_sl;
+            const IO* Ck = Cg + (int64_t)c * kTile * p.bc_sl;
+            uint32_t ox[4], od[4], oy[4], ob[kBcPer];
 #pragma unroll
-            for (int r = 0; r < 2; ++r) {
-                const int ch = co[r], q = qo[r];
-                float4 gB = make_float4(0.f, 0.f, 0.f, 0.f), dd = gB;
+            for (int j = 0; j < 4; ++j) {
+                ox[j] = offx[j];
+                od[j] = offd[j];
+                oy[j] = offy[j];
+            }
 #pragma unroll
-                for (int ww = 0; ww < NW; ++ww) {
-                    const float4 a = tile_ld(sP1 + ww * kTileF, ch, q);
-                    const float4 e = tile_ld(sP2 + ww * kTileF, ch, q);
-                    gB.x += a.x; gB.y += a.y; gB.z += a.z; gB.w += a.w;
-                    dd.x += e.x; dd.y += e.y; dd.z += e.z; dd.w += e.w;
+            for (int r = 0; r < kBcPer; ++r) ob[r] = offbc[r];
+            if ((c + 1) * kTile > p.L) {
+                const int tmax = p.L - c * kTile - 1;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const uint32_t tc = (uint32_t)min(4 * qi + j, tmax);
+                    ox[j] = (tc * (uint32_t)p.u_sl + (uint32_t)cic * (uint32_t)p.u_sd) * kES;
+                    od[j] = (tc * (uint32_t)p.d_sl + (uint32_t)cic * (uint32_t)p.d_sd) * kES;
+                    oy[j] = (tc * (uint32_t)p.y_sl + (uint32_t)cic * (uint32_t)p.y_sd) * kES;
                 }
-                gBs[r] = gB;
-                dds[r] = dd;
+#pragma unroll
+                for (int r = 0; r < kBcPer; ++r)
+                    ob[r] = ((uint32_t)min(bct[r], tmax) * (uint32_t)p.bc_sl + (uint32_t)min(bcn[r], p.N - 1)) * kES;
+            }
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                raw.x[j] = ld_off(xk, ox[j]);
+                raw.d[j] = ld_off(dk, od[j]);
+                raw.y[j] = ld_off(yk, oy[j]);
+            }
+#pragma unroll
+            for (int r = 0; r < kBcPer; ++r) {
+                raw.b[r] = ld_off(Bk, ob[r]);
+                raw.c[r] = ld_off(Ck, ob[r]);
+            }
+        };
+        auto stage_tile = [&](int k, const Raw& raw) {
+            const int c = chunk_of(k);
+            float xv[4], dv[4], yv[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                xv[j] = to_float(raw.x[j]);
+                dv[j] = to_float(raw.d[j]);
+                yv[j] = to_float(raw.y[j]);
+            }
+            if (p.softplus) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) dv[j] = softplus_f(dv[j] + bias);
+            }
+            if (!group_full || (c + 1) * kTile > p.L) {
+                // padding (beyond the sequence or the channel count): delta = 0, u = 0, dy = 0
+                // make the step an exact no-op in both sweeps
+                const int t0 = c * kTile + 4 * qi;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const bool ok = ci_ok && t0 + j < p.L;
+                    xv[j] = ok ? xv[j] : 0.0f;
+                    dv[j] = ok ? dv[j] : 0.0f;
+                    yv[j] = ok ? yv[j] : 0.0f;
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < 4; ++j) dDacc = __builtin_fmaf(yv[j], xv[j], dDacc);
+            const int s4 = (k & 3) * kTileF;
+            tile_st(sDl + s4, ci, qi, dv[0], dv[1], dv[2], dv[3]);
+            tile_st(sU + (k & 1) * kTileF, ci, qi, dv[0] * xv[0], dv[1] * xv[1], dv[2] * xv[2], dv[3] * xv[3]);
+            tile_st(sDy + s4, ci, qi, yv[0], yv[1], yv[2], yv[3]);
+            tile_st(sX + s4, ci, qi, xv[0], xv[1], xv[2], xv[3]);
+#pragma unroll
+            for (int r = 0; r < kBcPer; ++r) {
+                // states beyond d_state: B = C = 0 (padded steps need no care: u = dy = 0)
+                const bool ok = bcn[r] < p.N;
+                float* dst = sBC + (k & 1) * kBcF + bcn[r] * kTile + bct[r];
+                dst[0] = ok ? to_float(raw.b[r]) : 0.0f;
+                dst[NP * kTile] = ok ? to_float(raw.c[r]) : 0.0f;
+            }
+        };
+        auto reduce_tile = [&](int k) {
+            const int c = chunk_of(k);
+            float4 gB = make_float4(0.f, 0.f, 0.f, 0.f), dd = gB;
+#pragma unroll
+            for (int ww = 0; ww < NW; ++ww) {
+                const float4 a = tile_ld(sP1 + ww * kTileF, co, qo);
+                const float4 e = tile_ld(sP2 + ww * kTileF, co, qo);
+                gB.x += a.x; gB.y += a.y; gB.z += a.z; gB.w += a.w;
+                dd.x += e.x; dd.y += e.y; dd.z += e.z; dd.w += e.w;
             }
             // the partial sums of tile k are in registers: the scan waves may overwrite them
             // (the release orders this store after the LDS reads above)
             if (lane == 0)
                 __hip_atomic_store(sConsumed + sw, k, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
+            const float4 dl4 = tile_ld(sDl + (k & 3) * kTileF, co, qo);
+            const float4 x4 = tile_ld(sX + (k & 3) * kTileF, co, qo);
+            const float4 dy4 = tile_ld(sDy + (k & 3) * kTileF, co, qo);
+            // this thread's share of the tile's dB / dC sums over the 64 channels
+            const float* red = sRed + (k & 1) * kRedF + fw_e;
+            float fw[kFw];
 #pragma unroll
-            for (int r = 0; r < 2; ++r) {
-                const int ch = co[r], q = qo[r];
-                const float4 gB = gBs[r], dd = dds[r];
-                const float4 dl = tile_ld(sDl + (k & 3) * kTileF, ch, q);
-                const float4 xv = tile_ld(sX + (k & 3) * kTileF, ch, q);
-                const float4 ddy = tile_ld(sDy + (k & 3) * kTileF, ch, q);
-                const float gBv[4] = {gB.x, gB.y, gB.z, gB.w}, ddv[4] = {dd.x, dd.y, dd.z, dd.w};
-                const float dlv[4] = {dl.x, dl.y, dl.z, dl.w}, xvv[4] = {xv.x, xv.y, xv.z, xv.w};
-                const float dyv[4] = {ddy.x, ddy.y, ddy.z, ddy.w};
-                const int t0 = c * kTile + 4 * q;
+            for (int i = 0; i < kFw; ++i) fw[i] = red[i];
+            const float gBv[4] = {gB.x, gB.y, gB.z, gB.w}, ddv[4] = {dd.x, dd.y, dd.z, dd.w};
+            const float dlv[4] = {dl4.x, dl4.y, dl4.z, dl4.w}, xvv[4] = {x4.x, x4.y, x4.z, x4.w};
+            const float dyv[4] = {dy4.x, dy4.y, dy4.z, dy4.w};
+            float dxv[4], dv[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                dxv[j] = __builtin_fmaf(dlv[j], gBv[j], Dr * dyv[j]);
+                dv[j] = __builtin_fmaf(xvv[j], gBv[j], ddv[j] * kLn2);
+            }
+            if (p.softplus) {
+                // d softplus(r)/dr = sigmoid(r) = 1 - exp(-softplus(r)); padded elements have
+                // delta = 0 and all-zero partial sums, so they add nothing to ddelta_bias
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
-                    const float dxv = __builtin_fmaf(dlv[j], gBv[j], Dr[r] * dyv[j]);
-                    float dv = __builtin_fmaf(xvv[j], gBv[j], ddv[j] * kLn2);
-                    if (p.softplus) {
-                        // d softplus(r)/dr = sigmoid(r) = 1 - exp(-softplus(r))
-                        dv *= (1.0f - __expf(-dlv[j]));
-                        if (co_ok[r] && t0 + j < p.L) dDb[r] += dv;
-                    }
-                    if (co_ok[r] && t0 + j < p.L) {
-                        const uint32_t o = (uint32_t)(4 * q + j) * (uint32_t)p.g_sl + cgo[r];
-                        dxk[o] = from_float<IO>(dxv);
-                        ddk[o] = from_float<IO>(dv);
-                    }
+                    dv[j] *= 1.0f - fast_exp2(-dlv[j] * kLog2e);
+                    dDb += dv[j];
                 }
             }
-            // forward this tile's dB / dC sums over the 64 channels to the partial buffers
-            const float* red = sRed + (k & 1) * (kTile * 2 * NP);
-            for (int e = rtid; e < kTile * 2 * NP; e += 2 * kWave) {
-                const int tt = e / (2 * NP), which = (e / NP) & 1, n = e % NP;
-                const int t = c * kTile + tt;
-                if (t < p.L && n < p.N) {
-                    float* dst = which ? p.partC : p.partB;
-                    dst[(((int64_t)cg * p.batch + b) * p.L + t) * p.N + n] = red[e];
+            IO* dxk = dxg + (int64_t)c * kTile * p.g_sl;
+            IO* ddk = ddg + (int64_t)c * kTile * p.g_sl;
+            float* fwk = fw_base + (int64_t)c * kTile * p.N;
+            if (group_full && (c + 1) * kTile <= p.L && fw_vec) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    st_off(dxk, offg[j], from_float<IO>(dxv[j]));
+                    st_off(ddk, offg[j], from_float<IO>(dv[j]));
                 }
+                if constexpr (kFw == 2)
+                    st_off(reinterpret_cast<float2*>(fwk), fw_off, make_float2(fw[0], fw[1]));
+                else
+                    st_off(reinterpret_cast<float4*>(fwk), fw_off, make_float4(fw[0], fw[1], fw[2], fw[3]));
+            } else {
+                const int t0 = c * kTile + 4 * qo;
+                for (int j = 0; j < 4; ++j)
+                    if (co_ok && t0 + j < p.L) {
+                        st_off(dxk, offg[j], from_float<IO>(dxv[j]));
+                        st_off(ddk, offg[j], from_float<IO>(dv[j]));
+                    }
+                for (int i = 0; i < kFw; ++i)
+                    if (c * kTile + fw_tt < p.L && fw_n + i < p.N) st_off(fwk, fw_off + 4u * i, fw[i]);
             }
         };
 
+        // tile j travels in register set j % 3; staging runs two tiles ahead of the scan, the
+        // reduction one tile behind
+        Raw ra, rb, rc;
         if (lane == 0) sConsumed[sw] = -1;
-        __syncthreads();
-        __syncthreads();
-        for (int k = 0; k < ntiles; ++k) {
-            if (k >= 1) reduce_store(k - 1);
-            __syncthreads();  // end of interval k
-        }
-        reduce_store(ntiles - 1);
-        if (p.softplus) {
-#pragma unroll
-            for (int r = 0; r < 2; ++r) sDD[(4 + qo[r]) * kWave + co[r]] = dDb[r];
-        }
-        __syncthreads();  // final
-        return;
-    }
-
-    if (w >= NW) {
-        // ================================ loaders ================================
-        const int sw = w - NW;
-        int ci[2], qi[2];
-        bool ci_ok[2];
-        uint32_t cx[2], cd[2], cy[2];
-        float bias[2], dDacc[2] = {0.0f, 0.0f};
-#pragma unroll
-        for (int r = 0; r < 2; ++r) {
-            const int item = sw * kWave + lane + r * 2 * kWave;
-            ci[r] = p.in_tmajor ? item / NQ : item % kWave;
-            qi[r] = p.in_tmajor ? item % NQ : item / kWave;
-            ci_ok[r] = ci[r] <= cmax;
-            const int cic = min(ci[r], cmax);
-            cx[r] = (uint32_t)cic * (uint32_t)p.u_sd;
-            cd[r] = (uint32_t)cic * (uint32_t)p.d_sd;
-            cy[r] = (uint32_t)cic * (uint32_t)p.y_sd;
-            bias[r] = p.dbias ? p.dbias[d0 + cic] : 0.0f;
-        }
-        const IO* const xg = static_cast<const IO*>(p.x) + (b * p.u_sb + (int64_t)d0 * p.u_sd);
-        const IO* const dg = static_cast<const IO*>(p.delta) + (b * p.d_sb + (int64_t)d0 * p.d_sd);
-        const IO* const yg = static_cast<const IO*>(p.dy) + (b * p.y_sb + (int64_t)d0 * p.y_sd);
-
-        IO rx[2][4], rd[2][4], ry[2][4];
-        auto load_tile = [&](int k) {
-            // steps beyond the sequence end are clamped to the last one: loads stay in bounds
-            // and free of branches
-            const int c = chunk_of(k);
-            const int tmax = min(kTile, p.L - c * kTile) - 1;
-            const IO* xk = xg + (int64_t)c * kTile * p.u_sl;
-            const IO* dk = dg + (int64_t)c * kTile * p.d_sl;
-            const IO* yk = yg + (int64_t)c * kTile * p.y_sl;
-#pragma unroll
-            for (int r = 0; r < 2; ++r) {
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const uint32_t tc = (uint32_t)min(4 * qi[r] + j, tmax);
-                    rx[r][j] = xk[tc * (uint32_t)p.u_sl + cx[r]];
-                    rd[r][j] = dk[tc * (uint32_t)p.d_sl + cd[r]];
-                    ry[r][j] = yk[tc * (uint32_t)p.y_sl + cy[r]];
-                }
-            }
-        };
-        auto stage_tile = [&](int k) {
-            const int c = chunk_of(k);
-#pragma unroll
-            for (int r = 0; r < 2; ++r) {
-                const int t0 = c * kTile + 4 * qi[r];
-                float dl[4], uu[4], xx[4], yy[4];
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    // padding (beyond the sequence or the channel count): delta = 0, u = 0,
-                    // dy = 0 make the step an exact no-op in both sweeps
-                    const bool ok = ci_ok[r] && t0 + j < p.L;
-                    const float xv = ok ? to_float(rx[r][j]) : 0.0f;
-                    const float yv = ok ? to_float(ry[r][j]) : 0.0f;
-                    float dv = to_float(rd[r][j]);
-                    if (p.softplus) dv = softplus_f(dv + bias[r]);
-                    dv = ok ? dv : 0.0f;
-                    dl[j] = dv;
-                    uu[j] = dv * xv;
-                    xx[j] = xv;
-                    yy[j] = yv;
-                    dDacc[r] = __builtin_fmaf(yv, xv, dDacc[r]);
-                }
-                const int ch = ci[r], q = qi[r], s4 = (k & 3) * kTileF;
-                tile_st(sDl + s4, ch, q, dl[0], dl[1], dl[2], dl[3]);
-                tile_st(sU + (k & 1) * kTileF, ch, q, uu[0], uu[1], uu[2], uu[3]);
-                tile_st(sDy + s4, ch, q, yy[0], yy[1], yy[2], yy[3]);
-                tile_st(sX + s4, ch, q, xx[0], xx[1], xx[2], xx[3]);
-            }
-        };
-
-        load_tile(0);
-        stage_tile(0);
-        if (ntiles > 1) {
-            load_tile(1);
-            stage_tile(1);
-        }
-        if (ntiles > 2) load_tile(2);
+        load_tile(0, ra);
+        load_tile(1, rb);
+        load_tile(2, rc);
+        stage_tile(0, ra);
+        load_tile(3, ra);
+        if (ntiles > 1) stage_tile(1, rb);
+        load_tile(4, rb);
         __syncthreads();  // tiles 0 and 1 are published
         __syncthreads();
-        for (int k = 0; k < ntiles; ++k) {
-            if (k + 2 < ntiles) stage_tile(k + 2);
-            if (k + 3 < ntiles) load_tile(k + 3);
+        for (int k = 0; k < ntiles; k += 3) {
+            if (k >= 1) reduce_tile(k - 1);
+            if (k + 2 < ntiles) stage_tile(k + 2, rc);
+            load_tile(k + 5, rc);
             __syncthreads();  // end of interval k
+            if (k + 1 >= ntiles) break;
+            reduce_tile(k);
+            if (k + 3 < ntiles) stage_tile(k + 3, ra);
+            load_tile(k + 6, ra);
+            __syncthreads();  // end of interval k + 1
+            if (k + 2 >= ntiles) break;
+            reduce_tile(k + 1);
+            if (k + 4 < ntiles) stage_tile(k + 4, rb);
+            load_tile(k + 7, rb);
+            __syncthreads();  // end of interval k + 2
         }
-#pragma unroll
-        for (int r = 0; r < 2; ++r) sDD[qi[r] * kWave + ci[r]] = dDacc[r];
+        reduce_tile(ntiles - 1);
+        sDD[qi * kWave + ci] = dDacc;
+        sDD[(4 + qo) * kWave + co] = dDb;
         __syncthreads();  // final
         // dD (and ddelta_bias): sum the four step groups of every channel
         if (sw == 0 && lane <= cmax) {
@@ -338,90 +423,85 @@ __global__ void __launch_bounds__((NW + 4) * kWave)
         dAacc[i] = 0.0f;
     }
     // state at the start of chunk c: checkpoint written after chunk c-1, or h0 / zero
-    const int64_t ck_lane = (int64_t)min(d, p.ED - 1);
+    // (uniform base + 32-bit lane offset, the offset rebuilt from lane_now() at each use)
     auto load_state = [&](int k, float (&hs)[NS]) {
         const int c = chunk_of(min(k, ntiles - 1));
+        const uint32_t ck_lane = (uint32_t)min(d0 + lane_now(), p.ED - 1);
+        const float* ck_base = p.ckpt + ((int64_t)b * ntiles + max(c - 1, 0)) * p.N * p.ED;
+        const float* h0_base = p.h0 ? p.h0 + (int64_t)b * p.ED * p.N : ck_base;
+        const bool first = c == 0;
 #pragma unroll
         for (int i = 0; i < NS; ++i) {
-            const int n = min(w * NS + i, p.N - 1);
+            const uint32_t n = (uint32_t)min(w * NS + i, p.N - 1);
             // branch-free: chunk 0 reads slot 0 (or h0) and the value is masked below
-            const float* src = p.ckpt + (((int64_t)b * ntiles + max(c - 1, 0)) * p.N + n) * p.ED + ck_lane;
-            const float* src0 = p.h0 ? p.h0 + ((int64_t)b * p.ED + ck_lane) * p.N + n : src;
-            const float v = *(c > 0 ? src : src0);
-            hs[i] = (c > 0 || p.h0) ? v : 0.0f;
+            const uint32_t off = first && p.h0 ? ck_lane * (uint32_t)p.N + n : n * (uint32_t)p.ED + ck_lane;
+            const float v = (first ? h0_base : ck_base)[off];
+            hs[i] = (!first || p.h0) ? v : 0.0f;
         }
     };
-    const float* bc = bcpack + ((int64_t)b * ntiles * NW + w) * (NSUB * kSub);
-    const int64_t bc_tile = (int64_t)NW * NSUB * kSub;
 
-    auto read_fwd_inputs = [&](int k, float (&dl)[kTile], float (&uu)[kTile]) {
+    // registers of one tile: delta and u of the lane's channel, and one register per state for
+    // B and for C whose lane t of every row holds step t
+    struct TileIn {
+        float dl[kTile], uu[kTile], vb[NS], vc[NS];
+    };
+    auto read_fwd_inputs = [&](int k, TileIn& r) {
 #pragma unroll
         for (int q = 0; q < NQ; ++q) {
             const float4 v = tile_ld(sDl + (k & 3) * kTileF, lane, q);
             const float4 u4 = tile_ld(sU + (k & 1) * kTileF, lane, q);
-            dl[4 * q] = v.x; dl[4 * q + 1] = v.y; dl[4 * q + 2] = v.z; dl[4 * q + 3] = v.w;
-            uu[4 * q] = u4.x; uu[4 * q + 1] = u4.y; uu[4 * q + 2] = u4.z; uu[4 * q + 3] = u4.w;
+            r.dl[4 * q] = v.x; r.dl[4 * q + 1] = v.y; r.dl[4 * q + 2] = v.z; r.dl[4 * q + 3] = v.w;
+            r.uu[4 * q] = u4.x; r.uu[4 * q + 1] = u4.y; r.uu[4 * q + 2] = u4.z; r.uu[4 * q + 3] = u4.w;
+        }
+        const float* bck = sBC + (k & 1) * kBcF + (w * NS) * kTile + (lane_now() & (kTile - 1));
+#pragma unroll
+        for (int i = 0; i < NS; ++i) {
+            r.vb[i] = bck[i * kTile];
+            r.vc[i] = bck[NP * kTile + i * kTile];
         }
     };
 
-    // B/C sub-tiles are consumed in the order F0..F(NSUB-1) (recompute, B only) then
-    // R(NSUB-1)..R0 (reverse sweep, B and C); fetch number s of a tile lands in bcb[s & 1]
-    float bcb[2][kSub];
     float hnext[NS];
 
-    auto tile_pass = [&](int k, const float (&dl)[kTile], const float (&uu)[kTile],
-                         float (&dl_next)[kTile], float (&uu_next)[kTile]) {
-        const int c = chunk_of(k);
-        const float* bck = bc + (int64_t)c * bc_tile;
-        const float* bck_next = bc + (int64_t)max(c - 1, 0) * bc_tile;
+    auto tile_pass = [&](int k, const TileIn& in, TileIn& next) {
         float h[NS];
 #pragma unroll
         for (int i = 0; i < NS; ++i) h[i] = hnext[i];
 
         // ---- 1. recompute the tile forward, keeping a and a*h[t-1] ----
         float aS[kTile][NS], tS[kTile][NS], dyq[2][4];
-#pragma unroll
-        for (int tt = 0; tt < kTile; ++tt) {
-            const int sub = tt / kSS, ts = tt % kSS;
-            const float(&cur)[kSub] = bcb[sub & 1];
+        static_for<0, kTile>([&](auto TT) {
+            constexpr int tt = decltype(TT)::value;
 #pragma unroll
             for (int i = 0; i < NS; ++i) {
-                const float a = fast_exp2(dl[tt] * A2[i]);
+                const float a = fast_exp2(in.dl[tt] * A2[i]);
                 const float th = a * h[i];
                 aS[tt][i] = a;
                 tS[tt][i] = th;
-                h[i] = __builtin_fmaf(uu[tt], cur[ts * NS + i], th);
+                h[i] = fmac_bcast<tt>(th, in.vb[i], in.uu[tt]);
             }
-            if (ts == 0) {
-                // next fetch right after the first use of the current one (the wait before a
-                // first use drains every scalar load and LDS read in flight)
+            if (tt == 0) {
+                // checkpoint of the next tile: a global load with a whole tile to arrive
                 __builtin_amdgcn_sched_barrier(0);
-                if (sub + 1 < NSUB)
-                    scalar_load<kSub>(bck + (sub + 1) * kSub, bcb[(sub + 1) & 1]);
-                else
-                    scalar_load<kSub>(bck + (NSUB - 1) * kSub, bcb[NSUB & 1]);
-                if (sub == 0) load_state(k + 1, hnext);
-                if (sub == NSUB - 1) {
-                    // dy of the last four steps, needed when the reverse sweep starts
-                    const float4 v = tile_ld(sDy + (k & 3) * kTileF, lane, NQ - 1);
-                    dyq[(NQ - 1) & 1][0] = v.x; dyq[(NQ - 1) & 1][1] = v.y;
-                    dyq[(NQ - 1) & 1][2] = v.z; dyq[(NQ - 1) & 1][3] = v.w;
-                }
+                load_state(k + 1, hnext);
                 __builtin_amdgcn_sched_barrier(0);
             }
-        }
+            if (tt == kTile - 4) {
+                // dy of the last four steps, needed when the reverse sweep starts
+                const float4 v = tile_ld(sDy + (k & 3) * kTileF, lane, NQ - 1);
+                dyq[(NQ - 1) & 1][0] = v.x; dyq[(NQ - 1) & 1][1] = v.y;
+                dyq[(NQ - 1) & 1][2] = v.z; dyq[(NQ - 1) & 1][3] = v.w;
+            }
+        });
 
         // ---- 2. reverse sweep ----
         float gBv[kTile], ddv[kTile];
         float pend[4];
-#pragma unroll
-        for (int tt = kTile - 1; tt >= 0; --tt) {
-            const int sub = tt / kSS, ts = tt % kSS;
-            const int fetch = NSUB + (NSUB - 1 - sub);  // fetch number of this sub-tile
-            const float(&cur)[kSub] = bcb[fetch & 1];
-            if ((tt & 3) == 3 && tt >= 4) {
+        static_for<0, kTile>([&](auto RT) {
+            constexpr int tt = kTile - 1 - decltype(RT)::value;
+            if constexpr ((tt & 3) == 3 && tt >= 4) {
                 // dy of the next (earlier) four steps, one group ahead of use
-                const int qn = (tt >> 2) - 1;
+                constexpr int qn = (tt >> 2) - (tt >= 4 ? 1 : 0);
                 const float4 v = tile_ld(sDy + (k & 3) * kTileF, lane, qn);
                 dyq[qn & 1][0] = v.x; dyq[qn & 1][1] = v.y; dyq[qn & 1][2] = v.z; dyq[qn & 1][3] = v.w;
             }
@@ -430,35 +510,23 @@ __global__ void __launch_bounds__((NW + 4) * kWave)
             float pB[NS], pC[NS];
 #pragma unroll
             for (int i = 0; i < NS; ++i) {
-                const float bv = cur[ts * NS + i];
-                const float cv = cur[kSS * NS + ts * NS + i];
-                const float g = __builtin_fmaf(dyv, cv, ag[i]);
-                const float hh = __builtin_fmaf(uu[tt], bv, tS[tt][i]);
+                const float g = fmac_bcast<tt>(ag[i], in.vc[i], dyv);
+                const float hh = fmac_bcast<tt>(tS[tt][i], in.vb[i], in.uu[tt]);
                 const float gha = g * tS[tt][i];
-                dAacc[i] = __builtin_fmaf(gha, dl[tt], dAacc[i]);
+                dAacc[i] = __builtin_fmaf(gha, in.dl[tt], dAacc[i]);
                 dd = __builtin_fmaf(gha, A2[i], dd);
-                gB = __builtin_fmaf(g, bv, gB);
+                gB = fmac_bcast<tt>(gB, in.vb[i], g);
                 ag[i] = aS[tt][i] * g;
-                pB[i] = g * uu[tt];
+                pB[i] = g * in.uu[tt];
                 pC[i] = dyv * hh;
             }
             gBv[tt] = gB;
             ddv[tt] = dd;
 
-            if (ts == kSS - 1) {
-                // first use of this sub-tile is done: fetch the next one in reverse order, or
-                // the first forward sub-tile of the next tile
-                __builtin_amdgcn_sched_barrier(0);
-                if (sub > 0)
-                    scalar_load<kSub>(bck + (sub - 1) * kSub, bcb[(fetch + 1) & 1]);
-                else
-                    scalar_load<kSub>(bck_next, bcb[0]);
-                __builtin_amdgcn_sched_barrier(0);
-            }
             if (tt == 2) {
-                // the registers of the consumed steps are free: fetch delta/u of the next tile
+                // fetch delta, u, B, C of the next tile (published two intervals ahead)
                 __builtin_amdgcn_sched_barrier(0);
-                read_fwd_inputs(k + 1, dl_next, uu_next);
+                read_fwd_inputs(k + 1, next);
                 __builtin_amdgcn_sched_barrier(0);
             }
             // ---- channel reduction of this step's dB / dC products (see rs_stage) ----
@@ -474,49 +542,56 @@ __global__ void __launch_bounds__((NW + 4) * kWave)
                     const float a2 = rs_stage<1>(pB[2], pC[2], lane), a3 = rs_stage<1>(pB[3], pC[3], lane);
                     r = rs_stage<3>(rs_stage<2>(a0, a2, lane), rs_stage<2>(a1, a3, lane), lane);
                 }
-                const int sb = tt % kBatch;  // step inside the batch
-                if (sb & 1) {
+                constexpr int sb = tt % kBatch;  // step inside the batch
+                if constexpr ((sb & 1) != 0) {
                     pend[0] = r;
                 } else {
                     r = rs_stage<kStepBits + 1>(r, pend[0], lane);
-                    if (sb & 2) {
+                    if constexpr ((sb & 2) != 0) {
                         pend[1] = r;
                     } else {
                         r = rs_stage<kStepBits + 2>(r, pend[1], lane);
-                        if (sb & 4) {
+                        if constexpr ((sb & 4) != 0) {
                             pend[2] = r;
                         } else {
                             r = rs_stage<kStepBits + 3>(r, pend[2], lane);
+                            bool done = true;
                             if constexpr (kBatch == 16) {
-                                if (sb & 8) {
+                                if constexpr ((sb & 8) != 0) {
                                     pend[3] = r;
+                                    done = false;
                                 } else {
                                     r = rs_stage<6>(r, pend[3], lane);
                                 }
                             }
-                            if (sb == 0) {
+                            if (done && sb == 0) {
                                 // lane l holds value number l: decode (step, dB|dC, state)
-                                const int which = lane >> 5;
-                                const int st = NS == 2 ? (lane >> 4) & 1 : (((lane >> 4) & 1) << 1) | ((lane >> 3) & 1);
-                                const int stp = NS == 2 ? (lane & 1) << 3 | (lane & 2) << 1 | (lane & 4) >> 1 | (lane & 8) >> 3
-                                                        : (lane & 1) << 2 | (lane & 2) | (lane & 4) >> 2;
-                                sRed[(k & 1) * (kTile * 2 * NP) + ((tt + stp) * 2 + which) * NP + w * NS + st] = r;
+                                const int ln = lane_now();
+                                const int which = ln >> 5;
+                                const int st = NS == 2 ? (ln >> 4) & 1 : (((ln >> 4) & 1) << 1) | ((ln >> 3) & 1);
+                                const int stp = NS == 2 ? (ln & 1) << 3 | (ln & 2) << 1 | (ln & 4) >> 1 | (ln & 8) >> 3
+                                                        : (ln & 1) << 2 | (ln & 2) | (ln & 4) >> 2;
+                                sRed[(k & 1) * kRedF + ((tt + stp) * 2 + which) * NP + w * NS + st] = r;
                             }
                         }
                     }
                 }
             }
-        }
-        // The partial sums go to single-buffered LDS tiles.  The reducers read tile k-1 at the
-        // start of this interval and publish that in sConsumed; by the end of the sweep that
-        // has long happened, so this wait normally falls through (bounded: a wave never
-        // spins forever).
+        });
+        // The partial sums go to single-buffered LDS tiles.  The service waves read tile k-1 at
+        // the start of this interval and publish that in sConsumed; by the end of the sweep
+        // that has normally happened, so this wait falls through (bounded: a wave never spins
+        // forever).
         if (k >= 1) {
             int spins = 0;
-            while ((__hip_atomic_load(sConsumed, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP) < k - 1 ||
-                    __hip_atomic_load(sConsumed + 1, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP) < k - 1) &&
-                   ++spins < (1 << 20))
+            for (;;) {
+                int done = k - 1;
+#pragma unroll
+                for (int i = 0; i < kSvc; ++i)
+                    done = min(done, __hip_atomic_load(sConsumed + i, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP));
+                if (done >= k - 1 || ++spins >= (1 << 20)) break;
                 __builtin_amdgcn_s_sleep(1);
+            }
         }
 #pragma unroll
         for (int q = 0; q < NQ; ++q) {
@@ -526,16 +601,15 @@ __global__ void __launch_bounds__((NW + 4) * kWave)
         __syncthreads();  // end of interval k: partial sums and dB/dC sums of tile k are visible
     };
 
-    float dlA[kTile], uuA[kTile], dlB[kTile], uuB[kTile];
-    scalar_load<kSub>(bc + (int64_t)chunk_of(0) * bc_tile, bcb[0]);
+    TileIn ta, tb;
     load_state(0, hnext);
     __syncthreads();
-    read_fwd_inputs(0, dlA, uuA);
+    read_fwd_inputs(0, ta);
     __syncthreads();
     for (int k = 0; k < ntiles; k += 2) {
-        tile_pass(k, dlA, uuA, dlB, uuB);
+        tile_pass(k, ta, tb);
         if (k + 1 >= ntiles) break;
-        tile_pass(k + 1, dlB, uuB, dlA, uuA);
+        tile_pass(k + 1, tb, ta);
     }
     // per-batch partial of dA
     if (dvalid) {
@@ -549,25 +623,24 @@ __global__ void __launch_bounds__((NW + 4) * kWave)
 }
 
 template <typename IO, int NS, int NW>
-static int launch_fast(const BwdParams& p, const float* bcpack, hipStream_t stream) {
+static int launch_fast(const BwdParams& p, hipStream_t stream) {
     dim3 grid((p.ED + kWave - 1) / kWave, p.batch);
-    dim3 block((NW + 4) * kWave);
+    dim3 block((NW + kSvc) * kWave);
     constexpr size_t lds = sizeof(float) * BwdFastLds<NS, NW>::floats;
     static_assert(lds <= 160 * 1024, "LDS budget");
     static const int attr_rc = allow_dynamic_lds(sscan_bwd_fast_kernel<IO, NS, NW>, lds);
     if (attr_rc != MPA_OK) return attr_rc;
-    hipLaunchKernelGGL((sscan_bwd_fast_kernel<IO, NS, NW>), grid, block, lds, stream, p, bcpack);
+    hipLaunchKernelGGL((sscan_bwd_fast_kernel<IO, NS, NW>), grid, block, lds, stream, p);
     return check_launch();
 }
 
 bool bwd_fast_supported(int ns, int nw) { return (ns == 2 && nw == 8) || (ns == 4 && nw == 4); }
 
-int launch_bwd_fast(const BwdParams& p, const float* bcpack, int ns, int nw, int io_dtype,
-                    hipStream_t stream) {
-#define MPA_CASE(NS_, NW_)                                                           \
-    if (ns == NS_ && nw == NW_)                                                      \
-        return io_dtype == MPA_F32 ? launch_fast<float, NS_, NW_>(p, bcpack, stream) \
-                                   : launch_fast<bf16_t, NS_, NW_>(p, bcpack, stream);
+int launch_bwd_fast(const BwdParams& p, int ns, int nw, int io_dtype, hipStream_t stream) {
+#define MPA_CASE(NS_, NW_)                                                   \
+    if (ns == NS_ && nw == NW_)                                              \
+        return io_dtype == MPA_F32 ? launch_fast<float, NS_, NW_>(p, stream) \
+                                   : launch_fast<bf16_t, NS_, NW_>(p, stream);
     MPA_CASE(2, 8) MPA_CASE(4, 4)
 #undef MPA_CASE
     return MPA_ERR_BAD_SHAPE;

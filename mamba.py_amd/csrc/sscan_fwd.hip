@@ -176,6 +176,7 @@ __global__ void __launch_bounds__((NW + kService) * kWave) sscan_fwd_kernel(cons
         const int sw = w - NW;                       // 0..3: loaders   4..7: reducers
         const int cmax = min(kWave, p.ED - d0) - 1;  // last valid channel of the group
         const int item = (sw & 3) * kWave + lane;    // 0 .. 255
+        constexpr uint32_t kES = sizeof(IO);
         if (sw < kLoaders) {
             // ------------------------------- loaders -------------------------------
             const int ci = p.in_tmajor ? item / NQ : item % kWave;
@@ -193,8 +194,9 @@ __global__ void __launch_bounds__((NW + kService) * kWave) sscan_fwd_kernel(cons
             uint32_t offx[4], offd[4];
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                offx[j] = (uint32_t)(4 * qi + j) * (uint32_t)p.u_sl + (uint32_t)cic * (uint32_t)p.u_sd;
-                offd[j] = (uint32_t)(4 * qi + j) * (uint32_t)p.d_sl + (uint32_t)cic * (uint32_t)p.d_sd;
+                // byte offsets (see ld_off)
+                offx[j] = ((uint32_t)(4 * qi + j) * (uint32_t)p.u_sl + (uint32_t)cic * (uint32_t)p.u_sd) * kES;
+                offd[j] = ((uint32_t)(4 * qi + j) * (uint32_t)p.d_sl + (uint32_t)cic * (uint32_t)p.d_sd) * kES;
             }
             const bool group_full = cmax == kWave - 1;
             // B/C of a tile: kTile * NP elements each, kBcPer per loader thread, step fastest
@@ -209,7 +211,7 @@ __global__ void __launch_bounds__((NW + kService) * kWave) sscan_fwd_kernel(cons
                 const int e = item + r * (kLoaders * kWave);
                 bct[r] = e % kTile;
                 bcn[r] = e / kTile;
-                offbc[r] = (uint32_t)bct[r] * (uint32_t)p.bc_sl + (uint32_t)min(bcn[r], p.N - 1);
+                offbc[r] = ((uint32_t)bct[r] * (uint32_t)p.bc_sl + (uint32_t)min(bcn[r], p.N - 1)) * kES;
             }
 
             // Raw values of three tiles in flight: HBM latency under load is longer than one
@@ -248,23 +250,23 @@ __global__ void __launch_bounds__((NW + kService) * kWave) sscan_fwd_kernel(cons
 #pragma unroll
                     for (int j = 0; j < 4; ++j) {
                         const uint32_t tc = (uint32_t)min(4 * qi + j, tmax);
-                        ox[j] = tc * (uint32_t)p.u_sl + (uint32_t)cic * (uint32_t)p.u_sd;
-                        od[j] = tc * (uint32_t)p.d_sl + (uint32_t)cic * (uint32_t)p.d_sd;
+                        ox[j] = (tc * (uint32_t)p.u_sl + (uint32_t)cic * (uint32_t)p.u_sd) * kES;
+                        od[j] = (tc * (uint32_t)p.d_sl + (uint32_t)cic * (uint32_t)p.d_sd) * kES;
                     }
 #pragma unroll
                     for (int r = 0; r < kBcPer; ++r)
-                        ob[r] = (uint32_t)min(bct[r], tmax) * (uint32_t)p.bc_sl + (uint32_t)min(bcn[r], p.N - 1);
+                        ob[r] = ((uint32_t)min(bct[r], tmax) * (uint32_t)p.bc_sl + (uint32_t)min(bcn[r], p.N - 1)) * kES;
                 }
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
-                    raw.x[j] = xk[ox[j]];
-                    raw.d[j] = dk[od[j]];
-                    if (has_z) raw.z[j] = zk[ox[j]];
+                    raw.x[j] = ld_off(xk, ox[j]);
+                    raw.d[j] = ld_off(dk, od[j]);
+                    if (has_z) raw.z[j] = ld_off(zk, ox[j]);
                 }
 #pragma unroll
                 for (int r = 0; r < kBcPer; ++r) {
-                    raw.b[r] = Bk[ob[r]];
-                    raw.c[r] = Ck[ob[r]];
+                    raw.b[r] = ld_off(Bk, ob[r]);
+                    raw.c[r] = ld_off(Ck, ob[r]);
                 }
                 if (!kBcast) raw.warm = warm[(int64_t)k * kPackVec];
             };
@@ -347,7 +349,7 @@ __global__ void __launch_bounds__((NW + kService) * kWave) sscan_fwd_kernel(cons
             uint32_t offy[4];
 #pragma unroll
             for (int j = 0; j < 4; ++j)
-                offy[j] = (uint32_t)(q4 + j) * (uint32_t)p.y_sl + (uint32_t)min(co, cmax) * (uint32_t)p.y_sd;
+                offy[j] = ((uint32_t)(q4 + j) * (uint32_t)p.y_sl + (uint32_t)min(co, cmax) * (uint32_t)p.y_sd) * kES;
             IO* const yg = static_cast<IO*>(p.y) + (b * p.y_sb + (int64_t)d0 * p.y_sd);
             auto reduce_store = [&](int k) {
                 IO* yk = yg + (int64_t)k * kTile * p.y_sl;
@@ -365,10 +367,10 @@ __global__ void __launch_bounds__((NW + kService) * kWave) sscan_fwd_kernel(cons
                 const int t0 = k * kTile + q4;
                 if (co_ok && t0 + 3 < p.L) {
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) yk[offy[j]] = from_float<IO>(sv[j]);
+                    for (int j = 0; j < 4; ++j) st_off(yk, offy[j], from_float<IO>(sv[j]));
                 } else if (co_ok) {
                     for (int j = 0; j < 4; ++j)
-                        if (t0 + j < p.L) yk[offy[j]] = from_float<IO>(sv[j]);
+                        if (t0 + j < p.L) st_off(yk, offy[j], from_float<IO>(sv[j]));
                 }
             };
             // the reducers run one tile behind the scan waves
@@ -567,11 +569,15 @@ int validate_shape(const mpa_sscan_shape* s) {
                           s->y_sd, s->g_sb, s->g_sl, s->g_sd, s->bc_sb, s->bc_sl, s->dbc_sb, s->dbc_sl};
     for (int64_t v : st)
         if (v < 0) return MPA_ERR_BAD_STRIDE;
-    // one (kTile steps x 64 channels) tile is addressed with 32-bit element offsets
+    // one (kTile steps x 64 channels) tile is addressed with 32-bit byte offsets; so are a
+    // tile of B / C and one checkpoint (d_state x dim floats)
     const int64_t tile[][2] = {{s->u_sl, s->u_sd}, {s->d_sl, s->d_sd}, {s->y_sl, s->y_sd},
                                {s->g_sl, s->g_sd}};
     for (const auto& v : tile)
-        if (v[0] * kTile + v[1] * kWave >= ((int64_t)1 << 31)) return MPA_ERR_BAD_STRIDE;
+        if (v[0] * kTile + v[1] * kWave >= ((int64_t)1 << 30)) return MPA_ERR_BAD_STRIDE;
+    if (s->bc_sl * kTile + s->dstate >= ((int64_t)1 << 30) || s->dbc_sl * kTile + s->dstate >= ((int64_t)1 << 30))
+        return MPA_ERR_BAD_STRIDE;
+    if (s->dstate * s->dim >= ((int64_t)1 << 30)) return MPA_ERR_BAD_SHAPE;
     return MPA_OK;
 }
 
