@@ -128,7 +128,8 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
     float* const sP2 = sP1 + NW * kTileF;         // [NW] sum_n g*a*h[t-1]*A*log2(e)
     float* const sRed = sP2 + NW * kTileF;        // [2][kTile][2][NP] dB | dC tile sums
     float* const sBC = sRed + 2 * kRedF;          // [2][B|C][NP][kTile]
-    // one word per service wave: index of the last tile whose partial sums it has consumed
+    // counts (service wave, tile) pairs whose partial sums have been consumed: kSvc * (k + 1)
+    // once every service wave is done with tile k
     int* const sConsumed = reinterpret_cast<int*>(sBC + 2 * kBcF);
 
     const int lane = threadIdx.x & (kWave - 1);
@@ -310,7 +311,7 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
             // the partial sums of tile k are in registers: the scan waves may overwrite them
             // (the release orders this store after the LDS reads above)
             if (lane == 0)
-                __hip_atomic_store(sConsumed + sw, k, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
+                __hip_atomic_fetch_add(sConsumed, 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
             const float4 dl4 = tile_ld(sDl + (k & 3) * kTileF, co, qo);
             const float4 x4 = tile_ld(sX + (k & 3) * kTileF, co, qo);
             const float4 dy4 = tile_ld(sDy + (k & 3) * kTileF, co, qo);
@@ -365,7 +366,7 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
         // tile j travels in register set j % 3; staging runs two tiles ahead of the scan, the
         // reduction one tile behind
         Raw ra, rb, rc;
-        if (lane == 0) sConsumed[sw] = -1;
+        if (sw == 0 && lane == 0) sConsumed[0] = 0;
         load_tile(0, ra);
         load_tile(1, rb);
         load_tile(2, rc);
@@ -497,6 +498,7 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
         // ---- 2. reverse sweep ----
         float gBv[kTile], ddv[kTile];
         float pend[4];
+        int consumed = 0;
         static_for<0, kTile>([&](auto RT) {
             constexpr int tt = kTile - 1 - decltype(RT)::value;
             if constexpr ((tt & 3) == 3 && tt >= 4) {
@@ -523,6 +525,10 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
             gBv[tt] = gB;
             ddv[tt] = dd;
 
+            if (tt == 4) {
+                // first look at the consumption counter, early enough to hide the LDS latency
+                consumed = __hip_atomic_load(sConsumed, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP);
+            }
             if (tt == 2) {
                 // fetch delta, u, B, C of the next tile (published two intervals ahead)
                 __builtin_amdgcn_sched_barrier(0);
@@ -584,13 +590,9 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
         // forever).
         if (k >= 1) {
             int spins = 0;
-            for (;;) {
-                int done = k - 1;
-#pragma unroll
-                for (int i = 0; i < kSvc; ++i)
-                    done = min(done, __hip_atomic_load(sConsumed + i, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP));
-                if (done >= k - 1 || ++spins >= (1 << 20)) break;
+            while (consumed < kSvc * k && ++spins < (1 << 20)) {
                 __builtin_amdgcn_s_sleep(1);
+                consumed = __hip_atomic_load(sConsumed, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP);
             }
         }
 #pragma unroll
