@@ -142,6 +142,14 @@ __device__ __forceinline__ float fmac_bcast(float acc, float v, float x) {
         : "v"(v), "v"(x), "n"(T));
     return acc;
 }
+// v[lane T of the reader's row] * x (same broadcast, no accumulator)
+template <int T>
+__device__ __forceinline__ float mul_bcast(float v, float x) {
+    static_assert(T >= 0 && T < 16, "lane inside a row");
+    float r;
+    asm("v_mul_f32_dpp %0, %1, %2 row_newbcast:%3 row_mask:0xf bank_mask:0xf" : "=v"(r) : "v"(v), "v"(x), "n"(T));
+    return r;
+}
 
 inline int check_launch() { return hipGetLastError() == hipSuccess ? MPA_OK : MPA_ERR_LAUNCH; }
 

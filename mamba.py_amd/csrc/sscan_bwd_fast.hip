@@ -4,7 +4,7 @@
 // kTile steps to the first.
 //   * NW scan waves split d_state (NS states per lane, one channel per lane).  Per tile a
 //     scan wave reloads the state at the tile start from the forward checkpoints, recomputes
-//     the kTile steps keeping a[t] and a[t]*h[t-1] in registers (the recurrence is never
+//     the kTile steps keeping a[t] and h[t] in registers (the recurrence is never
 //     inverted: dividing by a[t] amplifies rounding error), then sweeps the tile backwards:
 //         g[t] = dy[t]*C[t] + a[t+1]*g[t+1]
 //         d(delta*A) = g*a*h[t-1]   -> dA += .*delta ;  ddelta += .*A
@@ -465,21 +465,22 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
     float hnext[NS];
 
     auto tile_pass = [&](int k, const TileIn& in, TileIn& next) {
-        float h[NS];
+        float hin[NS];  // state at the tile start
 #pragma unroll
-        for (int i = 0; i < NS; ++i) h[i] = hnext[i];
+        for (int i = 0; i < NS; ++i) hin[i] = hnext[i];
 
-        // ---- 1. recompute the tile forward, keeping a and a*h[t-1] ----
-        float aS[kTile][NS], tS[kTile][NS], dyq[2][4];
+        // ---- 1. recompute the tile forward, keeping a[t] and h[t] ----
+        float aS[kTile][NS], hS[kTile][NS], dyq[2][4];
         static_for<0, kTile>([&](auto TT) {
             constexpr int tt = decltype(TT)::value;
 #pragma unroll
             for (int i = 0; i < NS; ++i) {
                 const float a = fast_exp2(in.dl[tt] * A2[i]);
-                const float th = a * h[i];
+                float hprev;
+                if constexpr (tt == 0) hprev = hin[i];
+                else hprev = hS[tt > 0 ? tt - 1 : 0][i];
                 aS[tt][i] = a;
-                tS[tt][i] = th;
-                h[i] = fmac_bcast<tt>(th, in.vb[i], in.uu[tt]);
+                hS[tt][i] = fmac_bcast<tt>(a * hprev, in.vb[i], in.uu[tt]);
             }
             if (tt == 0) {
                 // checkpoint of the next tile: a global load with a whole tile to arrive
@@ -508,19 +509,23 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
                 dyq[qn & 1][0] = v.x; dyq[qn & 1][1] = v.y; dyq[qn & 1][2] = v.z; dyq[qn & 1][3] = v.w;
             }
             const float dyv = dyq[(tt >> 2) & 1][tt & 3];
-            float gB = 0.0f, dd = 0.0f;
+            float gB, dd = 0.0f;
             float pB[NS], pC[NS];
 #pragma unroll
             for (int i = 0; i < NS; ++i) {
+                // g[t] = dy*C + a[t+1]*g[t+1];  a[t]*g[t] serves the next (earlier) step and,
+                // times h[t-1], is d(delta*A)
                 const float g = fmac_bcast<tt>(ag[i], in.vc[i], dyv);
-                const float hh = fmac_bcast<tt>(tS[tt][i], in.vb[i], in.uu[tt]);
-                const float gha = g * tS[tt][i];
+                float hprev;
+                if constexpr (tt == 0) hprev = hin[i];
+                else hprev = hS[tt > 0 ? tt - 1 : 0][i];
+                ag[i] = aS[tt][i] * g;
+                const float gha = ag[i] * hprev;
                 dAacc[i] = __builtin_fmaf(gha, in.dl[tt], dAacc[i]);
                 dd = __builtin_fmaf(gha, A2[i], dd);
-                gB = fmac_bcast<tt>(gB, in.vb[i], g);
-                ag[i] = aS[tt][i] * g;
+                gB = i == 0 ? mul_bcast<tt>(in.vb[i], g) : fmac_bcast<tt>(gB, in.vb[i], g);
                 pB[i] = g * in.uu[tt];
-                pC[i] = dyv * hh;
+                pC[i] = dyv * hS[tt][i];
             }
             gBv[tt] = gB;
             ddv[tt] = dd;

@@ -120,12 +120,12 @@ struct FwdLds {
 template <int TT, int NS>
 __device__ __forceinline__ float scan_step_bcast(float dlv, float uuv, const float (&A2)[NS], float (&h)[NS],
                                                  const float (&vb)[NS], const float (&vc)[NS]) {
-    float sum = 0.0f;
+    float sum;
 #pragma unroll
     for (int i = 0; i < NS; ++i) {
         const float a = fast_exp2(dlv * A2[i]);
         h[i] = fmac_bcast<TT>(a * h[i], vb[i], uuv);
-        sum = fmac_bcast<TT>(sum, vc[i], h[i]);
+        sum = i == 0 ? mul_bcast<TT>(vc[i], h[i]) : fmac_bcast<TT>(sum, vc[i], h[i]);
     }
     return sum;
 }
