@@ -32,7 +32,7 @@ WORKLOADS = {
 # HBM bytes per launch of the backward entry point measured with rocprofv3 --pmc
 # (FETCH_SIZE + WRITE_SIZE, scaled by a copy kernel of known size); filled from the
 # summaries under profiles/.  None = not measured for that workload.
-MEASURED_TRAFFIC_BYTES = {"c2": 1.2526e9}
+MEASURED_TRAFFIC_BYTES = {"c2": 1.2196e9}
 
 
 def algorithmic_bytes(B, L, ED, N, s):
@@ -161,11 +161,11 @@ def main():
         "data": "synthetic (seeded, S4D-real A, softplus delta; values resident in HBM)",
         "config": {"workload": desc, "B": B, "L": L, "ED": ED, "N": N,
                    "algorithmic_bytes_fwd": fwd_b, "algorithmic_bytes_bwd": bwd_b},
-        "roofline": {"bound": "hbm", "kernel": "mpa_sscan_bwd (pack_bc_kernel + sscan_bwd_fast_kernel + sscan_bwd_finish_kernel)",
+        "roofline": {"bound": "hbm", "kernel": "mpa_sscan_bwd (sscan_bwd_fast_kernel + sscan_bwd_finish_kernel)",
                      "achieved": bwd_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": bwd_gbs / HBM_PEAK_GBS,
                      "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload)},
-        "forward": {"kernel": "mpa_sscan_fwd (pack_bc_kernel + sscan_fwd_kernel)",
+        "forward": {"kernel": "mpa_sscan_fwd (sscan_fwd_kernel)",
                     "achieved": fwd_b / (fwd_ms * 1e-3) / 1e9, "unit": "GB/s",
                     "frac": fwd_b / (fwd_ms * 1e-3) / 1e9 / HBM_PEAK_GBS},
     }
