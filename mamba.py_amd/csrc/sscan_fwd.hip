@@ -8,16 +8,19 @@
 //  * A workgroup owns 64 channels of one batch row.  NW "scan" waves split the d_state axis:
 //    wave w keeps NS states (n = w*NS ..) of the 64 channels in registers, one channel per
 //    lane, and walks the sequence in tiles of kTile steps.
-//  * Four "service" waves do everything that is per (step, channel) rather than per state,
-//    one tile ahead / behind the scan waves: they load x, delta (z) from HBM, convert them,
-//    apply softplus, form u = delta*x and D*x, and publish float32 tiles in LDS; one tile
-//    later they sum the NW partial readouts, apply the gate and store y.  Scan and service
-//    waves meet at ONE workgroup barrier per tile, so HBM latency, conversions and the
-//    cross-wave reduction overlap with the recurrence arithmetic instead of preceding it.
-//  * B and C are wave-uniform (they do not depend on the channel).  A small pre-pass packs
-//    them as float32 in the order each scan wave consumes them, and the scan waves fetch
-//    them with scalar loads into SGPRs: no LDS traffic, no vector registers, no conversions
-//    in the loop.
+//  * Eight "service" waves do everything that is per (step, channel) rather than per state.
+//    Four loader waves request x, delta (z), B, C five tiles ahead, convert them, apply
+//    softplus, form u = delta*x and D*x, and publish float32 tiles in LDS two tiles ahead of
+//    the scan; four reducer waves, one tile behind, sum the NW partial readouts, apply the
+//    gate and store y.  Scan and service waves meet at ONE workgroup barrier per tile, so HBM
+//    latency, conversions and the cross-wave reduction overlap with the recurrence
+//    arithmetic instead of preceding it.
+//  * B and C are wave-uniform (they do not depend on the channel).  Up to 8 states per lane
+//    they are staged in LDS and each scan wave loads, per state, one register whose lane t of
+//    every 16-lane row holds step t; the FMAs read their step through a DPP row broadcast
+//    (fmac_bcast), so B and C cost no extra instructions and no scalar registers.  Above that
+//    a small pre-pass packs them as float32 in the order each scan wave consumes them and the
+//    scan waves fetch them with scalar loads into SGPRs.
 //  * Both channel-contiguous and time-contiguous ((B,ED,L) memory) operands are read and
 //    written coalesced: a service thread owns 4 consecutive steps of one channel, and the
 //    thread -> (channel, step group) map follows the unit-stride axis.
@@ -641,6 +644,9 @@ extern "C" int64_t mpa_sscan_ckpt_elems(const mpa_sscan_shape* s) {
 
 extern "C" size_t mpa_sscan_fwd_workspace_bytes(const mpa_sscan_shape* s) {
     if (validate_shape(s) != MPA_OK) return 0;
+    // the packed B/C exist only on the scalar-load path (more than 8 states per lane)
+    const int ns = pick_states_per_lane(s->batch, s->dim, s->dstate, 32, "MPA_FWD_NS");
+    if (ns <= 8) return 256;
     return (bcpack_floats(s) * sizeof(float) + 255) / 256 * 256;
 }
 
