@@ -77,12 +77,101 @@ def cpu_baseline(workload, torch, so):
     }
 
 
+def _timed(torch, fn, steps, warmup):
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        fn()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / steps
+
+
+def bench_decode(args, torch, pkg, dev):
+    """configs[3]: decode with cached state at the mamba-2.8b layer shape, batch 64; one bench
+    step = 256 tokens through (a) the state-update kernel alone (mpa_ssm_step, in place) and
+    (b) one whole MambaBlock.step (projections and conv window on PyTorch-ROCm)."""
+    Bsz, d_model, ED, N, tokens = 64, 2560, 5120, 16, 256
+    g = torch.Generator().manual_seed(1003)
+    r = lambda *sh: torch.randn(*sh, generator=g).to(dev)
+    h = r(Bsz, ED, N)
+    x, dl, z, Bm, C = r(Bsz, ED), r(Bsz, ED), r(Bsz, ED), r(Bsz, N), r(Bsz, N)
+    A = -torch.arange(1, N + 1, dtype=torch.float32).repeat(ED, 1).to(dev)
+    D, bias = torch.ones(ED, device=dev), r(ED) * 0.1
+
+    def kernel_tokens():
+        for _ in range(tokens):
+            pkg.ssm_step(x, dl, A, Bm, C, D, h, z=z, delta_bias=bias, delta_softplus=True, inplace=True)
+
+    cfg = pkg.MambaConfig(d_model=d_model, n_layers=1, d_state=N)
+    block = pkg.MambaBlock(cfg).to(dev)
+    cache = (r(Bsz, ED, N), r(Bsz, ED, cfg.d_conv - 1))
+    xin = r(Bsz, d_model)
+
+    def block_tokens():
+        c = cache
+        with torch.no_grad():
+            for _ in range(tokens):
+                _, c = block.step(xin, c)
+
+    steps, warmup = max(1, args.steps // 10), 1
+    t_kernel = _timed(torch, kernel_tokens, steps, warmup) / tokens
+    t_block = _timed(torch, block_tokens, steps, warmup) / tokens
+    bytes_step = 2 * 4 * Bsz * ED * N + 4 * 4 * Bsz * ED + 4 * (ED * N + 2 * ED) + 2 * 4 * Bsz * N
+    out = {
+        "metric": "decode step latency per token (state-update kernel), mamba-2.8b layer, batch 64",
+        "value": t_kernel * 1e6, "unit": "us/token-step", "higher_is_better": False,
+        "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": t_kernel * tokens * 1e3,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic (seeded)",
+        "tokens_per_s_layer_kernel": Bsz / t_kernel,
+        "block_step_us": t_block * 1e6, "tokens_per_s_layer_block": Bsz / t_block,
+        "config": {"workload": "configs[3]: decode step, ED=5120 N=16 batch 64, 256 tokens per bench step",
+                   "algorithmic_bytes_per_token_step": bytes_step},
+        "roofline": {"bound": "hbm", "kernel": "ssm_step_kernel", "achieved": bytes_step / t_kernel / 1e9,
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": bytes_step / t_kernel / 1e9 / HBM_PEAK_GBS,
+                     "traffic": None},
+    }
+    print(json.dumps(out))
+
+
+def bench_lm_forward(args, torch, pkg, dev, L):
+    """configs[4]: random-init LM forward at the mamba-130m architecture, bf16 weights and
+    activations, fp32 scan state, B=8, uniform-random token ids."""
+    Bsz, vocab = 8, 50280
+    cfg = pkg.MambaConfig(d_model=768, n_layers=24, d_state=16)
+    torch.manual_seed(1004)
+    model = pkg.LM(cfg, vocab, pad_vocab_size_multiple=8).to(dev).to(torch.bfloat16)
+    ids = torch.randint(0, vocab, (Bsz, L), generator=torch.Generator().manual_seed(1004)).to(dev)
+
+    def fwd():
+        with torch.no_grad():
+            model(ids)
+
+    steps, warmup = max(2, args.steps // 5), 2
+    t = _timed(torch, fwd, steps, warmup)
+    ED, N = cfg.d_inner, cfg.d_state
+    scan_bytes = cfg.n_layers * (2 * (3 * Bsz * L * ED + 2 * Bsz * L * N) + 4 * (ED * N + ED))
+    out = {
+        "metric": f"LM forward tokens/s, mamba-130m architecture, B=8 L={L}",
+        "value": Bsz * L / t, "unit": "tokens/s", "higher_is_better": True,
+        "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": t * 1e3,
+        "scaling": "weak", "vs_baseline": None, "dtype": "bf16 weights/activations, f32 scan state",
+        "data": "synthetic (random-init weights, uniform-random token ids)",
+        "config": {"workload": f"configs[4]: LM forward 24 layers d_model=768 vocab 50280, B=8 L={L}",
+                   "scan_algorithmic_bytes_all_layers": scan_bytes},
+    }
+    print(json.dumps(out))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS))
+    ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS) + ["c3", "c4", "c4-3000"],
+                    help="c2 (default) is the headline workload; c3 = decode step, c4 = LM forward "
+                         "(reported with their own metric, same one-line schema)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run a plain 256 MiB device copy (reference point that scales the "
@@ -99,6 +188,11 @@ def main():
     if not torch.cuda.is_available():
         sys.exit("bench.py: no GPU visible")
     dev = torch.device("cuda:0")
+
+    if args.workload == "c3":
+        return bench_decode(args, torch, pkg, dev)
+    if args.workload.startswith("c4"):
+        return bench_lm_forward(args, torch, pkg, dev, 3000 if args.workload == "c4-3000" else 4096)
 
     B, L, ED, N, dtname, seed, desc = WORKLOADS[args.workload]
     dtype = getattr(torch, dtname)

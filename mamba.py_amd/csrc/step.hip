@@ -77,6 +77,66 @@ __global__ void __launch_bounds__(256) ssm_step_kernel(const StepParams p) {
     store_from_float<IO>(p.y, row, yv);
 }
 
+// Variant for d_state = 4*Q with Q a power of two: Q lanes share one row, four states each.
+// A wave then reads and writes h as one contiguous, fully used block per instruction (the
+// one-lane-per-row kernel touches every cache line of a 4 KB block with each of its loads),
+// all of a lane's loads are issued before the first use, and four times as many waves are in
+// flight, which is what a kernel this short needs.  The readout is summed over the Q lanes of
+// a row with lane exchanges.
+template <typename IO, int Q>
+__global__ void __launch_bounds__(256) ssm_step_quad_kernel(const StepParams p) {
+    const int64_t gid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t row = gid / Q;  // b*ED + d
+    const int part = (int)(gid % Q);
+    if (row >= (int64_t)p.batch * p.ED) return;  // Q divides 64: a row's lanes leave together
+    const int b = (int)(row / p.ED);
+    const int d = (int)(row % p.ED);
+    const int n0 = 4 * part;
+    const float4 h4 = p.hin ? *reinterpret_cast<const float4*>(p.hin + row * p.N + n0) : make_float4(0, 0, 0, 0);
+    const float4 a4 = *reinterpret_cast<const float4*>(p.A + (int64_t)d * p.N + n0);
+    const int64_t bc = (int64_t)b * p.bc_stride + n0;
+    float bv[4], cv[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        bv[k] = load_as_float<IO>(p.Bm, bc + k);
+        cv[k] = load_as_float<IO>(p.C, bc + k);
+    }
+    const float xv = load_as_float<IO>(p.x, row);
+    float dv = load_as_float<IO>(p.delta, row);
+    const float zv = p.z ? load_as_float<IO>(p.z, row) : 0.0f;
+    const float Dv = p.D[d];
+    if (p.softplus) dv = softplus_f(dv + (p.dbias ? p.dbias[d] : 0.0f));
+    const float dl2 = dv * kLog2e;
+    const float u = dv * xv;
+    const float av[4] = {a4.x, a4.y, a4.z, a4.w};
+    float hv[4] = {h4.x, h4.y, h4.z, h4.w};
+    float acc = 0.0f;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        hv[k] = __builtin_fmaf(u, bv[k], fast_exp2(dl2 * av[k]) * hv[k]);
+        acc = __builtin_fmaf(cv[k], hv[k], acc);
+    }
+    *reinterpret_cast<float4*>(p.hout + row * p.N + n0) = make_float4(hv[0], hv[1], hv[2], hv[3]);
+#pragma unroll
+    for (int m = 1; m < Q; m *= 2) acc += __shfl_xor(acc, m);
+    if (part == 0) {
+        float yv = __builtin_fmaf(Dv, xv, acc);
+        if (p.z) yv *= zv * sigmoid_f(zv);
+        store_from_float<IO>(p.y, row, yv);
+    }
+}
+
+template <typename IO>
+static bool launch_step_quad(const StepParams& p, int q, hipStream_t st) {
+    const int64_t threads = (int64_t)p.batch * p.ED * q;
+    dim3 grid((unsigned)((threads + 255) / 256));
+#define MPA_Q(Q_) \
+    if (q == Q_) { hipLaunchKernelGGL((ssm_step_quad_kernel<IO, Q_>), grid, dim3(256), 0, st, p); return true; }
+    MPA_Q(1) MPA_Q(2) MPA_Q(4) MPA_Q(8) MPA_Q(16)
+#undef MPA_Q
+    return false;
+}
+
 }  // namespace mpa
 
 using namespace mpa;
@@ -108,6 +168,12 @@ extern "C" int mpa_ssm_step(const void* x, const void* delta, const float* A, co
     const int64_t rows = batch * dim;
     dim3 grid((unsigned)((rows + 255) / 256));
     hipStream_t st = static_cast<hipStream_t>(stream);
+    // d_state = 4*Q, Q a power of two up to 16: the lanes-per-row kernel
+    const int q = (int)(dstate / 4);
+    if (vec4 && q >= 1 && q <= 16 && (q & (q - 1)) == 0 && rows * q < ((int64_t)1 << 31) * 256) {
+        const bool ok = io_dtype == MPA_F32 ? launch_step_quad<float>(p, q, st) : launch_step_quad<bf16_t>(p, q, st);
+        if (ok) return check_launch();
+    }
     if (io_dtype == MPA_F32) {
         if (vec4) hipLaunchKernelGGL((ssm_step_kernel<float, 4>), grid, dim3(256), 0, st, p);
         else hipLaunchKernelGGL((ssm_step_kernel<float, 1>), grid, dim3(256), 0, st, p);
