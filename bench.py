@@ -128,9 +128,56 @@ def bench_decode(args, torch, pkg, dev):
         "block_step_us": t_block * 1e6, "tokens_per_s_layer_block": Bsz / t_block,
         "config": {"workload": "configs[3]: decode step, ED=5120 N=16 batch 64, 256 tokens per bench step",
                    "algorithmic_bytes_per_token_step": bytes_step},
-        "roofline": {"bound": "hbm", "kernel": "ssm_step_kernel", "achieved": bytes_step / t_kernel / 1e9,
+        "roofline": {"bound": "hbm", "kernel": "ssm_step_quad_kernel", "achieved": bytes_step / t_kernel / 1e9,
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": bytes_step / t_kernel / 1e9 / HBM_PEAK_GBS,
                      "traffic": None},
+    }
+    print(json.dumps(out))
+
+
+def bench_pscan(args, torch, pkg, dev):
+    """Generic PScan.apply(A, X) on materialised (B, L, ED, N) operands at the configs[1]
+    shape, fp32: forward moves 3 tensors, backward 5."""
+    B, L, ED, N = 8, 2048, 1536, 16
+    g = torch.Generator().manual_seed(1005)
+    A = (torch.rand(B, L, ED, N, generator=g) * 0.5 + 0.5).to(dev).requires_grad_()
+    X = torch.randn(B, L, ED, N, generator=g).to(dev).requires_grad_()
+    gH = torch.randn(B, L, ED, N, generator=g).to(dev)
+    steps, warmup = max(3, args.steps // 5), 2
+
+    def step(ev=None):
+        A.grad = None
+        X.grad = None
+        if ev:
+            ev[0].record()
+        H = pkg.pscan(A, X)
+        if ev:
+            ev[1].record()
+        H.backward(gH)
+        if ev:
+            ev[2].record()
+
+    t = _timed(torch, step, steps, warmup)
+    evs = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(steps)]
+    for ev in evs:
+        step(ev)
+    torch.cuda.synchronize()
+    fwd_ms = sum(e[0].elapsed_time(e[1]) for e in evs) / steps
+    bwd_ms = sum(e[1].elapsed_time(e[2]) for e in evs) / steps
+    S = B * L * ED * N * 4
+    out = {
+        "metric": "generic pscan(A, X) fwd+bwd GB/s, (8, 2048, 1536, 16) fp32",
+        "value": 8 * S / t / 1e9, "unit": "GB/s", "higher_is_better": True,
+        "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": t * 1e3,
+        "fwd_ms": fwd_ms, "bwd_ms": bwd_ms,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic (seeded)",
+        "config": {"workload": "PScan.apply on materialised operands, configs[1] shape",
+                   "algorithmic_bytes_fwd": 3 * S, "algorithmic_bytes_bwd": 5 * S},
+        "roofline": {"bound": "hbm", "kernel": "pscan_bwd_kernel", "achieved": 5 * S / (bwd_ms * 1e-3) / 1e9,
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": 5 * S / (bwd_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                     "traffic": None},
+        "forward": {"kernel": "pscan_fwd_kernel", "achieved": 3 * S / (fwd_ms * 1e-3) / 1e9, "unit": "GB/s",
+                    "frac": 3 * S / (fwd_ms * 1e-3) / 1e9 / HBM_PEAK_GBS},
     }
     print(json.dumps(out))
 
@@ -169,7 +216,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS) + ["c3", "c4", "c4-3000"],
+    ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS) + ["c3", "c4", "c4-3000", "pscan"],
                     help="c2 (default) is the headline workload; c3 = decode step, c4 = LM forward "
                          "(reported with their own metric, same one-line schema)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -191,6 +238,8 @@ def main():
 
     if args.workload == "c3":
         return bench_decode(args, torch, pkg, dev)
+    if args.workload == "pscan":
+        return bench_pscan(args, torch, pkg, dev)
     if args.workload.startswith("c4"):
         return bench_lm_forward(args, torch, pkg, dev, 3000 if args.workload == "c4-3000" else 4096)
 
