@@ -90,12 +90,15 @@ const char* mpa_status_string(int status);
  *            gradient is needed.
  *   h_last   optional (batch, dim, dstate) float32: state after the last step, in the
  *            layout of the decode cache `h` (mamba.py:335, 341).
+ *   y_pregate  optional, only with z: the output before the gate (C.h + D*x), io_dtype, strides
+ *            of y.  mpa_sscan_bwd needs it on its fast path; NULL when no gradient is needed.
  *   workspace  scratch of mpa_sscan_fwd_workspace_bytes() bytes.
  */
 int mpa_sscan_fwd(const mpa_sscan_shape* s, const void* x, const void* delta, const float* A,
                   const void* B, const void* C, const float* D, const void* z,
-                  const float* delta_bias, const float* h0, void* y, float* h_ckpt,
-                  float* h_last, void* workspace, size_t workspace_bytes, void* stream);
+                  const float* delta_bias, const float* h0, void* y, void* y_pregate,
+                  float* h_ckpt, float* h_last, void* workspace, size_t workspace_bytes,
+                  void* stream);
 
 /* Number of float32 elements of the h_ckpt buffer for this shape. */
 int64_t mpa_sscan_ckpt_elems(const mpa_sscan_shape* s);
@@ -113,12 +116,14 @@ size_t mpa_sscan_fwd_workspace_bytes(const mpa_sscan_shape* s);
  * MPA_SSCAN_DELTA_SOFTPLUS and h0 must be the ones given to the forward call; dz (io_dtype,
  * u-strides of g_*) is required when z is given, ddelta is then the gradient w.r.t. the
  * raw (pre-softplus) delta, and ddelta_bias (dim) float32 is written when delta_bias is
- * given.  `workspace` needs mpa_sscan_bwd_workspace_bytes() bytes, 256-byte aligned.
+ * given.  y_pregate (strides of dy) is what the forward call wrote for the same inputs; with z
+ * and y_pregate == NULL the pre-gate output is recomputed by a slower, more general kernel.
+ * `workspace` needs mpa_sscan_bwd_workspace_bytes() bytes, 256-byte aligned.
  */
 int mpa_sscan_bwd(const mpa_sscan_shape* s, const void* x, const void* delta, const float* A,
                   const void* B, const void* C, const float* D, const void* z,
                   const float* delta_bias, const float* h0, const void* dy,
-                  const float* h_ckpt, void* dx, void* ddelta, float* dA, void* dB, void* dC,
+                  const void* y_pregate, const float* h_ckpt, void* dx, void* ddelta, float* dA, void* dB, void* dC,
                   float* dD, void* dz, float* ddelta_bias, void* workspace,
                   size_t workspace_bytes, void* stream);
 

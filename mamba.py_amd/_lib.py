@@ -55,12 +55,12 @@ def load():
     lib.mpa_status_string.restype = ctypes.c_char_p
     lib.mpa_status_string.argtypes = [ctypes.c_int]
     sp = ctypes.POINTER(SscanShape)
-    lib.mpa_sscan_fwd.argtypes = [sp] + [vp] * 13 + [sz, vp]
+    lib.mpa_sscan_fwd.argtypes = [sp] + [vp] * 14 + [sz, vp]
     lib.mpa_sscan_fwd_workspace_bytes.argtypes = [sp]
     lib.mpa_sscan_fwd_workspace_bytes.restype = sz
     lib.mpa_sscan_ckpt_elems.argtypes = [sp]
     lib.mpa_sscan_ckpt_elems.restype = i64
-    lib.mpa_sscan_bwd.argtypes = [sp] + [vp] * 20 + [sz, vp]
+    lib.mpa_sscan_bwd.argtypes = [sp] + [vp] * 21 + [sz, vp]
     lib.mpa_sscan_bwd_workspace_bytes.argtypes = [sp]
     lib.mpa_sscan_bwd_workspace_bytes.restype = sz
     pp = ctypes.POINTER(PscanShape)

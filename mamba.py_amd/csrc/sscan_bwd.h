@@ -12,6 +12,7 @@ struct BwdParams {
     const void* C;
     const void* z;
     const void* dy;
+    const void* ypre;  // output before the gate saved by the forward (strides of dy); fast path with z
     const float* A;
     const float* D;
     const float* dbias;

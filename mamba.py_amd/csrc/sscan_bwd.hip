@@ -471,7 +471,8 @@ extern "C" size_t mpa_sscan_bwd_workspace_bytes(const mpa_sscan_shape* s) {
 extern "C" int mpa_sscan_bwd(const mpa_sscan_shape* s, const void* x, const void* delta,
                              const float* A, const void* B, const void* C, const float* D,
                              const void* z, const float* delta_bias, const float* h0,
-                             const void* dy, const float* h_ckpt, void* dx, void* ddelta,
+                             const void* dy, const void* y_pregate, const float* h_ckpt, void* dx,
+                             void* ddelta,
                              float* dA, void* dB, void* dC, float* dD, void* dz,
                              float* ddelta_bias, void* workspace, size_t workspace_bytes,
                              void* stream) {
@@ -489,7 +490,8 @@ extern "C" int mpa_sscan_bwd(const mpa_sscan_shape* s, const void* x, const void
     if (!aligned_to(x, es) || !aligned_to(delta, es) || !aligned_to(B, es) || !aligned_to(C, es) ||
         !aligned_to(dy, es) || !aligned_to(dx, es) || !aligned_to(ddelta, es) ||
         !aligned_to(dB, es) || !aligned_to(dC, es) || (z && !aligned_to(z, es)) ||
-        (dz && !aligned_to(dz, es)) || !aligned_to(workspace, 256))
+        (dz && !aligned_to(dz, es)) || (y_pregate && !aligned_to(y_pregate, es)) ||
+        !aligned_to(workspace, 256))
         return MPA_ERR_MISALIGNED;
     const BwdWorkspace ws = bwd_workspace(s);
     if (workspace_bytes < ws.total) return MPA_ERR_WORKSPACE;
@@ -497,6 +499,7 @@ extern "C" int mpa_sscan_bwd(const mpa_sscan_shape* s, const void* x, const void
     float* wsf = static_cast<float*>(workspace);
     BwdParams p{};
     p.x = x; p.delta = delta; p.Bm = B; p.C = C; p.z = z; p.dy = dy; p.A = A; p.D = D;
+    p.ypre = z ? y_pregate : nullptr;
     p.dbias = delta_bias; p.h0 = h0; p.ckpt = h_ckpt; p.dx = dx; p.ddelta = ddelta; p.dz = dz;
     p.partB = wsf + ws.offB; p.partC = wsf + ws.offC; p.partA = wsf + ws.offA;
     p.partD = wsf + ws.offD; p.partDb = wsf + ws.offDb;
@@ -517,7 +520,7 @@ extern "C" int mpa_sscan_bwd(const mpa_sscan_shape* s, const void* x, const void
     const int nw = np / ns;
     hipStream_t st = static_cast<hipStream_t>(stream);
     const char* force_general = getenv("MPA_BWD_GENERAL");
-    if (!z && bwd_fast_supported(ns, nw) && !(force_general && force_general[0] == '1')) {
+    if ((!z || p.ypre) && bwd_fast_supported(ns, nw) && !(force_general && force_general[0] == '1')) {
         rc = launch_bwd_fast(p, ns, nw, s->io_dtype, st);
     } else if (s->io_dtype == MPA_F32)
         rc = z ? dispatch_bwd<float, true>(p, ns, nw, st) : dispatch_bwd<float, false>(p, ns, nw, st);

@@ -1,4 +1,4 @@
-// Fused selective-scan backward for gfx950, fast path (no output gate).
+// Fused selective-scan backward for gfx950, fast path.
 //
 // A workgroup owns 64 channels of one batch row and walks the sequence from the last tile of
 // kTile steps to the first.
@@ -106,7 +106,10 @@ struct BwdFastLds {
         (kInputs + 2 * NW) * kTileF + 2 * kTile * 2 * NP + 2 * 2 * NP * kTile + 4;
 };
 
-template <typename IO, int NS, int NW>
+// HAS_Z: the forward multiplied its output by silu(z).  The service waves then read z and the
+// saved pre-gate output next to dy, publish dy*silu(z) as the dy tile (everything downstream is
+// unchanged) and store dz = dy * y_pre * d silu(z)/dz.
+template <typename IO, int NS, int NW, bool HAS_Z>
 __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(const BwdParams p) {
     constexpr int NP = NS * NW;
     constexpr int NQ = kTile / 4;
@@ -162,11 +165,15 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
         const IO* const xg = static_cast<const IO*>(p.x) + (b * p.u_sb + (int64_t)d0 * p.u_sd);
         const IO* const dg = static_cast<const IO*>(p.delta) + (b * p.d_sb + (int64_t)d0 * p.d_sd);
         const IO* const yg = static_cast<const IO*>(p.dy) + (b * p.y_sb + (int64_t)d0 * p.y_sd);
+        const IO* const zg = static_cast<const IO*>(p.z) + (b * p.u_sb + (int64_t)d0 * p.u_sd);
+        const IO* const ypg = static_cast<const IO*>(p.ypre) + (b * p.y_sb + (int64_t)d0 * p.y_sd);
+        IO* const dzg = static_cast<IO*>(p.dz) + (b * p.g_sb + (int64_t)d0 * p.g_sd);
         const IO* const Bg = static_cast<const IO*>(p.Bm) + b * p.bc_sb;
         const IO* const Cg = static_cast<const IO*>(p.C) + b * p.bc_sb;
-        uint32_t offx[4], offd[4], offy[4];
+        uint32_t offx[4], offd[4], offy[4], offz[4];  // offz: dz, addressed like dx
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
+            offz[j] = ((uint32_t)(4 * qi + j) * (uint32_t)p.g_sl + (uint32_t)cic * (uint32_t)p.g_sd) * kES;
             // byte offsets (see ld_off)
             offx[j] = ((uint32_t)(4 * qi + j) * (uint32_t)p.u_sl + (uint32_t)cic * (uint32_t)p.u_sd) * kES;
             offd[j] = ((uint32_t)(4 * qi + j) * (uint32_t)p.d_sl + (uint32_t)cic * (uint32_t)p.d_sd) * kES;
@@ -212,7 +219,7 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
 
         // Raw values of three tiles in flight (see the forward kernel: HBM latency under load
         // is longer than one tile interval)
-        struct Raw { IO x[4], d[4], y[4], b[kBcPer], c[kBcPer]; };
+        struct Raw { IO x[4], d[4], y[4], z[HAS_Z ? 4 : 1], yp[HAS_Z ? 4 : 1], b[kBcPer], c[kBcPer]; };
         auto load_tile = [&](int kk, Raw& raw) {
             // tiles and steps beyond the sequence are clamped, so the loads stay in bounds;
             // only the offsets depend on the (uniform) branch, the loads are unconditional
@@ -221,6 +228,8 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
             const IO* xk = xg + (int64_t)c * kTile * p.u_sl;
             const IO* dk = dg + (int64_t)c * kTile * p.d_sl;
             const IO* yk = yg + (int64_t)c * kTile * p.y_sl;
+            const IO* zk = zg + (int64_t)c * kTile * p.u_sl;
+            const IO* ypk = ypg + (int64_t)c * kTile * p.y_sl;
             const IO* Bk = Bg + (int64_t)c * kTile * p.bc_sl;
             const IO* Ck = Cg + (int64_t)c * kTile * p.bc_sl;
             uint32_t ox[4], od[4], oy[4], ob[kBcPer];
@@ -250,6 +259,10 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
                 raw.x[j] = ld_off(xk, ox[j]);
                 raw.d[j] = ld_off(dk, od[j]);
                 raw.y[j] = ld_off(yk, oy[j]);
+                if constexpr (HAS_Z) {
+                    raw.z[j] = ld_off(zk, ox[j]);
+                    raw.yp[j] = ld_off(ypk, oy[j]);
+                }
             }
 #pragma unroll
             for (int r = 0; r < kBcPer; ++r) {
@@ -270,7 +283,30 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
 #pragma unroll
                 for (int j = 0; j < 4; ++j) dv[j] = softplus_f(dv[j] + bias);
             }
-            if (!group_full || (c + 1) * kTile > p.L) {
+            float dzv[4];
+            if constexpr (HAS_Z) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const float zv = to_float(raw.z[j]);
+                    const float sg = sigmoid_f(zv);
+                    // d/dz (z*sigmoid(z)) = sigmoid(z) * (1 + z*(1 - sigmoid(z)))
+                    dzv[j] = yv[j] * to_float(raw.yp[j]) * sg * __builtin_fmaf(zv, 1.0f - sg, 1.0f);
+                    yv[j] *= zv * sg;
+                }
+            }
+            const bool ragged = !group_full || (c + 1) * kTile > p.L;
+            if constexpr (HAS_Z) {
+                IO* dzk = dzg + (int64_t)c * kTile * p.g_sl;
+                if (!ragged) {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) st_off(dzk, offz[j], from_float<IO>(dzv[j]));
+                } else {
+                    const int t0 = c * kTile + 4 * qi;
+                    for (int j = 0; j < 4; ++j)
+                        if (ci_ok && t0 + j < p.L) st_off(dzk, offz[j], from_float<IO>(dzv[j]));
+                }
+            }
+            if (ragged) {
                 // padding (beyond the sequence or the channel count): delta = 0, u = 0, dy = 0
                 // make the step an exact no-op in both sweeps
                 const int t0 = c * kTile + 4 * qi;
@@ -629,25 +665,29 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
     __syncthreads();  // final
 }
 
-template <typename IO, int NS, int NW>
+template <typename IO, int NS, int NW, bool HAS_Z>
 static int launch_fast(const BwdParams& p, hipStream_t stream) {
     dim3 grid((p.ED + kWave - 1) / kWave, p.batch);
     dim3 block((NW + kSvc) * kWave);
     constexpr size_t lds = sizeof(float) * BwdFastLds<NS, NW>::floats;
     static_assert(lds <= 160 * 1024, "LDS budget");
-    static const int attr_rc = allow_dynamic_lds(sscan_bwd_fast_kernel<IO, NS, NW>, lds);
+    static const int attr_rc = allow_dynamic_lds(sscan_bwd_fast_kernel<IO, NS, NW, HAS_Z>, lds);
     if (attr_rc != MPA_OK) return attr_rc;
-    hipLaunchKernelGGL((sscan_bwd_fast_kernel<IO, NS, NW>), grid, block, lds, stream, p);
+    hipLaunchKernelGGL((sscan_bwd_fast_kernel<IO, NS, NW, HAS_Z>), grid, block, lds, stream, p);
     return check_launch();
 }
 
 bool bwd_fast_supported(int ns, int nw) { return (ns == 2 && nw == 8) || (ns == 4 && nw == 4); }
 
 int launch_bwd_fast(const BwdParams& p, int ns, int nw, int io_dtype, hipStream_t stream) {
-#define MPA_CASE(NS_, NW_)                                                   \
-    if (ns == NS_ && nw == NW_)                                              \
-        return io_dtype == MPA_F32 ? launch_fast<float, NS_, NW_>(p, stream) \
-                                   : launch_fast<bf16_t, NS_, NW_>(p, stream);
+#define MPA_CASE(NS_, NW_)                                                                \
+    if (ns == NS_ && nw == NW_) {                                                         \
+        if (p.z)                                                                          \
+            return io_dtype == MPA_F32 ? launch_fast<float, NS_, NW_, true>(p, stream)    \
+                                       : launch_fast<bf16_t, NS_, NW_, true>(p, stream);  \
+        return io_dtype == MPA_F32 ? launch_fast<float, NS_, NW_, false>(p, stream)       \
+                                   : launch_fast<bf16_t, NS_, NW_, false>(p, stream);     \
+    }
     MPA_CASE(2, 8) MPA_CASE(4, 4)
 #undef MPA_CASE
     return MPA_ERR_BAD_SHAPE;

@@ -41,6 +41,7 @@ struct FwdParams {
     const void* C;
     int64_t bc_sb, bc_sl;
     void* y;
+    void* ypre;  // output before the gate (only with z), strides of y
     float* ckpt;
     float* hlast;
     int batch, L, ED, N, nchunks;
@@ -354,20 +355,27 @@ __global__ void __launch_bounds__((NW + kService) * kWave) sscan_fwd_kernel(cons
             for (int j = 0; j < 4; ++j)
                 offy[j] = ((uint32_t)(q4 + j) * (uint32_t)p.y_sl + (uint32_t)min(co, cmax) * (uint32_t)p.y_sd) * kES;
             IO* const yg = static_cast<IO*>(p.y) + (b * p.y_sb + (int64_t)d0 * p.y_sd);
+            IO* const ypg = static_cast<IO*>(p.ypre) + (b * p.y_sb + (int64_t)d0 * p.y_sd);
             auto reduce_store = [&](int k) {
                 IO* yk = yg + (int64_t)k * kTile * p.y_sl;
+                IO* ypk = ypg + (int64_t)k * kTile * p.y_sl;
                 float4 s = *reinterpret_cast<const float4*>(&sDx[k & 3][co][q4]);
 #pragma unroll
                 for (int ww = 0; ww < NW; ++ww) {
                     const float4 v = *reinterpret_cast<const float4*>(&sY[(k & 1) * NW + ww][co][q4]);
                     s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
                 }
+                const int t0 = k * kTile + q4;
                 if (has_z) {
+                    if (p.ypre) {
+                        const float pv[4] = {s.x, s.y, s.z, s.w};
+                        for (int j = 0; j < 4; ++j)
+                            if (co_ok && t0 + j < p.L) st_off(ypk, offy[j], from_float<IO>(pv[j]));
+                    }
                     const float4 g = *reinterpret_cast<const float4*>(&sG[k & 3][co][q4]);
                     s.x *= g.x; s.y *= g.y; s.z *= g.z; s.w *= g.w;
                 }
                 const float sv[4] = {s.x, s.y, s.z, s.w};
-                const int t0 = k * kTile + q4;
                 if (co_ok && t0 + 3 < p.L) {
 #pragma unroll
                     for (int j = 0; j < 4; ++j) st_off(yk, offy[j], from_float<IO>(sv[j]));
@@ -653,7 +661,7 @@ extern "C" size_t mpa_sscan_fwd_workspace_bytes(const mpa_sscan_shape* s) {
 extern "C" int mpa_sscan_fwd(const mpa_sscan_shape* s, const void* x, const void* delta,
                              const float* A, const void* B, const void* C, const float* D,
                              const void* z, const float* delta_bias, const float* h0, void* y,
-                             float* h_ckpt, float* h_last, void* workspace,
+                             void* y_pregate, float* h_ckpt, float* h_last, void* workspace,
                              size_t workspace_bytes, void* stream) {
     int rc = validate_shape(s);
     if (rc != MPA_OK) return rc;
@@ -662,7 +670,7 @@ extern "C" int mpa_sscan_fwd(const mpa_sscan_shape* s, const void* x, const void
     if (!softplus && delta_bias) return MPA_ERR_BAD_SHAPE;
     const size_t es = dtype_size(s->io_dtype);
     if (!aligned_to(x, es) || !aligned_to(delta, es) || !aligned_to(B, es) || !aligned_to(C, es) ||
-        !aligned_to(y, es) || (z && !aligned_to(z, es)) || !aligned_to(A, 4) || !aligned_to(D, 4) ||
+        !aligned_to(y, es) || (z && !aligned_to(z, es)) || (y_pregate && !aligned_to(y_pregate, es)) || !aligned_to(A, 4) || !aligned_to(D, 4) ||
         !aligned_to(workspace, 256))
         return MPA_ERR_MISALIGNED;
     if (workspace_bytes < mpa_sscan_fwd_workspace_bytes(s)) return MPA_ERR_WORKSPACE;
@@ -681,7 +689,7 @@ extern "C" int mpa_sscan_fwd(const mpa_sscan_shape* s, const void* x, const void
     p.x = x; p.delta = delta; p.z = z; p.A = A; p.D = D;
     p.dbias = delta_bias; p.h0 = h0; p.bcpack = static_cast<const float*>(workspace);
     p.Bm = B; p.C = C; p.bc_sb = s->bc_sb; p.bc_sl = s->bc_sl;
-    p.y = y; p.ckpt = h_ckpt; p.hlast = h_last;
+    p.y = y; p.ypre = z ? y_pregate : nullptr; p.ckpt = h_ckpt; p.hlast = h_last;
     p.batch = (int)s->batch; p.L = (int)s->seqlen; p.ED = (int)s->dim; p.N = (int)s->dstate;
     p.nchunks = (p.L + kTile - 1) / kTile;
     p.softplus = softplus ? 1 : 0;

@@ -103,10 +103,12 @@ class SelectiveScanFn(torch.autograd.Function):
                         for t in (x, delta, A, B, C, D, z, delta_bias))
         flags = _lib.MPA_SSCAN_DELTA_SOFTPLUS if delta_softplus else 0
         shape = _sscan_shape(x_, delta_, B_, y, y, B_, N, flags)
-        ckpt = None
+        ckpt = y_pre = None
         if need_grad:
             ckpt = torch.empty(lib.mpa_sscan_ckpt_elems(ctypes.byref(shape)), dtype=torch.float32,
                                device=x.device)
+            if z_ is not None:
+                y_pre = torch.empty_like(y)  # output before the gate, read again by the backward
         h_last = torch.empty((Bsz, ED, N), dtype=torch.float32, device=x.device) \
             if return_last_state else None
         nbytes = lib.mpa_sscan_fwd_workspace_bytes(ctypes.byref(shape))
@@ -114,9 +116,10 @@ class SelectiveScanFn(torch.autograd.Function):
         with torch.cuda.device(x.device):
             rc = lib.mpa_sscan_fwd(ctypes.byref(shape), _ptr(x_), _ptr(delta_), _ptr(A_), _ptr(B_),
                                    _ptr(C_), _ptr(D_), _ptr(z_), _ptr(bias_), _ptr(h0_), _ptr(y),
-                                   _ptr(ckpt), _ptr(h_last), _ptr(ws), nbytes, _stream(x.device))
+                                   _ptr(y_pre), _ptr(ckpt), _ptr(h_last), _ptr(ws), nbytes,
+                                   _stream(x.device))
         _lib.check(rc, "mpa_sscan_fwd")
-        ctx.save_for_backward(x_, delta_, A_, B_, C_, D_, z_, bias_, h0_, ckpt)
+        ctx.save_for_backward(x_, delta_, A_, B_, C_, D_, z_, bias_, h0_, ckpt, y_pre)
         ctx.flags = flags
         ctx.in_dtypes = (x.dtype, delta.dtype, A.dtype, B.dtype, C.dtype, D.dtype,
                          None if z is None else z.dtype,
@@ -129,13 +132,15 @@ class SelectiveScanFn(torch.autograd.Function):
     @staticmethod
     def backward(ctx, dy, *unused):
         lib = _lib.load()
-        x, delta, A, B, C, D, z, bias, h0, ckpt = ctx.saved_tensors
+        x, delta, A, B, C, D, z, bias, h0, ckpt, y_pre = ctx.saved_tensors
         if ckpt is None:
             raise RuntimeError("backward called on a selective scan that saved no checkpoints")
         dt = x.dtype
         Bsz, L, ED = x.shape
         N = A.shape[-1]
         dy = dy.to(dt)
+        if y_pre is not None and dy.stride() != y_pre.stride():
+            dy = dy.contiguous()  # the saved pre-gate output is addressed with dy's strides
         dx = torch.empty((Bsz, L, ED), dtype=dt, device=x.device)
         ddelta = torch.empty_like(dx)
         dz = torch.empty_like(dx) if z is not None else None
@@ -150,7 +155,7 @@ class SelectiveScanFn(torch.autograd.Function):
         with torch.cuda.device(x.device):
             rc = lib.mpa_sscan_bwd(ctypes.byref(shape), _ptr(x), _ptr(delta), _ptr(A), _ptr(B),
                                    _ptr(C), _ptr(D), _ptr(z), _ptr(bias), _ptr(h0), _ptr(dy),
-                                   _ptr(ckpt), _ptr(dx), _ptr(ddelta), _ptr(dA), _ptr(dB), _ptr(dC),
+                                   _ptr(y_pre), _ptr(ckpt), _ptr(dx), _ptr(ddelta), _ptr(dA), _ptr(dB), _ptr(dC),
                                    _ptr(dD), _ptr(dz), _ptr(dbias), _ptr(ws), nbytes,
                                    _stream(x.device))
         _lib.check(rc, "mpa_sscan_bwd")

@@ -36,15 +36,15 @@ def test_status_codes_without_launch(pkg):
     L = pkg._lib
     lib = L.load()
     s = L.SscanShape()
-    assert lib.mpa_sscan_fwd(None, *([None] * 13), 0, None) == 1          # MPA_ERR_NULL_POINTER
+    assert lib.mpa_sscan_fwd(None, *([None] * 14), 0, None) == 1          # MPA_ERR_NULL_POINTER
     s.batch, s.seqlen, s.dim, s.dstate = 1, 0, 8, 16
-    assert lib.mpa_sscan_fwd(ctypes.byref(s), *([None] * 13), 0, None) == 2  # bad shape
+    assert lib.mpa_sscan_fwd(ctypes.byref(s), *([None] * 14), 0, None) == 2  # bad shape
     s.seqlen, s.dstate = 8, 1000
-    assert lib.mpa_sscan_fwd(ctypes.byref(s), *([None] * 13), 0, None) == 2  # d_state too large
+    assert lib.mpa_sscan_fwd(ctypes.byref(s), *([None] * 14), 0, None) == 2  # d_state too large
     s.dstate, s.io_dtype = 16, 7
-    assert lib.mpa_sscan_fwd(ctypes.byref(s), *([None] * 13), 0, None) == 3  # bad dtype
+    assert lib.mpa_sscan_fwd(ctypes.byref(s), *([None] * 14), 0, None) == 3  # bad dtype
     s.io_dtype = 0
-    assert lib.mpa_sscan_fwd(ctypes.byref(s), *([None] * 13), 0, None) == 1  # null data pointers
+    assert lib.mpa_sscan_fwd(ctypes.byref(s), *([None] * 14), 0, None) == 1  # null data pointers
     assert lib.mpa_sscan_ckpt_elems(ctypes.byref(s)) == 1 * 1 * 16 * 8
     assert lib.mpa_sscan_bwd_workspace_bytes(ctypes.byref(s)) > 0
     assert lib.mpa_status_string(6) == b"workspace too small"

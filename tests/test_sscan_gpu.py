@@ -144,6 +144,55 @@ def test_gate_softplus_bias_h0_and_last_state(pkg, dev):
         assert e <= TOL[torch.float32], f"{k}: {e:.3e}"
 
 
+
+def _gated_case(pkg, dev, Bs, L, ED, N, dtype, seed, tmajor=False):
+    inp = so.make_inputs(Bs, L, ED, N, seed=seed, dtype=dtype)
+    g = torch.Generator().manual_seed(seed + 1)
+    z = torch.randn(Bs, L, ED, generator=g).to(dtype)
+    f64 = lambda t: t.double().requires_grad_()
+    names = ("x", "delta", "A", "B", "C", "D")
+    ref_in = [f64(inp[k]) for k in names] + [f64(z)]
+    yr = so.selective_scan_ref(*ref_in[:6]) * (ref_in[6] * torch.sigmoid(ref_in[6]))
+    yr.backward(inp["dy"].double())
+    ref = dict(y=yr, dz=ref_in[6].grad, **{k: a.grad for k, a in zip(GRAD_KEYS, ref_in)})
+
+    def to_dev(t):
+        t = t.to(dev)
+        if tmajor and t.dim() == 3 and t.shape[-1] == ED:
+            t = t.transpose(1, 2).contiguous().transpose(1, 2)  # (B, ED, L) memory
+        return t.requires_grad_()
+
+    gin = [to_dev(inp[k]) for k in names] + [to_dev(z)]
+    y = pkg.selective_scan_fn(*gin[:6], z=gin[6])
+    y.backward(inp["dy"].to(dev))
+    got = dict(y=y, dz=gin[6].grad, **{k: a.grad for k, a in zip(GRAD_KEYS, gin)})
+    return got, ref
+
+
+@pytest.mark.parametrize("Bs,L,ED,N", [(2, 64, 64, 16), (1, 37, 70, 16), (3, 129, 200, 12)])
+def test_gated_backward_fast_path_fp32(pkg, dev, Bs, L, ED, N):
+    got, ref = _gated_case(pkg, dev, Bs, L, ED, N, torch.float32, 300 + L)
+    for k in ref:
+        e = rel_err(got[k], ref[k])
+        assert e <= TOL[torch.float32], f"{k}: {e:.3e}"
+
+
+def test_gated_backward_bf16_and_time_contiguous(pkg, dev):
+    got, ref = _gated_case(pkg, dev, 2, 100, 96, 16, torch.bfloat16, 311, tmajor=True)
+    for k in ref:
+        e = rel_err(got[k], ref[k])
+        assert e <= TOL[torch.bfloat16], f"{k}: {e:.3e}"
+
+
+def test_gated_backward_fast_equals_general_kernel(pkg, dev, monkeypatch):
+    # the two backward kernels (saved pre-gate output vs recomputed one) must agree
+    a, _ = _gated_case(pkg, dev, 2, 80, 128, 16, torch.float32, 321)
+    monkeypatch.setenv("MPA_BWD_GENERAL", "1")
+    b, _ = _gated_case(pkg, dev, 2, 80, 128, 16, torch.float32, 321)
+    for k in a:
+        assert rel_err(a[k], b[k]) <= 2e-6, k
+
+
 def test_bitwise_reproducible(pkg, dev):
     inp = so.make_inputs(2, 130, 200, 16, seed=61)
     a = run_gpu_fwd_bwd(pkg, inp, dev)
