@@ -129,6 +129,39 @@ int mpa_sscan_bwd(const mpa_sscan_shape* s, const void* x, const void* delta, co
 
 size_t mpa_sscan_bwd_workspace_bytes(const mpa_sscan_shape* s);
 
+/* ---- causal depthwise convolution along time (+ bias, + SiLU) ------------------------------
+ * Replaces, in MambaBlock.forward (mambapy/mamba.py:217-221),
+ *     x.transpose(1,2) -> Conv1d(ED, ED, kernel, groups=ED, padding=kernel-1)(.)[:, :, :L]
+ *       -> transpose(1,2) -> silu
+ * on the (batch, seqlen, dim) tensor directly (any element strides: the caller passes the x half
+ * of the in_proj output, mamba.py:213-214, without a copy), and its gradient.  weight is the
+ * Conv1d weight (dim, 1, kernel) viewed as (dim, kernel) float32, bias (dim) float32 or NULL.
+ * window_in  optional (batch, dim, kernel-1), io_dtype: the inputs before step 0 (the decode
+ *            cache of mamba.py:344-346, 379), NULL = zeros (the reference's left padding).
+ * window_out optional (batch, dim, kernel-1): the last kernel-1 inputs, i.e. the cache to
+ *            continue from with MambaBlock.step.
+ * y has the y_* strides, dy too; dx the g_* strides; dweight (dim, kernel), dbias (dim) float32,
+ * overwritten.  No gradient flows into window_in.
+ */
+#define MPA_CONV_SILU 1
+typedef struct mpa_conv_shape {
+    int64_t batch, seqlen, dim;
+    int32_t kernel;   /* d_conv, 2..4 */
+    int32_t io_dtype; /* enum mpa_dtype */
+    int32_t flags;    /* bit set of MPA_CONV_* */
+    int32_t reserved;
+    int64_t x_sb, x_sl, x_sd;
+    int64_t y_sb, y_sl, y_sd;
+    int64_t g_sb, g_sl, g_sd;
+} mpa_conv_shape;
+
+int mpa_conv1d_fwd(const mpa_conv_shape* s, const void* x, const float* weight, const float* bias,
+                   const void* window_in, void* y, void* window_out, void* stream);
+int mpa_conv1d_bwd(const mpa_conv_shape* s, const void* x, const float* weight, const float* bias,
+                   const void* window_in, const void* dy, void* dx, float* dweight, float* dbias,
+                   void* workspace, size_t workspace_bytes, void* stream);
+size_t mpa_conv1d_bwd_workspace_bytes(const mpa_conv_shape* s);
+
 /* ---- generic first-order scan -----------------------------------------------------------
  * Replaces pscan = PScan.apply (mambapy/pscan.py:226; forward :151-186, backward :188-224)
  * for callers that hold materialised A, X of logical shape (batch, seqlen, dim, dstate):

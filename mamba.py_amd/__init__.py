@@ -5,12 +5,13 @@ The directory is named `mamba.py_amd`; import it as `mambapy_amd` (see INTEGRATI
 """
 from . import _lib
 from .scan import PScan, pscan, selective_scan, selective_scan_fn, ssm_step, SelectiveScanFn
+from .conv import CausalConv1dFn, causal_conv1d_fn
 from .modules import Mamba, MambaBlock, MambaConfig, ResidualBlock, RMSNorm
 from .language_model import LM
 from .patch import patch_mambapy
 
 __all__ = ["PScan", "pscan", "selective_scan", "selective_scan_fn", "ssm_step",
-           "SelectiveScanFn", "Mamba", "MambaBlock", "MambaConfig", "ResidualBlock", "RMSNorm",
+           "SelectiveScanFn", "CausalConv1dFn", "causal_conv1d_fn", "Mamba", "MambaBlock", "MambaConfig", "ResidualBlock", "RMSNorm",
            "LM", "patch_mambapy", "library_path", "library_version"]
 
 

@@ -11,12 +11,14 @@ LIB_PATH = os.path.join(_HERE, "csrc", "libmambapy_amd.so")
 
 MPA_F32, MPA_BF16 = 0, 1
 MPA_SSCAN_DELTA_SOFTPLUS = 1
+MPA_CONV_SILU = 1
 MPA_CKPT_STEPS = 16
 MPA_MAX_DSTATE = 256
 
 EXPORTS = ("mpa_version", "mpa_arch", "mpa_status_string", "mpa_sscan_fwd",
            "mpa_sscan_ckpt_elems", "mpa_sscan_fwd_workspace_bytes", "mpa_sscan_bwd", "mpa_sscan_bwd_workspace_bytes",
-           "mpa_pscan_fwd", "mpa_pscan_bwd", "mpa_ssm_step")
+           "mpa_pscan_fwd", "mpa_pscan_bwd", "mpa_ssm_step",
+           "mpa_conv1d_fwd", "mpa_conv1d_bwd", "mpa_conv1d_bwd_workspace_bytes")
 
 
 class SscanShape(ctypes.Structure):
@@ -25,6 +27,13 @@ class SscanShape(ctypes.Structure):
                [(n, ctypes.c_int64) for n in (
                    "u_sb", "u_sl", "u_sd", "d_sb", "d_sl", "d_sd", "y_sb", "y_sl", "y_sd",
                    "g_sb", "g_sl", "g_sd", "bc_sb", "bc_sl", "dbc_sb", "dbc_sl")]
+
+
+class ConvShape(ctypes.Structure):
+    _fields_ = [(n, ctypes.c_int64) for n in ("batch", "seqlen", "dim")] + \
+               [(n, ctypes.c_int32) for n in ("kernel", "io_dtype", "flags", "reserved")] + \
+               [(n, ctypes.c_int64) for n in (
+                   "x_sb", "x_sl", "x_sd", "y_sb", "y_sl", "y_sd", "g_sb", "g_sl", "g_sd")]
 
 
 class PscanShape(ctypes.Structure):
@@ -67,6 +76,11 @@ def load():
     lib.mpa_pscan_fwd.argtypes = [pp] + [vp] * 4
     lib.mpa_pscan_bwd.argtypes = [pp] + [vp] * 6
     lib.mpa_ssm_step.argtypes = [vp] * 11 + [i64] * 4 + [i32, i32, vp]
+    cp = ctypes.POINTER(ConvShape)
+    lib.mpa_conv1d_fwd.argtypes = [cp] + [vp] * 7
+    lib.mpa_conv1d_bwd.argtypes = [cp] + [vp] * 9 + [sz, vp]
+    lib.mpa_conv1d_bwd_workspace_bytes.argtypes = [cp]
+    lib.mpa_conv1d_bwd_workspace_bytes.restype = sz
     for name in EXPORTS:
         getattr(lib, name)
     _lib = lib

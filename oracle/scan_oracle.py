@@ -27,6 +27,9 @@ names the lines it follows.  What pins each function (see tests/test_oracle.py):
   ssm_step_ref           mambapy/mamba.py:400-412.  Pinned by "L steps == one scan".
   conv_window_step_ref   mambapy/mamba.py:366-367, 379.  Pinned against
                          torch.nn.functional.conv1d with left zero padding.
+  causal_conv1d_ref      mambapy/mamba.py:217-221.  Pinned against the definition written
+                         as explicit loops on small cases and against nn.Conv1d with
+                         padding=K-1 truncated to L (the reference's own expression).
 
 Floating-point rounding of torch's own elementwise kernels is not pinned by any
 reference fixture ("parity unpinned" at the torch boundary; irrelevant at the
@@ -293,6 +296,22 @@ def conv_window_step_ref(window, x_new, weight, bias):
     if bias is not None:
         out = out + bias
     return out, full[:, :, 1:].clone()
+
+
+def causal_conv1d_ref(x, weight, bias=None, window=None, silu=True):
+    """Depthwise causal convolution along time as MambaBlock.forward applies it
+    (mambapy/mamba.py:217-221): conv1d(x^T, padding=K-1)[:, :, :L]^T, then silu (:221).
+
+    x : (B, L, ED); weight : (ED, 1, K); bias : (ED) or None; window : optional (B, ED, K-1)
+    inputs that precede step 0 (the reference pads with zeros; the decode cache of
+    mamba.py:344-346 is the non-zero case).  Returns (B, L, ED).
+    """
+    K = weight.shape[-1]
+    xt = x.transpose(1, 2)                                            # (B, ED, L)
+    left = window if window is not None else xt.new_zeros(xt.shape[0], xt.shape[1], K - 1)
+    y = F.conv1d(torch.cat([left.to(xt.dtype), xt], dim=2), weight, bias, groups=xt.shape[1])
+    y = y.transpose(1, 2)
+    return F.silu(y) if silu else y
 
 
 def softplus_ref(v):

@@ -204,3 +204,32 @@ def test_softplus_ref_and_input_recipe():
     assert 5e-4 < inp["delta"].min().item() and inp["delta"].max().item() < 0.2
     assert torch.equal(inp["A"][0], -torch.arange(1, 17, dtype=torch.float32))
     assert torch.equal(inp["D"], torch.ones(64))
+
+
+def test_causal_conv1d_ref_against_explicit_loops_and_nn_conv1d():
+    # definition: y[b,t,d] = bias[d] + sum_k w[d,k] * x[b, t-(K-1)+k, d], inputs before step 0
+    # taken from `window` (zeros without one)  (mambapy/mamba.py:217-221, 344-346)
+    g = torch.Generator().manual_seed(5)
+    Bsz, L, ED, K = 2, 7, 3, 4
+    x = torch.randn(Bsz, L, ED, generator=g, dtype=torch.float64)
+    w = torch.randn(ED, 1, K, generator=g, dtype=torch.float64)
+    b = torch.randn(ED, generator=g, dtype=torch.float64)
+    win = torch.randn(Bsz, ED, K - 1, generator=g, dtype=torch.float64)
+    for window in (None, win):
+        want = torch.zeros(Bsz, L, ED, dtype=torch.float64)
+        for bb in range(Bsz):
+            for t in range(L):
+                for d in range(ED):
+                    acc = b[d].item()
+                    for k in range(K):
+                        src = t - (K - 1) + k
+                        if src >= 0:
+                            acc += w[d, 0, k].item() * x[bb, src, d].item()
+                        elif window is not None:
+                            acc += w[d, 0, k].item() * window[bb, d, src + K - 1].item()
+                    want[bb, t, d] = acc
+        got = so.causal_conv1d_ref(x, w, b, window, silu=False)
+        assert (got - want).abs().max().item() < 1e-12
+    conv = torch.nn.Conv1d(ED, ED, K, groups=ED, padding=K - 1).double()
+    ref = torch.nn.functional.silu(conv(x.transpose(1, 2))[:, :, :L].transpose(1, 2))
+    assert (so.causal_conv1d_ref(x, conv.weight, conv.bias) - ref).abs().max().item() < 1e-12
