@@ -48,7 +48,7 @@ enum mpa_dtype { MPA_F32 = 0, MPA_BF16 = 1 };
  *   x, delta, z, y, dy, dx, ddelta : (batch, seqlen, dim)      dim = ED = d_inner
  *   A : (dim, dstate) contiguous float32;  D, delta_bias : (dim) contiguous float32
  *   B, C, dB, dC : (batch, seqlen, dstate), innermost stride 1
- * u_* strides apply to x, z (inputs);  d_* to delta;  y_* to y, dy;  g_* to dx, ddelta;
+ * u_* strides apply to x;  z_* to z;  d_* to delta;  y_* to y, dy, y_pregate;  g_* to dx, ddelta, dz;
  * bc_* to B and C;  dbc_* to dB and dC.
  * The reference calls this path both with fresh channel-contiguous tensors
  * (tests/compare_seq_pscan.py:24-29: strides (L*ED, ED, 1)) and, from MambaBlock.forward,
@@ -60,6 +60,7 @@ typedef struct mpa_sscan_shape {
     int32_t io_dtype; /* enum mpa_dtype */
     int32_t flags;    /* bit set of MPA_SSCAN_* */
     int64_t u_sb, u_sl, u_sd;
+    int64_t z_sb, z_sl, z_sd;
     int64_t d_sb, d_sl, d_sd;
     int64_t y_sb, y_sl, y_sd;
     int64_t g_sb, g_sl, g_sd;

@@ -25,7 +25,7 @@ class SscanShape(ctypes.Structure):
     _fields_ = [(n, ctypes.c_int64) for n in ("batch", "seqlen", "dim", "dstate")] + \
                [("io_dtype", ctypes.c_int32), ("flags", ctypes.c_int32)] + \
                [(n, ctypes.c_int64) for n in (
-                   "u_sb", "u_sl", "u_sd", "d_sb", "d_sl", "d_sd", "y_sb", "y_sl", "y_sd",
+                   "u_sb", "u_sl", "u_sd", "z_sb", "z_sl", "z_sd", "d_sb", "d_sl", "d_sd", "y_sb", "y_sl", "y_sd",
                    "g_sb", "g_sl", "g_sd", "bc_sb", "bc_sl", "dbc_sb", "dbc_sl")]
 
 

@@ -30,6 +30,7 @@ struct BwdParams {
     int softplus;
     int in_tmajor, dy_tmajor, out_tmajor;
     int64_t u_sb, u_sl, u_sd;
+    int64_t z_sb, z_sl, z_sd;
     int64_t d_sb, d_sl, d_sd;
     int64_t y_sb, y_sl, y_sd;
     int64_t g_sb, g_sl, g_sd;

@@ -126,7 +126,7 @@ __global__ void __launch_bounds__(NW* kWave) sscan_bwd_kernel(const BwdParams p)
                 xv = load_as_float<IO>(p.x, b * p.u_sb + t * p.u_sl + ch * p.u_sd);
                 dv = load_as_float<IO>(p.delta, b * p.d_sb + t * p.d_sl + ch * p.d_sd);
                 dyv = load_as_float<IO>(p.dy, b * p.y_sb + t * p.y_sl + ch * p.y_sd);
-                if (HAS_Z) zv = load_as_float<IO>(p.z, b * p.u_sb + t * p.u_sl + ch * p.u_sd);
+                if (HAS_Z) zv = load_as_float<IO>(p.z, b * p.z_sb + t * p.z_sl + ch * p.z_sd);
             }
             rX[k] = xv;
             rDl[k] = dv;
@@ -326,7 +326,7 @@ __global__ void __launch_bounds__(NW* kWave) sscan_bwd_kernel(const BwdParams p)
                         for (int ww = 0; ww < NW; ++ww) yp += sP3[ww][ts][cc];
                         yp = __builtin_fmaf(Dv, xv, yp);  // pre-gate output
                         const float zv =
-                            load_as_float<IO>(p.z, b * p.u_sb + t * p.u_sl + ch * p.u_sd);
+                            load_as_float<IO>(p.z, b * p.z_sb + t * p.z_sl + ch * p.z_sd);
                         const float sg = sigmoid_f(zv);
                         const float dyraw = sZg[0][tt][cc];
                         // d(z*sigmoid(z))/dz = sg * (1 + z*(1-sg))
@@ -507,6 +507,7 @@ extern "C" int mpa_sscan_bwd(const mpa_sscan_shape* s, const void* x, const void
     p.nchunks = (p.L + kTile - 1) / kTile;
     p.softplus = softplus ? 1 : 0;
     p.u_sb = s->u_sb; p.u_sl = s->u_sl; p.u_sd = s->u_sd;
+    p.z_sb = s->z_sb; p.z_sl = s->z_sl; p.z_sd = s->z_sd;
     p.d_sb = s->d_sb; p.d_sl = s->d_sl; p.d_sd = s->d_sd;
     p.y_sb = s->y_sb; p.y_sl = s->y_sl; p.y_sd = s->y_sd;
     p.g_sb = s->g_sb; p.g_sl = s->g_sl; p.g_sd = s->g_sd;

@@ -165,15 +165,16 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
         const IO* const xg = static_cast<const IO*>(p.x) + (b * p.u_sb + (int64_t)d0 * p.u_sd);
         const IO* const dg = static_cast<const IO*>(p.delta) + (b * p.d_sb + (int64_t)d0 * p.d_sd);
         const IO* const yg = static_cast<const IO*>(p.dy) + (b * p.y_sb + (int64_t)d0 * p.y_sd);
-        const IO* const zg = static_cast<const IO*>(p.z) + (b * p.u_sb + (int64_t)d0 * p.u_sd);
+        const IO* const zg = static_cast<const IO*>(p.z) + (b * p.z_sb + (int64_t)d0 * p.z_sd);
         const IO* const ypg = static_cast<const IO*>(p.ypre) + (b * p.y_sb + (int64_t)d0 * p.y_sd);
         IO* const dzg = static_cast<IO*>(p.dz) + (b * p.g_sb + (int64_t)d0 * p.g_sd);
         const IO* const Bg = static_cast<const IO*>(p.Bm) + b * p.bc_sb;
         const IO* const Cg = static_cast<const IO*>(p.C) + b * p.bc_sb;
-        uint32_t offx[4], offd[4], offy[4], offz[4];  // offz: dz, addressed like dx
+        uint32_t offx[4], offd[4], offy[4], offz[4], offzi[4];  // offz: dz, addressed like dx; offzi: z
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             offz[j] = ((uint32_t)(4 * qi + j) * (uint32_t)p.g_sl + (uint32_t)cic * (uint32_t)p.g_sd) * kES;
+            offzi[j] = ((uint32_t)(4 * qi + j) * (uint32_t)p.z_sl + (uint32_t)cic * (uint32_t)p.z_sd) * kES;
             // byte offsets (see ld_off)
             offx[j] = ((uint32_t)(4 * qi + j) * (uint32_t)p.u_sl + (uint32_t)cic * (uint32_t)p.u_sd) * kES;
             offd[j] = ((uint32_t)(4 * qi + j) * (uint32_t)p.d_sl + (uint32_t)cic * (uint32_t)p.d_sd) * kES;
@@ -228,13 +229,14 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
             const IO* xk = xg + (int64_t)c * kTile * p.u_sl;
             const IO* dk = dg + (int64_t)c * kTile * p.d_sl;
             const IO* yk = yg + (int64_t)c * kTile * p.y_sl;
-            const IO* zk = zg + (int64_t)c * kTile * p.u_sl;
+            const IO* zk = zg + (int64_t)c * kTile * p.z_sl;
             const IO* ypk = ypg + (int64_t)c * kTile * p.y_sl;
             const IO* Bk = Bg + (int64_t)c * kTile * p.bc_sl;
             const IO* Ck = Cg + (int64_t)c * kTile * p.bc_sl;
-            uint32_t ox[4], od[4], oy[4], ob[kBcPer];
+            uint32_t ox[4], od[4], oy[4], oz[4], ob[kBcPer];
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
+                oz[j] = offzi[j];
                 ox[j] = offx[j];
                 od[j] = offd[j];
                 oy[j] = offy[j];
@@ -249,6 +251,7 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
                     ox[j] = (tc * (uint32_t)p.u_sl + (uint32_t)cic * (uint32_t)p.u_sd) * kES;
                     od[j] = (tc * (uint32_t)p.d_sl + (uint32_t)cic * (uint32_t)p.d_sd) * kES;
                     oy[j] = (tc * (uint32_t)p.y_sl + (uint32_t)cic * (uint32_t)p.y_sd) * kES;
+                    oz[j] = (tc * (uint32_t)p.z_sl + (uint32_t)cic * (uint32_t)p.z_sd) * kES;
                 }
 #pragma unroll
                 for (int r = 0; r < kBcPer; ++r)
@@ -260,7 +263,7 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
                 raw.d[j] = ld_off(dk, od[j]);
                 raw.y[j] = ld_off(yk, oy[j]);
                 if constexpr (HAS_Z) {
-                    raw.z[j] = ld_off(zk, ox[j]);
+                    raw.z[j] = ld_off(zk, oz[j]);
                     raw.yp[j] = ld_off(ypk, oy[j]);
                 }
             }

@@ -49,6 +49,7 @@ struct FwdParams {
     int in_tmajor;   // x / delta have unit stride along time
     int out_tmajor;  // y has unit stride along time
     int64_t u_sb, u_sl, u_sd;
+    int64_t z_sb, z_sl, z_sd;
     int64_t d_sb, d_sl, d_sd;
     int64_t y_sb, y_sl, y_sd;
 };
@@ -194,13 +195,14 @@ __global__ void __launch_bounds__((NW + kService) * kWave) sscan_fwd_kernel(cons
             // address arithmetic in the loop
             const IO* const xg = static_cast<const IO*>(p.x) + (b * p.u_sb + (int64_t)d0 * p.u_sd);
             const IO* const dg = static_cast<const IO*>(p.delta) + (b * p.d_sb + (int64_t)d0 * p.d_sd);
-            const IO* const zg = static_cast<const IO*>(p.z) + (b * p.u_sb + (int64_t)d0 * p.u_sd);
-            uint32_t offx[4], offd[4];
+            const IO* const zg = static_cast<const IO*>(p.z) + (b * p.z_sb + (int64_t)d0 * p.z_sd);
+            uint32_t offx[4], offd[4], offz[4];
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 // byte offsets (see ld_off)
                 offx[j] = ((uint32_t)(4 * qi + j) * (uint32_t)p.u_sl + (uint32_t)cic * (uint32_t)p.u_sd) * kES;
                 offd[j] = ((uint32_t)(4 * qi + j) * (uint32_t)p.d_sl + (uint32_t)cic * (uint32_t)p.d_sd) * kES;
+                offz[j] = ((uint32_t)(4 * qi + j) * (uint32_t)p.z_sl + (uint32_t)cic * (uint32_t)p.z_sd) * kES;
             }
             const bool group_full = cmax == kWave - 1;
             // B/C of a tile: kTile * NP elements each, kBcPer per loader thread, step fastest
@@ -238,14 +240,15 @@ __global__ void __launch_bounds__((NW + kService) * kWave) sscan_fwd_kernel(cons
                 const int k = min(kk, ntiles - 1);
                 const IO* xk = xg + (int64_t)k * kTile * p.u_sl;
                 const IO* dk = dg + (int64_t)k * kTile * p.d_sl;
-                const IO* zk = zg + (int64_t)k * kTile * p.u_sl;
+                const IO* zk = zg + (int64_t)k * kTile * p.z_sl;
                 const IO* Bk = Bg + (int64_t)k * kTile * p.bc_sl;
                 const IO* Ck = Cg + (int64_t)k * kTile * p.bc_sl;
-                uint32_t ox[4], od[4], ob[kBcPer > 0 ? kBcPer : 1];
+                uint32_t ox[4], od[4], oz[4], ob[kBcPer > 0 ? kBcPer : 1];
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
                     ox[j] = offx[j];
                     od[j] = offd[j];
+                    oz[j] = offz[j];
                 }
 #pragma unroll
                 for (int r = 0; r < kBcPer; ++r) ob[r] = offbc[r];
@@ -256,6 +259,7 @@ __global__ void __launch_bounds__((NW + kService) * kWave) sscan_fwd_kernel(cons
                         const uint32_t tc = (uint32_t)min(4 * qi + j, tmax);
                         ox[j] = (tc * (uint32_t)p.u_sl + (uint32_t)cic * (uint32_t)p.u_sd) * kES;
                         od[j] = (tc * (uint32_t)p.d_sl + (uint32_t)cic * (uint32_t)p.d_sd) * kES;
+                        oz[j] = (tc * (uint32_t)p.z_sl + (uint32_t)cic * (uint32_t)p.z_sd) * kES;
                     }
 #pragma unroll
                     for (int r = 0; r < kBcPer; ++r)
@@ -265,7 +269,7 @@ __global__ void __launch_bounds__((NW + kService) * kWave) sscan_fwd_kernel(cons
                 for (int j = 0; j < 4; ++j) {
                     raw.x[j] = ld_off(xk, ox[j]);
                     raw.d[j] = ld_off(dk, od[j]);
-                    if (has_z) raw.z[j] = ld_off(zk, ox[j]);
+                    if (has_z) raw.z[j] = ld_off(zk, oz[j]);
                 }
 #pragma unroll
                 for (int r = 0; r < kBcPer; ++r) {
@@ -576,13 +580,13 @@ int validate_shape(const mpa_sscan_shape* s) {
     if (s->dstate > MPA_MAX_DSTATE || s->batch > 65535) return MPA_ERR_BAD_SHAPE;
     if (s->seqlen > (int64_t)1 << 30 || s->dim > (int64_t)1 << 30) return MPA_ERR_BAD_SHAPE;
     if (s->io_dtype != MPA_F32 && s->io_dtype != MPA_BF16) return MPA_ERR_BAD_DTYPE;
-    const int64_t st[] = {s->u_sb, s->u_sl, s->u_sd, s->d_sb, s->d_sl, s->d_sd, s->y_sb, s->y_sl,
+    const int64_t st[] = {s->z_sb, s->z_sl, s->z_sd, s->u_sb, s->u_sl, s->u_sd, s->d_sb, s->d_sl, s->d_sd, s->y_sb, s->y_sl,
                           s->y_sd, s->g_sb, s->g_sl, s->g_sd, s->bc_sb, s->bc_sl, s->dbc_sb, s->dbc_sl};
     for (int64_t v : st)
         if (v < 0) return MPA_ERR_BAD_STRIDE;
     // one (kTile steps x 64 channels) tile is addressed with 32-bit byte offsets; so are a
     // tile of B / C and one checkpoint (d_state x dim floats)
-    const int64_t tile[][2] = {{s->u_sl, s->u_sd}, {s->d_sl, s->d_sd}, {s->y_sl, s->y_sd},
+    const int64_t tile[][2] = {{s->z_sl, s->z_sd}, {s->u_sl, s->u_sd}, {s->d_sl, s->d_sd}, {s->y_sl, s->y_sd},
                                {s->g_sl, s->g_sd}};
     for (const auto& v : tile)
         if (v[0] * kTile + v[1] * kWave >= ((int64_t)1 << 30)) return MPA_ERR_BAD_STRIDE;
@@ -694,6 +698,7 @@ extern "C" int mpa_sscan_fwd(const mpa_sscan_shape* s, const void* x, const void
     p.nchunks = (p.L + kTile - 1) / kTile;
     p.softplus = softplus ? 1 : 0;
     p.u_sb = s->u_sb; p.u_sl = s->u_sl; p.u_sd = s->u_sd;
+    p.z_sb = s->z_sb; p.z_sl = s->z_sl; p.z_sd = s->z_sd;
     p.d_sb = s->d_sb; p.d_sl = s->d_sl; p.d_sd = s->d_sd;
     p.y_sb = s->y_sb; p.y_sl = s->y_sl; p.y_sd = s->y_sd;
     p.in_tmajor = (s->u_sd != 1 && s->u_sl == 1) ? 1 : 0;

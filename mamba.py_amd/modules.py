@@ -16,6 +16,7 @@ import torch
 import torch.nn as nn
 import torch.nn.functional as F
 
+from .conv import causal_conv1d_fn
 from .scan import selective_scan, selective_scan_fn, ssm_step
 
 
@@ -139,36 +140,46 @@ class MambaBlock(nn.Module):
         L = x.shape[1]
         xz = self.in_proj(x)
         xin, z = xz.chunk(2, dim=-1)
-        # causal depthwise convolution along time, kept in (B, ED, L) memory: the scan kernel
-        # reads this layout directly
-        xc = self.conv1d(xin.transpose(1, 2))[:, :, :L]
-        xs = F.silu(xc).transpose(1, 2)                      # (B, L, ED), unit stride along L
+        K = self.config.d_conv
+        window = None
+        if 2 <= K <= 4:
+            # causal depthwise convolution + bias + silu in one kernel, reading the x half of
+            # the projection in place (no transposes) and returning the decode window
+            if return_cache:
+                xs, window = causal_conv1d_fn(xin, self.conv1d.weight, self.conv1d.bias, return_window=True)
+            else:
+                xs = causal_conv1d_fn(xin, self.conv1d.weight, self.conv1d.bias)
+        else:
+            xc = self.conv1d(xin.transpose(1, 2))[:, :, :L]
+            xs = F.silu(xc).transpose(1, 2)                  # (B, L, ED), unit stride along L
+        # the gate y * silu(z) is applied inside the scan kernel (z is read in place)
         if return_cache:
             y, h_last = self.ssm(xs, z, return_last_state=True)
         else:
             y = self.ssm(xs, z)
-        out = self.out_proj(y * F.silu(z))
+        out = self.out_proj(y)
         if not return_cache:
             return out
-        K = self.config.d_conv - 1
-        pre = xin.transpose(1, 2)
-        if L >= K:
-            window = pre[:, :, L - K:].contiguous()
-        else:
-            window = F.pad(pre, (K - L, 0)).contiguous()
+        if window is None:
+            pre = xin.transpose(1, 2)
+            if L >= K - 1:
+                window = pre[:, :, L - (K - 1):].contiguous()
+            else:
+                window = F.pad(pre, (K - 1 - L, 0)).contiguous()
         return out, (h_last, window)
 
     def ssm(self, x, z=None, return_last_state: bool = False):
         """(B, L, ED) -> (B, L, ED): projections to (delta, B, C), then the fused scan
-        (mambapy/mamba.py:236-272)."""
+        (mambapy/mamba.py:236-272); with z the result is already gated, y * silu(z), as on the
+        reference's fused path (mamba.py:259-260, 225-227)."""
         A, D = self._A(), self.D.float()
         dlow, Bm, C = self._split_projection(self.x_proj(x))
         delta = (self.dt_proj.weight @ dlow.transpose(1, 2)).transpose(1, 2)   # (B, L, ED) view
         if self.config.fused_softplus:
-            return selective_scan_fn(x, delta, A, Bm, C, D, delta_bias=self.dt_proj.bias,
+            return selective_scan_fn(x, delta, A, Bm, C, D, z=z, delta_bias=self.dt_proj.bias,
                                      delta_softplus=True, return_last_state=return_last_state)
         delta = F.softplus(delta + self.dt_proj.bias)
-        return selective_scan_fn(x, delta, A, Bm, C, D, return_last_state=return_last_state)
+        return selective_scan_fn(x, delta, A, Bm, C, D, z=z, return_last_state=return_last_state)
 
     def selective_scan(self, x, delta, A, B, C, D):
         """Same call as MambaBlock.selective_scan (mambapy/mamba.py:274-295)."""

@@ -50,13 +50,15 @@ def _rows_unit_stride(t):
     return t if t.stride(-1) == 1 else t.contiguous()
 
 
-def _sscan_shape(x, delta, Bm, y_like, g_like, dbc_like, N, flags):
+def _sscan_shape(x, delta, Bm, y_like, g_like, dbc_like, N, flags, z=None):
     s = _lib.SscanShape()
     s.batch, s.seqlen, s.dim = x.shape
     s.dstate = N
     s.io_dtype = _io_dtype(x)
     s.flags = flags
     s.u_sb, s.u_sl, s.u_sd = x.stride()
+    if z is not None:
+        s.z_sb, s.z_sl, s.z_sd = z.stride()
     s.d_sb, s.d_sl, s.d_sd = delta.stride()
     s.y_sb, s.y_sl, s.y_sd = y_like.stride()
     s.g_sb, s.g_sl, s.g_sd = g_like.stride()
@@ -91,18 +93,13 @@ class SelectiveScanFn(torch.autograd.Function):
         C_ = _rows_unit_stride(C.detach().to(dt))
         if C_.stride() != B_.stride():
             B_, C_ = B_.contiguous(), C_.contiguous()
-        z_ = None
-        if z is not None:
-            z_ = z.detach().to(dt)
-            if z_.stride() != x_.stride():
-                z_ = z_.contiguous()
-                x_ = x_.contiguous()
+        z_ = None if z is None else z.detach().to(dt)
         A_, D_, bias_, h0_ = _f32c(A), _f32c(D), _f32c(delta_bias), _f32c(h0)
         y = torch.empty((Bsz, L, ED), dtype=dt, device=x.device)
         need_grad = any(t is not None and t.requires_grad
                         for t in (x, delta, A, B, C, D, z, delta_bias))
         flags = _lib.MPA_SSCAN_DELTA_SOFTPLUS if delta_softplus else 0
-        shape = _sscan_shape(x_, delta_, B_, y, y, B_, N, flags)
+        shape = _sscan_shape(x_, delta_, B_, y, y, B_, N, flags, z_)
         ckpt = y_pre = None
         if need_grad:
             ckpt = torch.empty(lib.mpa_sscan_ckpt_elems(ctypes.byref(shape)), dtype=torch.float32,
@@ -149,7 +146,7 @@ class SelectiveScanFn(torch.autograd.Function):
         dB = torch.empty((Bsz, L, N), dtype=dt, device=x.device)
         dC = torch.empty_like(dB)
         dbias = torch.empty((ED,), dtype=torch.float32, device=x.device) if bias is not None else None
-        shape = _sscan_shape(x, delta, B, dy, dx, dB, N, ctx.flags)
+        shape = _sscan_shape(x, delta, B, dy, dx, dB, N, ctx.flags, z)
         nbytes = lib.mpa_sscan_bwd_workspace_bytes(ctypes.byref(shape))
         ws = torch.empty(nbytes, dtype=torch.uint8, device=x.device)
         with torch.cuda.device(x.device):
