@@ -174,7 +174,9 @@ class MambaBlock(nn.Module):
         reference's fused path (mamba.py:259-260, 225-227)."""
         A, D = self._A(), self.D.float()
         dlow, Bm, C = self._split_projection(self.x_proj(x))
-        delta = (self.dt_proj.weight @ dlow.transpose(1, 2)).transpose(1, 2)   # (B, L, ED) view
+        # (B, L, ED) with unit stride along ED, the layout of x: the reference forms the transposed
+        # product (mamba.py:247) only because its fused backend wants (B, ED, L)
+        delta = F.linear(dlow, self.dt_proj.weight)
         if self.config.fused_softplus:
             return selective_scan_fn(x, delta, A, Bm, C, D, z=z, delta_bias=self.dt_proj.bias,
                                      delta_softplus=True, return_last_state=return_last_state)
