@@ -153,6 +153,9 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
         // ================================ service waves ================================
         const int sw = w - NW;
         const int item = sw * kWave + lane;  // 0 .. 255
+        // with softplus or the gate the service waves carry long chains of transcendental
+        // functions and would reach the tile barrier last: they then go first when ready
+        if (HAS_Z || p.softplus) __builtin_amdgcn_s_setprio(2);
         constexpr uint32_t kES = sizeof(IO);
         const bool group_full = cmax == kWave - 1;
 

@@ -179,6 +179,10 @@ __global__ void __launch_bounds__((NW + kService) * kWave) sscan_fwd_kernel(cons
         // waves is kept short (offsets precomputed, one uniform branch for the ragged edge)
         // and spread over four waves per role.
         const int sw = w - NW;                       // 0..3: loaders   4..7: reducers
+        // With softplus or the gate the service waves carry long dependent chains of
+        // transcendental functions and would reach the tile barrier last: they then go first
+        // whenever they are ready (measured: -10 % with gate + softplus, +8 % without either)
+        if (has_z || p.softplus) __builtin_amdgcn_s_setprio(2);
         const int cmax = min(kWave, p.ED - d0) - 1;  // last valid channel of the group
         const int item = (sw & 3) * kWave + lane;    // 0 .. 255
         constexpr uint32_t kES = sizeof(IO);
