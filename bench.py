@@ -115,9 +115,19 @@ def bench_decode(args, torch, pkg, dev):
             for _ in range(tokens):
                 _, c = block.step(xin, c)
 
+    # the same block step recorded once in a HIP graph and replayed per token
+    stack = pkg.Mamba(cfg).to(dev)
+    stack.layers[0].mixer.load_state_dict(block.state_dict())
+    decoder = pkg.GraphedDecoder(stack, [cache])
+
+    def graph_tokens():
+        for _ in range(tokens):
+            decoder(xin)
+
     steps, warmup = max(1, args.steps // 10), 1
     t_kernel = _timed(torch, kernel_tokens, steps, warmup) / tokens
     t_block = _timed(torch, block_tokens, steps, warmup) / tokens
+    t_graph = _timed(torch, graph_tokens, steps, warmup) / tokens
     bytes_step = 2 * 4 * Bsz * ED * N + 4 * 4 * Bsz * ED + 4 * (ED * N + 2 * ED) + 2 * 4 * Bsz * N
     out = {
         "metric": "decode step latency per token (state-update kernel), mamba-2.8b layer, batch 64",
@@ -126,6 +136,7 @@ def bench_decode(args, torch, pkg, dev):
         "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic (seeded)",
         "tokens_per_s_layer_kernel": Bsz / t_kernel,
         "block_step_us": t_block * 1e6, "tokens_per_s_layer_block": Bsz / t_block,
+        "graphed_layer_step_us": t_graph * 1e6, "tokens_per_s_layer_graphed": Bsz / t_graph,
         "config": {"workload": "configs[3]: decode step, ED=5120 N=16 batch 64, 256 tokens per bench step",
                    "algorithmic_bytes_per_token_step": bytes_step},
         "roofline": {"bound": "hbm", "kernel": "ssm_step_quad_kernel", "achieved": bytes_step / t_kernel / 1e9,

@@ -8,11 +8,12 @@ from .scan import PScan, pscan, selective_scan, selective_scan_fn, ssm_step, Sel
 from .conv import CausalConv1dFn, causal_conv1d_fn
 from .modules import Mamba, MambaBlock, MambaConfig, ResidualBlock, RMSNorm
 from .language_model import LM
+from .decode import GraphedDecoder
 from .patch import patch_mambapy
 
 __all__ = ["PScan", "pscan", "selective_scan", "selective_scan_fn", "ssm_step",
            "SelectiveScanFn", "CausalConv1dFn", "causal_conv1d_fn", "Mamba", "MambaBlock", "MambaConfig", "ResidualBlock", "RMSNorm",
-           "LM", "patch_mambapy", "library_path", "library_version"]
+           "LM", "GraphedDecoder", "patch_mambapy", "library_path", "library_version"]
 
 
 def library_path() -> str:

@@ -208,14 +208,28 @@ class MambaBlock(nn.Module):
         out = self.out_proj(y)
         return out, (h, window[:, :, 1:])
 
-    def ssm_step(self, x, h, z=None):
+    def ssm_step(self, x, h, z=None, inplace: bool = False):
         """x : (B, ED), h : (B, ED, N) or None -> (y, h'); mambapy/mamba.py:384-414.  With z
-        the gate y*silu(z) is applied inside the kernel."""
+        the gate y*silu(z) is applied inside the kernel; inplace=True updates h itself."""
         dlow, Bm, C = self._split_projection(self.x_proj(x))
         raw = F.linear(dlow, self.dt_proj.weight)                        # bias added in-kernel
         y, h_new = ssm_step(x, raw, self._A(), Bm, C, self.D.float(), h, z=z,
-                            delta_bias=self.dt_proj.bias, delta_softplus=True)
+                            delta_bias=self.dt_proj.bias, delta_softplus=True, inplace=inplace)
         return y, h_new
+
+    def step_(self, x, h, window):
+        """In-place decode step for loops that must not allocate new cache tensors (HIP graph
+        replay): x (B, D); h (B, ED, N) float32 and window (B, ED, d_conv-1) are updated in
+        place.  Same arithmetic as step()."""
+        xz = self.in_proj(x)
+        xin, z = xz.chunk(2, dim=1)
+        full = torch.cat([window, xin.unsqueeze(2)], dim=2)              # (B, ED, d_conv)
+        xc = (full * self.conv1d.weight[:, 0, :]).sum(-1)
+        if self.conv1d.bias is not None:
+            xc = xc + self.conv1d.bias
+        y, _ = self.ssm_step(F.silu(xc), h, z=z, inplace=True)
+        window.copy_(full[:, :, 1:])
+        return self.out_proj(y)
 
 
 class ResidualBlock(nn.Module):
@@ -235,6 +249,9 @@ class ResidualBlock(nn.Module):
     def step(self, x, cache):
         y, cache = self.mixer.step(self.norm(x), cache)
         return y + x, cache
+
+    def step_(self, x, h, window):
+        return self.mixer.step_(self.norm(x), h, window) + x
 
 
 class Mamba(nn.Module):
@@ -260,6 +277,13 @@ class Mamba(nn.Module):
         for i, layer in enumerate(self.layers):
             x, caches[i] = layer.step(x, caches[i])
         return x, caches
+
+    def step_(self, x, caches):
+        """In-place variant of step(): every (h, window) pair of `caches` is updated in place
+        (h must be a float32 tensor, not None)."""
+        for layer, (h, window) in zip(self.layers, caches):
+            x = layer.step_(x, h, window)
+        return x
 
     def empty_caches(self, batch: int, device=None, dtype=None):
         """Fresh decode caches: h = None (zero state), zero conv window (mamba.py:344-346)."""

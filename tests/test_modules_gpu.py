@@ -110,3 +110,34 @@ def test_softplus_path_without_gate_full_gradients(pkg, dev):
                            (gA.grad, A.grad, "dA"), (gB.grad, Bm.grad, "dB"), (gC.grad, C.grad, "dC"),
                            (gD.grad, D.grad, "dD"), (gb.grad, bb.grad, "dbias")):
         assert rel_err(got, ref) <= 1e-4, name
+
+
+def test_graphed_decoder_replays_match_eager_steps(pkg, dev):
+    # one decode step recorded in a HIP graph: every replay must equal the eager step, with
+    # eager work and synchronisations between the replays
+    torch.manual_seed(7)
+    cfg = pkg.MambaConfig(d_model=64, n_layers=3)
+    lm = pkg.LM(cfg, 100).to(dev)
+    prompt = torch.randint(0, 100, (4, 9), device=dev)
+    with torch.no_grad():
+        logits, caches = lm.prefill(prompt)
+        decoder = pkg.GraphedDecoder(lm, caches)
+        tok = logits.argmax(-1)
+        for i in range(6):
+            want, caches = lm.step(tok, caches)          # eager
+            got = decoder(tok).clone()                   # graph replay
+            torch.cuda.synchronize()
+            _ = (want.float() @ want.float().T).sum().item()   # unrelated eager work + sync
+            assert rel_err(got, want) <= 1e-5, i
+            for (h, w), (hg, wg) in zip(caches, decoder.caches):
+                assert rel_err(hg, h) <= 1e-5 and torch.equal(wg, w), i
+            tok = want.argmax(-1)
+    # a bare stack, starting from empty caches (h = None)
+    model = pkg.Mamba(cfg).to(dev)
+    x = torch.randn(5, 2, 64, device=dev)
+    with torch.no_grad():
+        caches = model.empty_caches(2)
+        decoder = pkg.GraphedDecoder(model, caches)
+        for t in range(5):
+            want, caches = model.step(x[t], caches)
+            assert rel_err(decoder(x[t]), want) <= 1e-5, t
