@@ -192,14 +192,25 @@ __global__ void __launch_bounds__(256) conv1d_bwd_kernel(const ConvParams p) {
     part[(int64_t)kConvMaxK * p.ED] = db;
 }
 
-// dweight[d][k] / dbias[d] = sum over (batch, span) of the partial sums, in index order
-__global__ void __launch_bounds__(256) conv1d_bwd_finish_kernel(const float* part, float* dweight,
-                                                                float* dbias, int ED, int K, int nparts) {
-    const int i = blockIdx.x * blockDim.x + threadIdx.x;  // (k5, d), d fastest
-    if (i >= (kConvMaxK + 1) * ED) return;
-    const int k5 = i / ED, d = i % ED;
+// dweight[d][k] / dbias[d] = sum over (batch, span) of the partial sums.  A block owns 64
+// columns of the [(K+1) * ED] partial rows; its 16 row groups each sum every 16th partial in
+// index order and the groups are combined in a fixed order through LDS (no atomics, so the
+// result does not depend on scheduling).
+constexpr int kFinCols = 64, kFinRows = 16;
+__global__ void __launch_bounds__(kFinCols* kFinRows)
+    conv1d_bwd_finish_kernel(const float* part, float* dweight, float* dbias, int ED, int K, int nparts) {
+    __shared__ float acc[kFinRows][kFinCols];
+    const int col = threadIdx.x % kFinCols, rg = threadIdx.x / kFinCols;
+    const int i = blockIdx.x * kFinCols + col;  // (k5, d), d fastest
+    const int width = (kConvMaxK + 1) * ED;
     float s = 0.0f;
-    for (int q = 0; q < nparts; ++q) s += part[(int64_t)q * (kConvMaxK + 1) * ED + i];
+    if (i < width)
+        for (int q = rg; q < nparts; q += kFinRows) s += part[(int64_t)q * width + i];
+    acc[rg][col] = s;
+    __syncthreads();
+    if (rg != 0 || i >= width) return;
+    for (int r = 1; r < kFinRows; ++r) s += acc[r][col];
+    const int k5 = i / ED, d = i % ED;
     if (k5 == kConvMaxK) {
         if (dbias) dbias[d] = s;
     } else {
@@ -294,7 +305,7 @@ extern "C" int mpa_conv1d_bwd(const mpa_conv_shape* s, const void* x, const floa
     rc = check_launch();
     if (rc != MPA_OK) return rc;
     const int total = (kConvMaxK + 1) * p.ED;
-    hipLaunchKernelGGL(conv1d_bwd_finish_kernel, dim3((total + 255) / 256), dim3(256), 0, st, p.part, dweight,
-                       dbias, p.ED, p.K, p.batch * p.nspan);
+    hipLaunchKernelGGL(conv1d_bwd_finish_kernel, dim3((total + kFinCols - 1) / kFinCols),
+                       dim3(kFinCols * kFinRows), 0, st, p.part, dweight, dbias, p.ED, p.K, p.batch * p.nspan);
     return check_launch();
 }
