@@ -63,33 +63,43 @@ __device__ __forceinline__ float sigmoid_f(float v) {
     return __builtin_amdgcn_rcpf(1.0f + fast_exp2(-v * kLog2e));
 }
 
-// Element at a 32-bit BYTE offset from a wave-uniform pointer, through the buffer instructions:
-// one instruction per access (scalar descriptor + 32-bit vector offset), no 64-bit address
-// arithmetic or address registers per lane.  The descriptor is raw (stride 0) with the maximum
-// range, i.e. the access is not bounds-checked; callers keep offsets inside their tensors.
+// Element at (wave-uniform pointer) + (32-bit per-lane BYTE offset) + (wave-uniform byte offset),
+// through the buffer instructions: one instruction per access (scalar descriptor, one vector
+// register of offset, one scalar register of offset), no 64-bit address arithmetic or address
+// registers per lane.  `bytes` is the size of the window that starts at the pointer: loads
+// beyond it return zero and stores beyond it are dropped by the hardware, so a caller that
+// passes "bytes left in the tensor" needs no clamping to keep ragged tiles inside the
+// allocation.  The default window is the maximum (no bounds check).
 typedef __amdgpu_buffer_rsrc_t rsrc_t;
-__device__ __forceinline__ rsrc_t make_rsrc(const void* base) {
-    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, 0xffffffff, 0x00020000);
+__device__ __forceinline__ rsrc_t make_rsrc(const void* base, uint32_t bytes = 0xffffffffu) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, bytes, 0x00020000);
 }
-__device__ __forceinline__ float ld_off(const float* base, uint32_t byte_off) {
-    return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(make_rsrc(base), byte_off, 0, 0));
+// bytes from element offset `at` to the end of a tensor of `end` elements, as a buffer window
+__device__ __forceinline__ uint32_t window_bytes(int64_t end, int64_t at, int es) {
+    const int64_t left = (end - at) * es;
+    return left <= 0 ? 0u : left > 0xffffffffll ? 0xffffffffu : (uint32_t)left;
 }
-__device__ __forceinline__ bf16_t ld_off(const bf16_t* base, uint32_t byte_off) {
-    return __builtin_bit_cast(bf16_t, __builtin_amdgcn_raw_buffer_load_b16(make_rsrc(base), byte_off, 0, 0));
+__device__ __forceinline__ float ld_off(const float* base, uint32_t voff, uint32_t soff = 0,
+                                        uint32_t bytes = 0xffffffffu) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(make_rsrc(base, bytes), voff, soff, 0));
 }
-__device__ __forceinline__ void st_off(float* base, uint32_t byte_off, float v) {
-    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, v), make_rsrc(base), byte_off, 0, 0);
+__device__ __forceinline__ bf16_t ld_off(const bf16_t* base, uint32_t voff, uint32_t soff = 0,
+                                         uint32_t bytes = 0xffffffffu) {
+    return __builtin_bit_cast(bf16_t, __builtin_amdgcn_raw_buffer_load_b16(make_rsrc(base, bytes), voff, soff, 0));
 }
-__device__ __forceinline__ void st_off(bf16_t* base, uint32_t byte_off, bf16_t v) {
-    __builtin_amdgcn_raw_buffer_store_b16(__builtin_bit_cast(unsigned short, v), make_rsrc(base), byte_off, 0, 0);
+__device__ __forceinline__ void st_off(float* base, uint32_t voff, float v, uint32_t soff = 0) {
+    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, v), make_rsrc(base), voff, soff, 0);
+}
+__device__ __forceinline__ void st_off(bf16_t* base, uint32_t voff, bf16_t v, uint32_t soff = 0) {
+    __builtin_amdgcn_raw_buffer_store_b16(__builtin_bit_cast(unsigned short, v), make_rsrc(base), voff, soff, 0);
 }
 typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
 typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
-__device__ __forceinline__ void st_off(float2* base, uint32_t byte_off, float2 v) {
-    __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(u32x2, v), make_rsrc(base), byte_off, 0, 0);
+__device__ __forceinline__ void st_off(float2* base, uint32_t voff, float2 v, uint32_t soff = 0) {
+    __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(u32x2, v), make_rsrc(base), voff, soff, 0);
 }
-__device__ __forceinline__ void st_off(float4* base, uint32_t byte_off, float4 v) {
-    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v), make_rsrc(base), byte_off, 0, 0);
+__device__ __forceinline__ void st_off(float4* base, uint32_t voff, float4 v, uint32_t soff = 0) {
+    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v), make_rsrc(base), voff, soff, 0);
 }
 
 // Lane index recomputed on the spot (two VALU instructions).  Per-lane addresses that are used

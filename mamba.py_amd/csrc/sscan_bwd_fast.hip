@@ -165,24 +165,23 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
         const bool ci_ok = ci <= cmax;
         const int cic = min(ci, cmax);
         const float bias = p.dbias ? p.dbias[d0 + cic] : 0.0f;
-        const IO* const xg = static_cast<const IO*>(p.x) + (b * p.u_sb + (int64_t)d0 * p.u_sd);
-        const IO* const dg = static_cast<const IO*>(p.delta) + (b * p.d_sb + (int64_t)d0 * p.d_sd);
-        const IO* const yg = static_cast<const IO*>(p.dy) + (b * p.y_sb + (int64_t)d0 * p.y_sd);
-        const IO* const zg = static_cast<const IO*>(p.z) + (b * p.z_sb + (int64_t)d0 * p.z_sd);
-        const IO* const ypg = static_cast<const IO*>(p.ypre) + (b * p.y_sb + (int64_t)d0 * p.y_sd);
         IO* const dzg = static_cast<IO*>(p.dz) + (b * p.g_sb + (int64_t)d0 * p.g_sd);
-        const IO* const Bg = static_cast<const IO*>(p.Bm) + b * p.bc_sb;
-        const IO* const Cg = static_cast<const IO*>(p.C) + b * p.bc_sb;
-        uint32_t offx[4], offd[4], offy[4], offz[4], offzi[4];  // offz: dz, addressed like dx; offzi: z
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            offz[j] = ((uint32_t)(4 * qi + j) * (uint32_t)p.g_sl + (uint32_t)cic * (uint32_t)p.g_sd) * kES;
-            offzi[j] = ((uint32_t)(4 * qi + j) * (uint32_t)p.z_sl + (uint32_t)cic * (uint32_t)p.z_sd) * kES;
-            // byte offsets (see ld_off)
-            offx[j] = ((uint32_t)(4 * qi + j) * (uint32_t)p.u_sl + (uint32_t)cic * (uint32_t)p.u_sd) * kES;
-            offd[j] = ((uint32_t)(4 * qi + j) * (uint32_t)p.d_sl + (uint32_t)cic * (uint32_t)p.d_sd) * kES;
-            offy[j] = ((uint32_t)(4 * qi + j) * (uint32_t)p.y_sl + (uint32_t)cic * (uint32_t)p.y_sd) * kES;
-        }
+        // byte offset of the item's first step (one vector register per tensor); its other three
+        // steps are one row stride further each, which goes into the scalar offset of the access
+        const uint32_t offx = ((uint32_t)(4 * qi) * (uint32_t)p.u_sl + (uint32_t)cic * (uint32_t)p.u_sd) * kES;
+        const uint32_t offd = ((uint32_t)(4 * qi) * (uint32_t)p.d_sl + (uint32_t)cic * (uint32_t)p.d_sd) * kES;
+        const uint32_t offy = ((uint32_t)(4 * qi) * (uint32_t)p.y_sl + (uint32_t)cic * (uint32_t)p.y_sd) * kES;
+        const uint32_t offzi = ((uint32_t)(4 * qi) * (uint32_t)p.z_sl + (uint32_t)cic * (uint32_t)p.z_sd) * kES;
+        const uint32_t offz = ((uint32_t)(4 * qi) * (uint32_t)p.g_sl + (uint32_t)cic * (uint32_t)p.g_sd) * kES;  // dz
+        const uint32_t sx = (uint32_t)p.u_sl * kES, sd = (uint32_t)p.d_sl * kES, sy = (uint32_t)p.y_sl * kES;
+        const uint32_t sz = (uint32_t)p.z_sl * kES, sg = (uint32_t)p.g_sl * kES;
+        // one past the last element of each input tensor, relative to its first: the loads of a
+        // ragged tile may run past the sequence end but never past this (they are windowed)
+        const int64_t endx = (p.batch - 1) * p.u_sb + (p.L - 1) * p.u_sl + (p.ED - 1) * p.u_sd + 1;
+        const int64_t endd = (p.batch - 1) * p.d_sb + (p.L - 1) * p.d_sl + (p.ED - 1) * p.d_sd + 1;
+        const int64_t endy = (p.batch - 1) * p.y_sb + (p.L - 1) * p.y_sl + (p.ED - 1) * p.y_sd + 1;
+        const int64_t endz = (p.batch - 1) * p.z_sb + (p.L - 1) * p.z_sl + (p.ED - 1) * p.z_sd + 1;
+        const int64_t endbc = (p.batch - 1) * p.bc_sb + (p.L - 1) * p.bc_sl + p.N;
         // B/C of a tile: kTile * NP elements each, kBcPer per service thread, step fastest
         constexpr int kBcPer = NP * kTile / (kSvc * kWave);
         static_assert(NP * kTile % (kSvc * kWave) == 0, "whole elements per thread");
@@ -201,10 +200,7 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
         const int qo = p.out_tmajor ? item % NQ : item / kWave;
         const bool co_ok = co <= cmax;
         const float Dr = p.D[d0 + min(co, cmax)];
-        uint32_t offg[4];
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-            offg[j] = ((uint32_t)(4 * qo + j) * (uint32_t)p.g_sl + (uint32_t)min(co, cmax) * (uint32_t)p.g_sd) * kES;
+        const uint32_t offg = ((uint32_t)(4 * qo) * (uint32_t)p.g_sl + (uint32_t)min(co, cmax) * (uint32_t)p.g_sd) * kES;
         IO* const dxg = static_cast<IO*>(p.dx) + (b * p.g_sb + (int64_t)d0 * p.g_sd);
         IO* const ddg = static_cast<IO*>(p.ddelta) + (b * p.g_sb + (int64_t)d0 * p.g_sd);
         // dB/dC forwarding: kFw consecutive states of one (step, dB|dC) per thread
@@ -225,55 +221,38 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
         // is longer than one tile interval)
         struct Raw { IO x[4], d[4], y[4], z[HAS_Z ? 4 : 1], yp[HAS_Z ? 4 : 1], b[kBcPer], c[kBcPer]; };
         auto load_tile = [&](int kk, Raw& raw) {
-            // tiles and steps beyond the sequence are clamped, so the loads stay in bounds;
-            // only the offsets depend on the (uniform) branch, the loads are unconditional
+            // tiles beyond the last one are clamped to it; steps beyond the sequence end are read
+            // as whatever follows inside the tensor (or zero past its end) and masked at staging
             const int k = min(kk, ntiles - 1);
             const int c = chunk_of(k);
-            const IO* xk = xg + (int64_t)c * kTile * p.u_sl;
-            const IO* dk = dg + (int64_t)c * kTile * p.d_sl;
-            const IO* yk = yg + (int64_t)c * kTile * p.y_sl;
-            const IO* zk = zg + (int64_t)c * kTile * p.z_sl;
-            const IO* ypk = ypg + (int64_t)c * kTile * p.y_sl;
-            const IO* Bk = Bg + (int64_t)c * kTile * p.bc_sl;
-            const IO* Ck = Cg + (int64_t)c * kTile * p.bc_sl;
-            uint32_t ox[4], od[4], oy[4], oz[4], ob[kBcPer];
+            const int64_t ex = b * p.u_sb + (int64_t)d0 * p.u_sd + (int64_t)c * kTile * p.u_sl;
+            const int64_t ed = b * p.d_sb + (int64_t)d0 * p.d_sd + (int64_t)c * kTile * p.d_sl;
+            const int64_t ey = b * p.y_sb + (int64_t)d0 * p.y_sd + (int64_t)c * kTile * p.y_sl;
+            const int64_t ez = b * p.z_sb + (int64_t)d0 * p.z_sd + (int64_t)c * kTile * p.z_sl;
+            const int64_t ebc = b * p.bc_sb + (int64_t)c * kTile * p.bc_sl;
+            const IO* xk = static_cast<const IO*>(p.x) + ex;
+            const IO* dk = static_cast<const IO*>(p.delta) + ed;
+            const IO* yk = static_cast<const IO*>(p.dy) + ey;
+            const IO* zk = static_cast<const IO*>(p.z) + ez;
+            const IO* ypk = static_cast<const IO*>(p.ypre) + ey;
+            const IO* Bk = static_cast<const IO*>(p.Bm) + ebc;
+            const IO* Ck = static_cast<const IO*>(p.C) + ebc;
+            const uint32_t wx = window_bytes(endx, ex, kES), wd = window_bytes(endd, ed, kES);
+            const uint32_t wy = window_bytes(endy, ey, kES), wbc = window_bytes(endbc, ebc, kES);
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                oz[j] = offzi[j];
-                ox[j] = offx[j];
-                od[j] = offd[j];
-                oy[j] = offy[j];
-            }
-#pragma unroll
-            for (int r = 0; r < kBcPer; ++r) ob[r] = offbc[r];
-            if ((c + 1) * kTile > p.L) {
-                const int tmax = p.L - c * kTile - 1;
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const uint32_t tc = (uint32_t)min(4 * qi + j, tmax);
-                    ox[j] = (tc * (uint32_t)p.u_sl + (uint32_t)cic * (uint32_t)p.u_sd) * kES;
-                    od[j] = (tc * (uint32_t)p.d_sl + (uint32_t)cic * (uint32_t)p.d_sd) * kES;
-                    oy[j] = (tc * (uint32_t)p.y_sl + (uint32_t)cic * (uint32_t)p.y_sd) * kES;
-                    oz[j] = (tc * (uint32_t)p.z_sl + (uint32_t)cic * (uint32_t)p.z_sd) * kES;
-                }
-#pragma unroll
-                for (int r = 0; r < kBcPer; ++r)
-                    ob[r] = ((uint32_t)min(bct[r], tmax) * (uint32_t)p.bc_sl + (uint32_t)min(bcn[r], p.N - 1)) * kES;
-            }
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                raw.x[j] = ld_off(xk, ox[j]);
-                raw.d[j] = ld_off(dk, od[j]);
-                raw.y[j] = ld_off(yk, oy[j]);
+                raw.x[j] = ld_off(xk, offx, j * sx, wx);
+                raw.d[j] = ld_off(dk, offd, j * sd, wd);
+                raw.y[j] = ld_off(yk, offy, j * sy, wy);
                 if constexpr (HAS_Z) {
-                    raw.z[j] = ld_off(zk, oz[j]);
-                    raw.yp[j] = ld_off(ypk, oy[j]);
+                    raw.z[j] = ld_off(zk, offzi, j * sz, window_bytes(endz, ez, kES));
+                    raw.yp[j] = ld_off(ypk, offy, j * sy, wy);
                 }
             }
 #pragma unroll
             for (int r = 0; r < kBcPer; ++r) {
-                raw.b[r] = ld_off(Bk, ob[r]);
-                raw.c[r] = ld_off(Ck, ob[r]);
+                raw.b[r] = ld_off(Bk, offbc[r], 0, wbc);
+                raw.c[r] = ld_off(Ck, offbc[r], 0, wbc);
             }
         };
         auto stage_tile = [&](int k, const Raw& raw) {
@@ -305,11 +284,11 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
                 IO* dzk = dzg + (int64_t)c * kTile * p.g_sl;
                 if (!ragged) {
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) st_off(dzk, offz[j], from_float<IO>(dzv[j]));
+                    for (int j = 0; j < 4; ++j) st_off(dzk, offz, from_float<IO>(dzv[j]), j * sg);
                 } else {
                     const int t0 = c * kTile + 4 * qi;
                     for (int j = 0; j < 4; ++j)
-                        if (ci_ok && t0 + j < p.L) st_off(dzk, offz[j], from_float<IO>(dzv[j]));
+                        if (ci_ok && t0 + j < p.L) st_off(dzk, offz, from_float<IO>(dzv[j]), j * sg);
                 }
             }
             if (ragged) {
@@ -386,8 +365,8 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
             if (group_full && (c + 1) * kTile <= p.L && fw_vec) {
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
-                    st_off(dxk, offg[j], from_float<IO>(dxv[j]));
-                    st_off(ddk, offg[j], from_float<IO>(dv[j]));
+                    st_off(dxk, offg, from_float<IO>(dxv[j]), j * sg);
+                    st_off(ddk, offg, from_float<IO>(dv[j]), j * sg);
                 }
                 if constexpr (kFw == 2)
                     st_off(reinterpret_cast<float2*>(fwk), fw_off, make_float2(fw[0], fw[1]));
@@ -397,8 +376,8 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
                 const int t0 = c * kTile + 4 * qo;
                 for (int j = 0; j < 4; ++j)
                     if (co_ok && t0 + j < p.L) {
-                        st_off(dxk, offg[j], from_float<IO>(dxv[j]));
-                        st_off(ddk, offg[j], from_float<IO>(dv[j]));
+                        st_off(dxk, offg, from_float<IO>(dxv[j]), j * sg);
+                        st_off(ddk, offg, from_float<IO>(dv[j]), j * sg);
                     }
                 for (int i = 0; i < kFw; ++i)
                     if (c * kTile + fw_tt < p.L && fw_n + i < p.N) st_off(fwk, fw_off + 4u * i, fw[i]);
