@@ -175,13 +175,19 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
         const uint32_t offz = ((uint32_t)(4 * qi) * (uint32_t)p.g_sl + (uint32_t)cic * (uint32_t)p.g_sd) * kES;  // dz
         const uint32_t sx = (uint32_t)p.u_sl * kES, sd = (uint32_t)p.d_sl * kES, sy = (uint32_t)p.y_sl * kES;
         const uint32_t sz = (uint32_t)p.z_sl * kES, sg = (uint32_t)p.g_sl * kES;
-        // one past the last element of each input tensor, relative to its first: the loads of a
-        // ragged tile may run past the sequence end but never past this (they are windowed)
-        const int64_t endx = (p.batch - 1) * p.u_sb + (p.L - 1) * p.u_sl + (p.ED - 1) * p.u_sd + 1;
-        const int64_t endd = (p.batch - 1) * p.d_sb + (p.L - 1) * p.d_sl + (p.ED - 1) * p.d_sd + 1;
-        const int64_t endy = (p.batch - 1) * p.y_sb + (p.L - 1) * p.y_sl + (p.ED - 1) * p.y_sd + 1;
-        const int64_t endz = (p.batch - 1) * p.z_sb + (p.L - 1) * p.z_sl + (p.ED - 1) * p.z_sd + 1;
-        const int64_t endbc = (p.batch - 1) * p.bc_sb + (p.L - 1) * p.bc_sl + p.N;
+        // tensor origins of this (batch row, channel group)
+        const IO* const xb = static_cast<const IO*>(p.x) + (b * p.u_sb + (int64_t)d0 * p.u_sd);
+        const IO* const db = static_cast<const IO*>(p.delta) + (b * p.d_sb + (int64_t)d0 * p.d_sd);
+        const IO* const yb = static_cast<const IO*>(p.dy) + (b * p.y_sb + (int64_t)d0 * p.y_sd);
+        const IO* const zb = static_cast<const IO*>(p.z) + (b * p.z_sb + (int64_t)d0 * p.z_sd);
+        const IO* const ypb = static_cast<const IO*>(p.ypre) + (b * p.y_sb + (int64_t)d0 * p.y_sd);
+        const IO* const Bb = static_cast<const IO*>(p.Bm) + b * p.bc_sb;
+        const IO* const Cb = static_cast<const IO*>(p.C) + b * p.bc_sb;
+        // Loads of a ragged tile run past the sequence end.  That is harmless (the values are
+        // masked at staging) as long as the address is inside the tensor, which only the last
+        // tile of the last batch row can violate: that one tile is read through windows that
+        // end with the tensor (out-of-window loads return zero).
+        const bool edge_row = b == p.batch - 1 && ntiles * kTile > p.L;
         // B/C of a tile: kTile * NP elements each, kBcPer per service thread, step fastest
         constexpr int kBcPer = NP * kTile / (kSvc * kWave);
         static_assert(NP * kTile % (kSvc * kWave) == 0, "whole elements per thread");
@@ -225,27 +231,30 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
             // as whatever follows inside the tensor (or zero past its end) and masked at staging
             const int k = min(kk, ntiles - 1);
             const int c = chunk_of(k);
-            const int64_t ex = b * p.u_sb + (int64_t)d0 * p.u_sd + (int64_t)c * kTile * p.u_sl;
-            const int64_t ed = b * p.d_sb + (int64_t)d0 * p.d_sd + (int64_t)c * kTile * p.d_sl;
-            const int64_t ey = b * p.y_sb + (int64_t)d0 * p.y_sd + (int64_t)c * kTile * p.y_sl;
-            const int64_t ez = b * p.z_sb + (int64_t)d0 * p.z_sd + (int64_t)c * kTile * p.z_sl;
-            const int64_t ebc = b * p.bc_sb + (int64_t)c * kTile * p.bc_sl;
-            const IO* xk = static_cast<const IO*>(p.x) + ex;
-            const IO* dk = static_cast<const IO*>(p.delta) + ed;
-            const IO* yk = static_cast<const IO*>(p.dy) + ey;
-            const IO* zk = static_cast<const IO*>(p.z) + ez;
-            const IO* ypk = static_cast<const IO*>(p.ypre) + ey;
-            const IO* Bk = static_cast<const IO*>(p.Bm) + ebc;
-            const IO* Ck = static_cast<const IO*>(p.C) + ebc;
-            const uint32_t wx = window_bytes(endx, ex, kES), wd = window_bytes(endd, ed, kES);
-            const uint32_t wy = window_bytes(endy, ey, kES), wbc = window_bytes(endbc, ebc, kES);
+            const IO* xk = xb + (int64_t)c * kTile * p.u_sl;
+            const IO* dk = db + (int64_t)c * kTile * p.d_sl;
+            const IO* yk = yb + (int64_t)c * kTile * p.y_sl;
+            const IO* zk = zb + (int64_t)c * kTile * p.z_sl;
+            const IO* ypk = ypb + (int64_t)c * kTile * p.y_sl;
+            const IO* Bk = Bb + (int64_t)c * kTile * p.bc_sl;
+            const IO* Ck = Cb + (int64_t)c * kTile * p.bc_sl;
+            uint32_t wx = 0xffffffffu, wd = wx, wy = wx, wz = wx, wbc = wx;
+            if (edge_row && c == ntiles - 1) {
+                const int64_t row = (int64_t)(p.L - 1 - c * kTile);  // last valid step of the tile
+                const int64_t chn = p.ED - 1 - d0;                   // last valid channel of the group
+                wx = window_bytes(row * p.u_sl + chn * p.u_sd + 1, 0, kES);
+                wd = window_bytes(row * p.d_sl + chn * p.d_sd + 1, 0, kES);
+                wy = window_bytes(row * p.y_sl + chn * p.y_sd + 1, 0, kES);
+                wz = window_bytes(row * p.z_sl + chn * p.z_sd + 1, 0, kES);
+                wbc = window_bytes(row * p.bc_sl + p.N, 0, kES);
+            }
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 raw.x[j] = ld_off(xk, offx, j * sx, wx);
                 raw.d[j] = ld_off(dk, offd, j * sd, wd);
                 raw.y[j] = ld_off(yk, offy, j * sy, wy);
                 if constexpr (HAS_Z) {
-                    raw.z[j] = ld_off(zk, offzi, j * sz, window_bytes(endz, ez, kES));
+                    raw.z[j] = ld_off(zk, offzi, j * sz, wz);
                     raw.yp[j] = ld_off(ypk, offy, j * sy, wy);
                 }
             }
