@@ -184,10 +184,10 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
         const IO* const Bb = static_cast<const IO*>(p.Bm) + b * p.bc_sb;
         const IO* const Cb = static_cast<const IO*>(p.C) + b * p.bc_sb;
         // Loads of a ragged tile run past the sequence end.  That is harmless (the values are
-        // masked at staging) as long as the address is inside the tensor, which only the last
-        // tile of the last batch row can violate: that one tile is read through windows that
-        // end with the tensor (out-of-window loads return zero).
-        const bool edge_row = b == p.batch - 1 && ntiles * kTile > p.L;
+        // masked at staging) as long as the address is inside the tensor: the ragged tile is
+        // read through windows that end with the tensor's last element, whatever the strides
+        // (out-of-window loads return zero).
+        const bool ragged_end = ntiles * kTile > p.L;
         // B/C of a tile: kTile * NP elements each, kBcPer per service thread, step fastest
         constexpr int kBcPer = NP * kTile / (kSvc * kWave);
         static_assert(NP * kTile % (kSvc * kWave) == 0, "whole elements per thread");
@@ -239,14 +239,18 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
             const IO* Bk = Bb + (int64_t)c * kTile * p.bc_sl;
             const IO* Ck = Cb + (int64_t)c * kTile * p.bc_sl;
             uint32_t wx = 0xffffffffu, wd = wx, wy = wx, wz = wx, wbc = wx;
-            if (edge_row && c == ntiles - 1) {
-                const int64_t row = (int64_t)(p.L - 1 - c * kTile);  // last valid step of the tile
-                const int64_t chn = p.ED - 1 - d0;                   // last valid channel of the group
-                wx = window_bytes(row * p.u_sl + chn * p.u_sd + 1, 0, kES);
-                wd = window_bytes(row * p.d_sl + chn * p.d_sd + 1, 0, kES);
-                wy = window_bytes(row * p.y_sl + chn * p.y_sd + 1, 0, kES);
-                wz = window_bytes(row * p.z_sl + chn * p.z_sd + 1, 0, kES);
-                wbc = window_bytes(row * p.bc_sl + p.N, 0, kES);
+            if (ragged_end && c == ntiles - 1) {
+                // elements from this tile's origin to one past the tensor's last element
+                const int64_t tb = (int64_t)c * kTile;
+                auto left = [&](int64_t sb_, int64_t sl_, int64_t sd_, int64_t width) {
+                    const int64_t end = (p.batch - 1) * sb_ + (p.L - 1) * sl_ + (width - 1) * sd_ + 1;
+                    return window_bytes(end, b * sb_ + tb * sl_ + (int64_t)d0 * sd_, kES);
+                };
+                wx = left(p.u_sb, p.u_sl, p.u_sd, p.ED);
+                wd = left(p.d_sb, p.d_sl, p.d_sd, p.ED);
+                wy = left(p.y_sb, p.y_sl, p.y_sd, p.ED);
+                wz = left(p.z_sb, p.z_sl, p.z_sd, p.ED);
+                wbc = window_bytes((p.batch - 1) * p.bc_sb + (p.L - 1) * p.bc_sl + p.N, b * p.bc_sb + tb * p.bc_sl, kES);
             }
 #pragma unroll
             for (int j = 0; j < 4; ++j) {

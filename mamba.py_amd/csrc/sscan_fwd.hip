@@ -200,14 +200,18 @@ __global__ void __launch_bounds__((NW + kService) * kWave) sscan_fwd_kernel(cons
             const IO* const xg = static_cast<const IO*>(p.x) + (b * p.u_sb + (int64_t)d0 * p.u_sd);
             const IO* const dg = static_cast<const IO*>(p.delta) + (b * p.d_sb + (int64_t)d0 * p.d_sd);
             const IO* const zg = static_cast<const IO*>(p.z) + (b * p.z_sb + (int64_t)d0 * p.z_sd);
-            uint32_t offx[4], offd[4], offz[4];
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                // byte offsets (see ld_off)
-                offx[j] = ((uint32_t)(4 * qi + j) * (uint32_t)p.u_sl + (uint32_t)cic * (uint32_t)p.u_sd) * kES;
-                offd[j] = ((uint32_t)(4 * qi + j) * (uint32_t)p.d_sl + (uint32_t)cic * (uint32_t)p.d_sd) * kES;
-                offz[j] = ((uint32_t)(4 * qi + j) * (uint32_t)p.z_sl + (uint32_t)cic * (uint32_t)p.z_sd) * kES;
-            }
+            // byte offset of the item's first step (one vector register per tensor, see ld_off);
+            // its other three steps are one row stride further each, which goes into the scalar
+            // offset of the access
+            const uint32_t offx = ((uint32_t)(4 * qi) * (uint32_t)p.u_sl + (uint32_t)cic * (uint32_t)p.u_sd) * kES;
+            const uint32_t offd = ((uint32_t)(4 * qi) * (uint32_t)p.d_sl + (uint32_t)cic * (uint32_t)p.d_sd) * kES;
+            const uint32_t offz = ((uint32_t)(4 * qi) * (uint32_t)p.z_sl + (uint32_t)cic * (uint32_t)p.z_sd) * kES;
+            const uint32_t sx = (uint32_t)p.u_sl * kES, sd = (uint32_t)p.d_sl * kES, sz = (uint32_t)p.z_sl * kES;
+            // Loads of a ragged tile run past the sequence end.  That is harmless (the values
+            // are masked at staging) as long as the address is inside the tensor: the ragged
+            // tile is read through windows that end with the tensor's last element, whatever
+            // the strides (out-of-window loads return zero).
+            const bool ragged_end = ntiles * kTile > p.L;
             const bool group_full = cmax == kWave - 1;
             // B/C of a tile: kTile * NP elements each, kBcPer per loader thread, step fastest
             constexpr int kBcPer = kBcast ? NP * kTile / (kLoaders * kWave) : 0;
@@ -237,48 +241,37 @@ __global__ void __launch_bounds__((NW + kService) * kWave) sscan_fwd_kernel(cons
                        : reinterpret_cast<const float4*>(p.bcpack) + (int64_t)b * ntiles * kPackVec + min(item, kPackVec - 1);
             struct Raw { IO x[4], d[4], z[4], b[kBcPer > 0 ? kBcPer : 1], c[kBcPer > 0 ? kBcPer : 1]; float4 warm; };
             auto load_tile = [&](int kk, Raw& raw) {
-                // tiles and steps beyond the sequence end are clamped to the last one, so the
-                // loads stay in bounds; only the offsets depend on the (uniform) branch, the
-                // loads themselves are unconditional (a branch around them would force a wait
-                // on their data)
+                // tiles beyond the last one are clamped to it; the loads are unconditional (a
+                // branch around them would force a wait on their data)
                 const int k = min(kk, ntiles - 1);
                 const IO* xk = xg + (int64_t)k * kTile * p.u_sl;
                 const IO* dk = dg + (int64_t)k * kTile * p.d_sl;
                 const IO* zk = zg + (int64_t)k * kTile * p.z_sl;
                 const IO* Bk = Bg + (int64_t)k * kTile * p.bc_sl;
                 const IO* Ck = Cg + (int64_t)k * kTile * p.bc_sl;
-                uint32_t ox[4], od[4], oz[4], ob[kBcPer > 0 ? kBcPer : 1];
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    ox[j] = offx[j];
-                    od[j] = offd[j];
-                    oz[j] = offz[j];
-                }
-#pragma unroll
-                for (int r = 0; r < kBcPer; ++r) ob[r] = offbc[r];
-                if ((k + 1) * kTile > p.L) {
-                    const int tmax = p.L - k * kTile - 1;
-#pragma unroll
-                    for (int j = 0; j < 4; ++j) {
-                        const uint32_t tc = (uint32_t)min(4 * qi + j, tmax);
-                        ox[j] = (tc * (uint32_t)p.u_sl + (uint32_t)cic * (uint32_t)p.u_sd) * kES;
-                        od[j] = (tc * (uint32_t)p.d_sl + (uint32_t)cic * (uint32_t)p.d_sd) * kES;
-                        oz[j] = (tc * (uint32_t)p.z_sl + (uint32_t)cic * (uint32_t)p.z_sd) * kES;
-                    }
-#pragma unroll
-                    for (int r = 0; r < kBcPer; ++r)
-                        ob[r] = ((uint32_t)min(bct[r], tmax) * (uint32_t)p.bc_sl + (uint32_t)min(bcn[r], p.N - 1)) * kES;
+                uint32_t wx = 0xffffffffu, wd = wx, wz = wx, wbc = wx;
+                if (ragged_end && k == ntiles - 1) {
+                    // elements from this tile's origin to one past the tensor's last element
+                    const int64_t tb = (int64_t)k * kTile;
+                    auto left = [&](int64_t sb_, int64_t sl_, int64_t sd_, int64_t width) {
+                        const int64_t end = (p.batch - 1) * sb_ + (p.L - 1) * sl_ + (width - 1) * sd_ + 1;
+                        return window_bytes(end, b * sb_ + tb * sl_ + (int64_t)d0 * sd_, kES);
+                    };
+                    wx = left(p.u_sb, p.u_sl, p.u_sd, p.ED);
+                    wd = left(p.d_sb, p.d_sl, p.d_sd, p.ED);
+                    wz = left(p.z_sb, p.z_sl, p.z_sd, p.ED);
+                    wbc = window_bytes((p.batch - 1) * p.bc_sb + (p.L - 1) * p.bc_sl + p.N, b * p.bc_sb + tb * p.bc_sl, kES);
                 }
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
-                    raw.x[j] = ld_off(xk, ox[j]);
-                    raw.d[j] = ld_off(dk, od[j]);
-                    if (has_z) raw.z[j] = ld_off(zk, oz[j]);
+                    raw.x[j] = ld_off(xk, offx, j * sx, wx);
+                    raw.d[j] = ld_off(dk, offd, j * sd, wd);
+                    if (has_z) raw.z[j] = ld_off(zk, offz, j * sz, wz);
                 }
 #pragma unroll
                 for (int r = 0; r < kBcPer; ++r) {
-                    raw.b[r] = ld_off(Bk, ob[r]);
-                    raw.c[r] = ld_off(Ck, ob[r]);
+                    raw.b[r] = ld_off(Bk, offbc[r], 0, wbc);
+                    raw.c[r] = ld_off(Ck, offbc[r], 0, wbc);
                 }
                 if (!kBcast) raw.warm = warm[(int64_t)k * kPackVec];
             };
@@ -358,10 +351,8 @@ __global__ void __launch_bounds__((NW + kService) * kWave) sscan_fwd_kernel(cons
             const int qo = p.out_tmajor ? item % NQ : item / kWave;
             const bool co_ok = co <= cmax;
             const int q4 = 4 * qo;
-            uint32_t offy[4];
-#pragma unroll
-            for (int j = 0; j < 4; ++j)
-                offy[j] = ((uint32_t)(q4 + j) * (uint32_t)p.y_sl + (uint32_t)min(co, cmax) * (uint32_t)p.y_sd) * kES;
+            const uint32_t offy = ((uint32_t)q4 * (uint32_t)p.y_sl + (uint32_t)min(co, cmax) * (uint32_t)p.y_sd) * kES;
+            const uint32_t sy = (uint32_t)p.y_sl * kES;
             IO* const yg = static_cast<IO*>(p.y) + (b * p.y_sb + (int64_t)d0 * p.y_sd);
             IO* const ypg = static_cast<IO*>(p.ypre) + (b * p.y_sb + (int64_t)d0 * p.y_sd);
             auto reduce_store = [&](int k) {
@@ -378,7 +369,7 @@ __global__ void __launch_bounds__((NW + kService) * kWave) sscan_fwd_kernel(cons
                     if (p.ypre) {
                         const float pv[4] = {s.x, s.y, s.z, s.w};
                         for (int j = 0; j < 4; ++j)
-                            if (co_ok && t0 + j < p.L) st_off(ypk, offy[j], from_float<IO>(pv[j]));
+                            if (co_ok && t0 + j < p.L) st_off(ypk, offy, from_float<IO>(pv[j]), j * sy);
                     }
                     const float4 g = *reinterpret_cast<const float4*>(&sG[k & 3][co][q4]);
                     s.x *= g.x; s.y *= g.y; s.z *= g.z; s.w *= g.w;
@@ -386,10 +377,10 @@ __global__ void __launch_bounds__((NW + kService) * kWave) sscan_fwd_kernel(cons
                 const float sv[4] = {s.x, s.y, s.z, s.w};
                 if (co_ok && t0 + 3 < p.L) {
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) st_off(yk, offy[j], from_float<IO>(sv[j]));
+                    for (int j = 0; j < 4; ++j) st_off(yk, offy, from_float<IO>(sv[j]), j * sy);
                 } else if (co_ok) {
                     for (int j = 0; j < 4; ++j)
-                        if (t0 + j < p.L) st_off(yk, offy[j], from_float<IO>(sv[j]));
+                        if (t0 + j < p.L) st_off(yk, offy, from_float<IO>(sv[j]), j * sy);
                 }
             };
             // the reducers run one tile behind the scan waves

@@ -193,6 +193,34 @@ def test_gated_backward_fast_equals_general_kernel(pkg, dev, monkeypatch):
         assert rel_err(a[k], b[k]) <= 2e-6, k
 
 
+
+def test_time_outermost_memory_and_ragged_tail(pkg, dev):
+    # (L, B, ED) memory viewed as (B, L, ED): the time stride is the largest one, so a ragged
+    # last tile of ANY batch row would run off the allocation if loads were not windowed;
+    # also a batch-expanded (stride 0) delta
+    Bs, L, ED, N = 3, 21, 70, 16
+    inp = so.make_inputs(Bs, L, ED, N, seed=91)
+    ref = c_oracle.sscan_fwd_bwd(**inp)
+    names = ("x", "delta", "A", "B", "C", "D")
+
+    def lbe(t):  # same values, time-outermost memory
+        return t.to(dev).permute(1, 0, 2).contiguous().permute(1, 0, 2).requires_grad_()
+
+    args = [lbe(inp[k]) if k in ("x", "delta", "B", "C") else inp[k].to(dev).requires_grad_() for k in names]
+    assert args[0].stride() == (ED, Bs * ED, 1)
+    y = pkg.selective_scan_fn(*args)
+    y.backward(lbe(inp["dy"]).detach())
+    got = dict(y=y, **{k: a.grad for k, a in zip(GRAD_KEYS, args)})
+    _check(got, ref, TOL[torch.float32], "time-outermost")
+
+    d1 = inp["delta"][:1]
+    with torch.no_grad():
+        y_exp = pkg.selective_scan_fn(inp["x"].to(dev), d1.to(dev).expand(Bs, L, ED), inp["A"].to(dev),
+                                      inp["B"].to(dev), inp["C"].to(dev), inp["D"].to(dev))
+    ref_exp = c_oracle.sscan_fwd(inp["x"], d1.expand(Bs, L, ED).contiguous(), inp["A"], inp["B"], inp["C"], inp["D"])
+    assert rel_err(y_exp, ref_exp) <= TOL[torch.float32]
+
+
 def test_bitwise_reproducible(pkg, dev):
     inp = so.make_inputs(2, 130, 200, 16, seed=61)
     a = run_gpu_fwd_bwd(pkg, inp, dev)
