@@ -163,6 +163,20 @@ int mpa_conv1d_bwd(const mpa_conv_shape* s, const void* x, const float* weight, 
                    void* workspace, size_t workspace_bytes, void* stream);
 size_t mpa_conv1d_bwd_workspace_bytes(const mpa_conv_shape* s);
 
+/* ---- RMSNorm --------------------------------------------------------------------------------
+ * Replaces RMSNorm.forward (mambapy/mamba.py:427-433): y = x * rsqrt(mean(x^2, -1) + eps) * weight
+ * on `rows` contiguous rows of `d` elements (io_dtype; d a multiple of 4 (float32) / 8 (bfloat16),
+ * d <= 2048 / 4096), weight (d) float32 or NULL (the muP variant has none), and its gradient:
+ * dx (io_dtype) and dweight (d) float32, overwritten.  rstd (rows) float32 is an optional output.
+ * Pointers to x, y, dy, dx must be 16-byte aligned.
+ */
+int mpa_rmsnorm_fwd(const void* x, const float* weight, void* y, float* rstd, int64_t rows, int64_t d,
+                    float eps, int32_t io_dtype, void* stream);
+int mpa_rmsnorm_bwd(const void* x, const float* weight, const void* dy, void* dx, float* dweight,
+                    int64_t rows, int64_t d, float eps, int32_t io_dtype, void* workspace,
+                    size_t workspace_bytes, void* stream);
+size_t mpa_rmsnorm_bwd_workspace_bytes(int64_t rows, int64_t d);
+
 /* ---- generic first-order scan -----------------------------------------------------------
  * Replaces pscan = PScan.apply (mambapy/pscan.py:226; forward :151-186, backward :188-224)
  * for callers that hold materialised A, X of logical shape (batch, seqlen, dim, dstate):

@@ -18,7 +18,8 @@ MPA_MAX_DSTATE = 256
 EXPORTS = ("mpa_version", "mpa_arch", "mpa_status_string", "mpa_sscan_fwd",
            "mpa_sscan_ckpt_elems", "mpa_sscan_fwd_workspace_bytes", "mpa_sscan_bwd", "mpa_sscan_bwd_workspace_bytes",
            "mpa_pscan_fwd", "mpa_pscan_bwd", "mpa_ssm_step",
-           "mpa_conv1d_fwd", "mpa_conv1d_bwd", "mpa_conv1d_bwd_workspace_bytes")
+           "mpa_conv1d_fwd", "mpa_conv1d_bwd", "mpa_conv1d_bwd_workspace_bytes",
+           "mpa_rmsnorm_fwd", "mpa_rmsnorm_bwd", "mpa_rmsnorm_bwd_workspace_bytes")
 
 
 class SscanShape(ctypes.Structure):
@@ -81,6 +82,11 @@ def load():
     lib.mpa_conv1d_bwd.argtypes = [cp] + [vp] * 9 + [sz, vp]
     lib.mpa_conv1d_bwd_workspace_bytes.argtypes = [cp]
     lib.mpa_conv1d_bwd_workspace_bytes.restype = sz
+    f32 = ctypes.c_float
+    lib.mpa_rmsnorm_fwd.argtypes = [vp] * 4 + [i64, i64, f32, i32, vp]
+    lib.mpa_rmsnorm_bwd.argtypes = [vp] * 5 + [i64, i64, f32, i32, vp, sz, vp]
+    lib.mpa_rmsnorm_bwd_workspace_bytes.argtypes = [i64, i64]
+    lib.mpa_rmsnorm_bwd_workspace_bytes.restype = sz
     for name in EXPORTS:
         getattr(lib, name)
     _lib = lib

@@ -13,7 +13,7 @@ from concurrent.futures import ThreadPoolExecutor
 _HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(_HERE, "csrc")
 LIB_PATH = os.path.join(CSRC, "libmambapy_amd.so")
-SOURCES = ["sscan_fwd.hip", "sscan_bwd.hip", "sscan_bwd_fast.hip", "pscan.hip", "step.hip", "conv1d.hip"]
+SOURCES = ["sscan_fwd.hip", "sscan_bwd.hip", "sscan_bwd_fast.hip", "pscan.hip", "step.hip", "conv1d.hip", "rmsnorm.hip"]
 ARCH = "gfx950"
 HIPCC_FLAGS = ["-O3", f"--offload-arch={ARCH}", "-fPIC", "-std=c++17",
                "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",

@@ -17,6 +17,7 @@ import torch.nn as nn
 import torch.nn.functional as F
 
 from .conv import causal_conv1d_fn
+from .norm import rmsnorm_fn, rmsnorm_supported
 from .scan import selective_scan, selective_scan_fn, ssm_step
 
 
@@ -73,6 +74,8 @@ class RMSNorm(nn.Module):
             self.weight = nn.Parameter(torch.ones(d_model))
 
     def forward(self, x):
+        if x.is_cuda and rmsnorm_supported(x):
+            return rmsnorm_fn(x, None if self.use_mup else self.weight, self.eps)
         y = x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + self.eps)
         return y if self.use_mup else y * self.weight
 

@@ -1,0 +1,53 @@
+"""GPU parity of the RMSNorm kernel against a float64 restatement of mambapy/mamba.py:427-433."""
+import pytest
+import torch
+
+from util import TOL, rel_err
+
+pytestmark = pytest.mark.gpu
+
+
+def rmsnorm_ref(x, weight, eps):
+    # output = x * rsqrt(x.pow(2).mean(-1, keepdim=True) + eps) [* weight]
+    y = x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps)
+    return y if weight is None else y * weight
+
+
+@pytest.mark.parametrize("shape,dtype,with_w", [
+    ((2, 37, 768), torch.float32, True), ((3, 5, 64), torch.float32, True), ((1, 1, 8), torch.bfloat16, True),
+    ((2, 129, 2560), torch.bfloat16, True), ((4, 33, 2048), torch.float32, False), ((7, 4096), torch.bfloat16, True),
+    ((5, 3, 4), torch.float32, True),
+])
+def test_rmsnorm_forward_backward(pkg, dev, shape, dtype, with_w):
+    g = torch.Generator().manual_seed(sum(shape))
+    x = (torch.randn(*shape, generator=g) * 1.5 + 0.3).to(dtype)
+    w = (torch.randn(shape[-1], generator=g) * 0.5 + 1.0).to(dtype) if with_w else None
+    dy = torch.randn(*shape, generator=g).to(dtype)
+    eps = 1e-5
+    xr = x.double().requires_grad_()
+    wr = None if w is None else w.double().requires_grad_()
+    yr = rmsnorm_ref(xr, wr, eps)
+    yr.backward(dy.double())
+    xg = x.to(dev).requires_grad_()
+    wg = None if w is None else w.to(dev).requires_grad_()
+    y = pkg.rmsnorm_fn(xg, wg, eps)
+    y.backward(dy.to(dev))
+    tol = TOL[dtype]
+    assert rel_err(y, yr) <= tol
+    assert rel_err(xg.grad, xr.grad) <= tol
+    if w is not None:
+        assert rel_err(wg.grad, wr.grad) <= tol
+
+
+def test_rmsnorm_module_uses_kernel_and_matches(pkg, dev):
+    torch.manual_seed(3)
+    norm = pkg.RMSNorm(96).to(dev)
+    with torch.no_grad():
+        norm.weight.mul_(torch.rand(96, device=dev) + 0.5)
+    x = torch.randn(4, 10, 96, device=dev)
+    want = rmsnorm_ref(x.double(), norm.weight.double(), norm.eps)
+    assert rel_err(norm(x), want) <= TOL[torch.float32]
+    # an unsupported width falls back to the same formula on PyTorch kernels
+    norm2 = pkg.RMSNorm(10).to(dev)
+    x2 = torch.randn(3, 10, device=dev)
+    assert rel_err(norm2(x2), rmsnorm_ref(x2.double(), norm2.weight.double(), norm2.eps)) <= TOL[torch.float32]
