@@ -11,7 +11,7 @@
 
 namespace mpa {
 
-constexpr int kNormRowsPerWave = 8;  // backward: rows walked by one wave (dweight partials per wave)
+constexpr int kNormRowsPerWave = 16;  // backward: rows walked by one wave (dweight partials per wave)
 
 template <typename IO>
 struct RowVec;
@@ -148,19 +148,20 @@ __global__ void __launch_bounds__(256) rmsnorm_bwd_kernel(const IO* __restrict__
     }
 }
 
-// dweight[c] = sum over the per-wave partial rows, fixed order (64 columns x 16 row groups per block)
+// dweight[c] = sum over the per-wave partial rows, fixed order (32 columns x 32 row groups per block)
+constexpr int kNormFinCols = 32, kNormFinRows = 32;
 __global__ void __launch_bounds__(1024) rmsnorm_bwd_finish_kernel(const float* part, float* dweight, int d,
                                                                   int64_t nparts) {
-    __shared__ float acc[16][64];
-    const int col = threadIdx.x % 64, rg = threadIdx.x / 64;
-    const int c = blockIdx.x * 64 + col;
+    __shared__ float acc[kNormFinRows][kNormFinCols + 1];
+    const int col = threadIdx.x % kNormFinCols, rg = threadIdx.x / kNormFinCols;
+    const int c = blockIdx.x * kNormFinCols + col;
     float s = 0.0f;
     if (c < d)
-        for (int64_t q = rg; q < nparts; q += 16) s += part[q * d + c];
+        for (int64_t q = rg; q < nparts; q += kNormFinRows) s += part[q * d + c];
     acc[rg][col] = s;
     __syncthreads();
     if (rg != 0 || c >= d) return;
-    for (int r = 1; r < 16; ++r) s += acc[r][col];
+    for (int r = 1; r < kNormFinRows; ++r) s += acc[r][col];
     dweight[c] = s;
 }
 
@@ -237,7 +238,7 @@ extern "C" int mpa_rmsnorm_bwd(const void* x, const float* weight, const void* d
     if (rc != MPA_OK || !weight) return rc;
     // rows of the partial buffer beyond the last wave of a partially filled block were written
     // by waves that own no row (all zeros), so every one of the grid's waves counts
-    hipLaunchKernelGGL(rmsnorm_bwd_finish_kernel, dim3((unsigned)((d + 63) / 64)), dim3(1024), 0, st, part, dweight,
+    hipLaunchKernelGGL(rmsnorm_bwd_finish_kernel, dim3((unsigned)((d + kNormFinCols - 1) / kNormFinCols)), dim3(1024), 0, st, part, dweight,
                        (int)d, (int64_t)grid.x * 4);
     return check_launch();
 }
