@@ -30,6 +30,10 @@ names the lines it follows.  What pins each function (see tests/test_oracle.py):
   causal_conv1d_ref      mambapy/mamba.py:217-221.  Pinned against the definition written
                          as explicit loops on small cases and against nn.Conv1d with
                          padding=K-1 truncated to L (the reference's own expression).
+  rmsnorm_ref            mambapy/mamba.py:427-433.  Pinned by a hand-computed vector
+                         ([3,4] -> [3,4]/sqrt(12.5)), by explicit loops, by unit mean
+                         square of the output rows at eps=0 and by invariance to a
+                         rescaling of the input row at eps=0.
 
 Floating-point rounding of torch's own elementwise kernels is not pinned by any
 reference fixture ("parity unpinned" at the torch boundary; irrelevant at the
@@ -312,6 +316,13 @@ def causal_conv1d_ref(x, weight, bias=None, window=None, silu=True):
     y = F.conv1d(torch.cat([left.to(xt.dtype), xt], dim=2), weight, bias, groups=xt.shape[1])
     y = y.transpose(1, 2)
     return F.silu(y) if silu else y
+
+
+def rmsnorm_ref(x, weight=None, eps=1e-5):
+    """x * rsqrt(mean(x^2, last axis) + eps) [* weight]  (mambapy/mamba.py:427-433;
+    no weight under muP, :421-424)."""
+    y = x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps)
+    return y if weight is None else y * weight
 
 
 def softplus_ref(v):

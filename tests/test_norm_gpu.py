@@ -1,16 +1,11 @@
-"""GPU parity of the RMSNorm kernel against a float64 restatement of mambapy/mamba.py:427-433."""
+"""GPU parity of the RMSNorm kernel against the float64 oracle (mambapy/mamba.py:427-433)."""
 import pytest
 import torch
 
+from oracle import scan_oracle as so
 from util import TOL, rel_err
 
 pytestmark = pytest.mark.gpu
-
-
-def rmsnorm_ref(x, weight, eps):
-    # output = x * rsqrt(x.pow(2).mean(-1, keepdim=True) + eps) [* weight]
-    y = x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps)
-    return y if weight is None else y * weight
 
 
 @pytest.mark.parametrize("shape,dtype,with_w", [
@@ -26,7 +21,7 @@ def test_rmsnorm_forward_backward(pkg, dev, shape, dtype, with_w):
     eps = 1e-5
     xr = x.double().requires_grad_()
     wr = None if w is None else w.double().requires_grad_()
-    yr = rmsnorm_ref(xr, wr, eps)
+    yr = so.rmsnorm_ref(xr, wr, eps)
     yr.backward(dy.double())
     xg = x.to(dev).requires_grad_()
     wg = None if w is None else w.to(dev).requires_grad_()
@@ -45,9 +40,9 @@ def test_rmsnorm_module_uses_kernel_and_matches(pkg, dev):
     with torch.no_grad():
         norm.weight.mul_(torch.rand(96, device=dev) + 0.5)
     x = torch.randn(4, 10, 96, device=dev)
-    want = rmsnorm_ref(x.double(), norm.weight.double(), norm.eps)
+    want = so.rmsnorm_ref(x.double(), norm.weight.double(), norm.eps)
     assert rel_err(norm(x), want) <= TOL[torch.float32]
     # an unsupported width falls back to the same formula on PyTorch kernels
     norm2 = pkg.RMSNorm(10).to(dev)
     x2 = torch.randn(3, 10, device=dev)
-    assert rel_err(norm2(x2), rmsnorm_ref(x2.double(), norm2.weight.double(), norm2.eps)) <= TOL[torch.float32]
+    assert rel_err(norm2(x2), so.rmsnorm_ref(x2.double(), norm2.weight.double(), norm2.eps)) <= TOL[torch.float32]

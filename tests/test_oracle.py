@@ -233,3 +233,23 @@ def test_causal_conv1d_ref_against_explicit_loops_and_nn_conv1d():
     conv = torch.nn.Conv1d(ED, ED, K, groups=ED, padding=K - 1).double()
     ref = torch.nn.functional.silu(conv(x.transpose(1, 2))[:, :, :L].transpose(1, 2))
     assert (so.causal_conv1d_ref(x, conv.weight, conv.bias) - ref).abs().max().item() < 1e-12
+
+
+def test_rmsnorm_ref_known_answer_loops_and_invariants():
+    # mambapy/mamba.py:427-433
+    x = torch.tensor([[3.0, 4.0]], dtype=torch.float64)
+    want = torch.tensor([[3.0, 4.0]], dtype=torch.float64) / math.sqrt(12.5)
+    assert (so.rmsnorm_ref(x, None, 0.0) - want).abs().max().item() < 1e-15
+    g = torch.Generator().manual_seed(9)
+    x = torch.randn(3, 5, 6, generator=g, dtype=torch.float64) * 2 + 0.5
+    w = torch.randn(6, generator=g, dtype=torch.float64)
+    eps = 1e-3
+    got = so.rmsnorm_ref(x, w, eps)
+    for i in range(3):
+        for j in range(5):
+            ms = sum(x[i, j, k].item() ** 2 for k in range(6)) / 6
+            for k in range(6):
+                assert abs(got[i, j, k].item() - x[i, j, k].item() / math.sqrt(ms + eps) * w[k].item()) < 1e-12
+    y0 = so.rmsnorm_ref(x, None, 0.0)
+    assert (y0.pow(2).mean(-1) - 1.0).abs().max().item() < 1e-12
+    assert (so.rmsnorm_ref(x * 7.5, None, 0.0) - y0).abs().max().item() < 1e-12
