@@ -1,7 +1,8 @@
 """mambapy_amd: MI355X (gfx950) kernels for the selective-scan hot path of alxndrTL/mamba.py.
 
-The directory is named `mamba.py_amd`; import it as `mambapy_amd` (or
-`__graft_entry__.load_package()`).
+The directory is named `mamba.py_amd`; import it under the name `mambapy_amd` with
+importlib.util.spec_from_file_location("mambapy_amd", ".../mamba.py_amd/__init__.py",
+submodule_search_locations=[".../mamba.py_amd"]), as `__graft_entry__.load_package()` does.
 """
 from . import _lib
 from .scan import PScan, pscan, selective_scan, selective_scan_fn, ssm_step, SelectiveScanFn
