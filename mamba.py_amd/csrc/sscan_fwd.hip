@@ -44,6 +44,9 @@ struct FwdParams {
     void* ypre;  // output before the gate (only with z), strides of y
     float* ckpt;
     float* hlast;
+    float* dsum;     // segmented mode, first pass: sums of delta per (row, step group, channel)
+    int nseg;        // > 1: every batch row is cut into nseg segments of seg_tiles tiles, one
+    int seg_tiles;   // workgroup row (blockIdx.y) per (batch row, segment)
     int batch, L, ED, N, nchunks;
     int softplus;
     int in_tmajor;   // x / delta have unit stride along time
@@ -164,9 +167,18 @@ __global__ void __launch_bounds__((NW + kService) * kWave) sscan_fwd_kernel(cons
 
     const int lane = threadIdx.x & (kWave - 1);
     const int w = wave_id();
-    const int b = blockIdx.y;
+    // Row of the launch: a batch row, or one segment of it (segmented mode).  h0 / h_last / dsum
+    // are indexed by the launch row, the caller's tensors by (batch row, first step of the row).
+    const int bs = blockIdx.y;
+    int b = bs, tile0 = 0, ntiles = p.nchunks;
+    if (p.nseg > 1) {
+        b = bs / p.nseg;
+        tile0 = (bs - b * p.nseg) * p.seg_tiles;
+        ntiles = min(p.seg_tiles, p.nchunks - tile0);
+    }
+    const int tbase = tile0 * kTile;               // first step of the row
+    const int Lrow = min(p.L - tbase, ntiles * kTile);  // steps of the row
     const int d0 = blockIdx.x * kWave;
-    const int ntiles = p.nchunks;
     constexpr bool has_z = HAS_Z;
 
     if (w >= NW) {
@@ -197,9 +209,9 @@ __global__ void __launch_bounds__((NW + kService) * kWave) sscan_fwd_kernel(cons
             // wave-uniform tile origins (scalar registers) + per-thread 32-bit element
             // offsets that do not change from tile to tile: one global_load per element and no
             // address arithmetic in the loop
-            const IO* const xg = static_cast<const IO*>(p.x) + (b * p.u_sb + (int64_t)d0 * p.u_sd);
-            const IO* const dg = static_cast<const IO*>(p.delta) + (b * p.d_sb + (int64_t)d0 * p.d_sd);
-            const IO* const zg = static_cast<const IO*>(p.z) + (b * p.z_sb + (int64_t)d0 * p.z_sd);
+            const IO* const xg = static_cast<const IO*>(p.x) + (b * p.u_sb + tbase * p.u_sl + (int64_t)d0 * p.u_sd);
+            const IO* const dg = static_cast<const IO*>(p.delta) + (b * p.d_sb + tbase * p.d_sl + (int64_t)d0 * p.d_sd);
+            const IO* const zg = static_cast<const IO*>(p.z) + (b * p.z_sb + tbase * p.z_sl + (int64_t)d0 * p.z_sd);
             // byte offset of the item's first step (one vector register per tensor, see ld_off);
             // its other three steps are one row stride further each, which goes into the scalar
             // offset of the access
@@ -211,13 +223,13 @@ __global__ void __launch_bounds__((NW + kService) * kWave) sscan_fwd_kernel(cons
             // are masked at staging) as long as the address is inside the tensor: the ragged
             // tile is read through windows that end with the tensor's last element, whatever
             // the strides (out-of-window loads return zero).
-            const bool ragged_end = ntiles * kTile > p.L;
+            const bool ragged_end = ntiles * kTile > Lrow;
             const bool group_full = cmax == kWave - 1;
             // B/C of a tile: kTile * NP elements each, kBcPer per loader thread, step fastest
             constexpr int kBcPer = kBcast ? NP * kTile / (kLoaders * kWave) : 0;
             static_assert(!kBcast || NP * kTile % (kLoaders * kWave) == 0, "whole elements per thread");
-            const IO* const Bg = static_cast<const IO*>(p.Bm) + b * p.bc_sb;
-            const IO* const Cg = static_cast<const IO*>(p.C) + b * p.bc_sb;
+            const IO* const Bg = static_cast<const IO*>(p.Bm) + (b * p.bc_sb + tbase * p.bc_sl);
+            const IO* const Cg = static_cast<const IO*>(p.C) + (b * p.bc_sb + tbase * p.bc_sl);
             int bct[kBcPer > 0 ? kBcPer : 1], bcn[kBcPer > 0 ? kBcPer : 1];
             uint32_t offbc[kBcPer > 0 ? kBcPer : 1];
 #pragma unroll
@@ -239,6 +251,7 @@ __global__ void __launch_bounds__((NW + kService) * kWave) sscan_fwd_kernel(cons
             const float4* const warm =
                 kBcast ? nullptr
                        : reinterpret_cast<const float4*>(p.bcpack) + (int64_t)b * ntiles * kPackVec + min(item, kPackVec - 1);
+            float dsum = 0.0f;  // delta summed over the thread's steps of the row
             struct Raw { IO x[4], d[4], z[4], b[kBcPer > 0 ? kBcPer : 1], c[kBcPer > 0 ? kBcPer : 1]; float4 warm; };
             auto load_tile = [&](int kk, Raw& raw) {
                 // tiles beyond the last one are clamped to it; the loads are unconditional (a
@@ -252,7 +265,7 @@ __global__ void __launch_bounds__((NW + kService) * kWave) sscan_fwd_kernel(cons
                 uint32_t wx = 0xffffffffu, wd = wx, wz = wx, wbc = wx;
                 if (ragged_end && k == ntiles - 1) {
                     // elements from this tile's origin to one past the tensor's last element
-                    const int64_t tb = (int64_t)k * kTile;
+                    const int64_t tb = (int64_t)k * kTile + tbase;
                     auto left = [&](int64_t sb_, int64_t sl_, int64_t sd_, int64_t width) {
                         const int64_t end = (p.batch - 1) * sb_ + (p.L - 1) * sl_ + (width - 1) * sd_ + 1;
                         return window_bytes(end, b * sb_ + tb * sl_ + (int64_t)d0 * sd_, kES);
@@ -296,16 +309,17 @@ __global__ void __launch_bounds__((NW + kService) * kWave) sscan_fwd_kernel(cons
 #pragma unroll
                     for (int j = 0; j < 4; ++j) dv[j] = softplus_f(dv[j] + bias);
                 }
-                if (!group_full || (k + 1) * kTile > p.L) {
+                if (!group_full || (k + 1) * kTile > Lrow) {
                     // ragged edge: delta = 0, u = 0 keeps the state of padded steps/channels
                     const int t0 = k * kTile + 4 * qi;
 #pragma unroll
                     for (int j = 0; j < 4; ++j) {
-                        const bool ok = ci_ok && t0 + j < p.L;
+                        const bool ok = ci_ok && t0 + j < Lrow;
                         xv[j] = ok ? xv[j] : 0.0f;
                         dv[j] = ok ? dv[j] : 0.0f;
                     }
                 }
+                dsum += (dv[0] + dv[1]) + (dv[2] + dv[3]);
                 const int q4 = 4 * qi;
                 *reinterpret_cast<float4*>(&sDl[k & 1][ci][q4]) = make_float4(dv[0], dv[1], dv[2], dv[3]);
                 *reinterpret_cast<float4*>(&sU[k & 1][ci][q4]) =
@@ -345,6 +359,7 @@ __global__ void __launch_bounds__((NW + kService) * kWave) sscan_fwd_kernel(cons
                 load_tile(k + 7, rb);
                 __syncthreads();
             }
+            if (p.dsum && ci_ok) p.dsum[((int64_t)bs * NQ + qi) * p.ED + d0 + ci] = dsum;
         } else {
             // ------------------------------- reducers -------------------------------
             const int co = p.out_tmajor ? item / NQ : item % kWave;
@@ -353,9 +368,10 @@ __global__ void __launch_bounds__((NW + kService) * kWave) sscan_fwd_kernel(cons
             const int q4 = 4 * qo;
             const uint32_t offy = ((uint32_t)q4 * (uint32_t)p.y_sl + (uint32_t)min(co, cmax) * (uint32_t)p.y_sd) * kES;
             const uint32_t sy = (uint32_t)p.y_sl * kES;
-            IO* const yg = static_cast<IO*>(p.y) + (b * p.y_sb + (int64_t)d0 * p.y_sd);
-            IO* const ypg = static_cast<IO*>(p.ypre) + (b * p.y_sb + (int64_t)d0 * p.y_sd);
+            IO* const yg = static_cast<IO*>(p.y) + (b * p.y_sb + tbase * p.y_sl + (int64_t)d0 * p.y_sd);
+            IO* const ypg = static_cast<IO*>(p.ypre) + (b * p.y_sb + tbase * p.y_sl + (int64_t)d0 * p.y_sd);
             auto reduce_store = [&](int k) {
+                if (!p.y) return;  // first pass of the segmented mode: only the end states count
                 IO* yk = yg + (int64_t)k * kTile * p.y_sl;
                 IO* ypk = ypg + (int64_t)k * kTile * p.y_sl;
                 float4 s = *reinterpret_cast<const float4*>(&sDx[k & 3][co][q4]);
@@ -369,18 +385,18 @@ __global__ void __launch_bounds__((NW + kService) * kWave) sscan_fwd_kernel(cons
                     if (p.ypre) {
                         const float pv[4] = {s.x, s.y, s.z, s.w};
                         for (int j = 0; j < 4; ++j)
-                            if (co_ok && t0 + j < p.L) st_off(ypk, offy, from_float<IO>(pv[j]), j * sy);
+                            if (co_ok && t0 + j < Lrow) st_off(ypk, offy, from_float<IO>(pv[j]), j * sy);
                     }
                     const float4 g = *reinterpret_cast<const float4*>(&sG[k & 3][co][q4]);
                     s.x *= g.x; s.y *= g.y; s.z *= g.z; s.w *= g.w;
                 }
                 const float sv[4] = {s.x, s.y, s.z, s.w};
-                if (co_ok && t0 + 3 < p.L) {
+                if (co_ok && t0 + 3 < Lrow) {
 #pragma unroll
                     for (int j = 0; j < 4; ++j) st_off(yk, offy, from_float<IO>(sv[j]), j * sy);
                 } else if (co_ok) {
                     for (int j = 0; j < 4; ++j)
-                        if (t0 + j < p.L) st_off(yk, offy, from_float<IO>(sv[j]), j * sy);
+                        if (t0 + j < Lrow) st_off(yk, offy, from_float<IO>(sv[j]), j * sy);
                 }
             };
             // the reducers run one tile behind the scan waves
@@ -405,7 +421,7 @@ __global__ void __launch_bounds__((NW + kService) * kWave) sscan_fwd_kernel(cons
         const bool ok = dvalid && n < p.N;
         const int64_t dn = (int64_t)min(d, p.ED - 1) * p.N + min(n, p.N - 1);
         const float av = p.A[dn];
-        const float hv = p.h0 ? p.h0[(int64_t)b * p.ED * p.N + dn] : 0.0f;
+        const float hv = p.h0 ? p.h0[(int64_t)bs * p.ED * p.N + dn] : 0.0f;
         A2[i] = ok ? av * kLog2e : 0.0f;
         h[i] = ok ? hv : 0.0f;
     }
@@ -433,7 +449,7 @@ __global__ void __launch_bounds__((NW + kService) * kWave) sscan_fwd_kernel(cons
         }
     };
     auto store_ckpt = [&](int k) {
-        if (p.ckpt && dvalid && k + 1 < ntiles) {
+        if (p.ckpt && dvalid && k + 1 < ntiles) {  // never in segmented mode (b, ntiles: whole rows)
 #pragma unroll
             for (int i = 0; i < NS; ++i) {
                 const int n = w * NS + i;
@@ -479,7 +495,7 @@ __global__ void __launch_bounds__((NW + kService) * kWave) sscan_fwd_kernel(cons
         constexpr int kSub = 2 * kSS * NS;           // floats per sub-tile: B then C
         constexpr int kRing = FwdPack<NS>::kRing;    // sub-tiles resident in scalar registers
         static_assert(NSUB % kRing == 0, "a sub-tile always lands in the same ring slot");
-        const float* bc = p.bcpack + ((int64_t)b * ntiles * NW + w) * (NSUB * kSub);
+        const float* bc = p.bcpack + ((int64_t)b * ntiles * NW + w) * (NSUB * kSub);  // whole rows only
         const int64_t bc_tile = (int64_t)NW * NSUB * kSub;
         float bcb[kRing][kSub];  // wave-uniform: live in SGPRs; sub-tile j of a tile uses slot j % kRing
         auto tile_compute = [&](int k, const TileRegs& cur_t, TileRegs& next) {
@@ -538,14 +554,76 @@ __global__ void __launch_bounds__((NW + kService) * kWave) sscan_fwd_kernel(cons
 #pragma unroll
         for (int i = 0; i < NS; ++i) {
             const int n = w * NS + i;
-            if (n < p.N) p.hlast[((int64_t)b * p.ED + d) * p.N + n] = h[i];
+            if (n < p.N) p.hlast[((int64_t)bs * p.ED + d) * p.N + n] = h[i];
         }
     }
 }
 
+// Segmented mode, between the passes: the state at the start of every segment.  The first pass
+// ran every segment from a zero state: hend = its end state, dsum = its sums of delta; with
+// P = exp(A * sum of delta) (the product of the segment's decay factors) the true end state of a
+// segment that starts from h is P*h + hend.  One thread per (batch row, channel, state) walks the
+// segments in order.
+__global__ void __launch_bounds__(256) seg_carry_kernel(const float* __restrict__ A, const float* __restrict__ h0,
+                                                        const float* __restrict__ hend, const float* __restrict__ dsum,
+                                                        float* __restrict__ segh0, float* __restrict__ hlast,
+                                                        int batch, int nseg, int ED, int N) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t per_b = (int64_t)ED * N;
+    if (i >= batch * per_b) return;
+    const int b = (int)(i / per_b);
+    const int64_t dn = i - b * per_b;
+    const int d = (int)(dn / N);
+    const float a2 = A[dn] * kLog2e;
+    float h = h0 ? h0[i] : 0.0f;
+    for (int sg = 0; sg < nseg; ++sg) {
+        const int64_t row = (int64_t)b * nseg + sg;
+        segh0[row * per_b + dn] = h;
+        const float* ds = dsum + row * (kTile / 4) * ED + d;
+        const float sd = (ds[0] + ds[ED]) + (ds[2 * (int64_t)ED] + ds[3 * (int64_t)ED]);
+        h = __builtin_fmaf(fast_exp2(a2 * sd), h, hend[row * per_b + dn]);
+    }
+    if (hlast) hlast[i] = h;
+}
+
+// Segments per batch row.  The scan is serial in time, so a launch has only batch * dim/64
+// workgroups; when those cover a fraction of the chip's 256 CUs and no checkpoints are wanted
+// (inference prefill), the sequence is cut into segments that run side by side: twice the
+// arithmetic, nseg times the parallelism.
+struct SegPlan {
+    int nseg, seg_tiles;
+    size_t off_hend, off_h0, off_dsum, floats;
+};
+static SegPlan seg_plan(const mpa_sscan_shape* s, int ns) {
+    SegPlan sp{1, 0, 0, 0, 0, 0};
+    if (ns > 8) return sp;
+    const int64_t ntiles = (s->seqlen + kTile - 1) / kTile;
+    const int64_t groups = s->batch * ((s->dim + kWave - 1) / kWave);
+    int64_t want = 1;
+    const char* v = getenv("MPA_FWD_NSEG");
+    if (v) {
+        want = atoi(v);
+    } else if (groups * 3 <= 256 && ntiles >= 64) {
+        want = 256 / groups;
+        if (want > ntiles / 16) want = ntiles / 16;  // segments of 256 steps or more
+        if (want > 64) want = 64;
+    }
+    if (want > ntiles) want = ntiles;
+    if (want < 2 || s->batch * want > 65535) return sp;
+    sp.seg_tiles = (int)((ntiles + want - 1) / want);
+    sp.nseg = (int)((ntiles + sp.seg_tiles - 1) / sp.seg_tiles);
+    if (sp.nseg < 2) return SegPlan{1, 0, 0, 0, 0, 0};
+    const size_t rows = (size_t)s->batch * sp.nseg, per = (size_t)s->dim * s->dstate;
+    sp.off_hend = 0;
+    sp.off_h0 = rows * per;
+    sp.off_dsum = 2 * rows * per;
+    sp.floats = sp.off_dsum + rows * (kTile / 4) * (size_t)s->dim;
+    return sp;
+}
+
 template <typename IO, int NS, int NW, bool HAS_Z>
 static int launch_fwd(const FwdParams& p, hipStream_t stream) {
-    dim3 grid((p.ED + kWave - 1) / kWave, p.batch);
+    dim3 grid((p.ED + kWave - 1) / kWave, p.batch * (p.nseg > 1 ? p.nseg : 1));
     dim3 block((NW + kService) * kWave);
     constexpr size_t lds = sizeof(float) * FwdLds<NS, NW>::floats;
     static const int attr_rc = allow_dynamic_lds(sscan_fwd_kernel<IO, NS, NW, HAS_Z>, lds);
@@ -653,7 +731,7 @@ extern "C" size_t mpa_sscan_fwd_workspace_bytes(const mpa_sscan_shape* s) {
     if (validate_shape(s) != MPA_OK) return 0;
     // the packed B/C exist only on the scalar-load path (more than 8 states per lane)
     const int ns = pick_states_per_lane(s->batch, s->dim, s->dstate, 32, "MPA_FWD_NS");
-    if (ns <= 8) return 256;
+    if (ns <= 8) return (seg_plan(s, ns).floats * sizeof(float) + 255) / 256 * 256 + 256;
     return (bcpack_floats(s) * sizeof(float) + 255) / 256 * 256;
 }
 
@@ -698,6 +776,27 @@ extern "C" int mpa_sscan_fwd(const mpa_sscan_shape* s, const void* x, const void
     p.y_sb = s->y_sb; p.y_sl = s->y_sl; p.y_sd = s->y_sd;
     p.in_tmajor = (s->u_sd != 1 && s->u_sl == 1) ? 1 : 0;
     p.out_tmajor = (s->y_sd != 1 && s->y_sl == 1) ? 1 : 0;
-    if (s->io_dtype == MPA_F32) return dispatch_fwd<float>(p, ns, nw, st);
-    return dispatch_fwd<bf16_t>(p, ns, nw, st);
+    auto run = [&](const FwdParams& q) {
+        return s->io_dtype == MPA_F32 ? dispatch_fwd<float>(q, ns, nw, st) : dispatch_fwd<bf16_t>(q, ns, nw, st);
+    };
+    const SegPlan sp = h_ckpt ? SegPlan{1, 0, 0, 0, 0, 0} : seg_plan(s, ns);
+    if (sp.nseg <= 1) return run(p);
+
+    // segmented mode: end states of every segment from zero, carry, then the real pass
+    float* wsf = static_cast<float*>(workspace);
+    FwdParams p1 = p;
+    p1.nseg = sp.nseg; p1.seg_tiles = sp.seg_tiles;
+    p1.z = nullptr; p1.y = nullptr; p1.ypre = nullptr; p1.h0 = nullptr;
+    p1.hlast = wsf + sp.off_hend; p1.dsum = wsf + sp.off_dsum;
+    rc = run(p1);
+    if (rc != MPA_OK) return rc;
+    const int64_t total = (int64_t)p.batch * p.ED * p.N;
+    hipLaunchKernelGGL(seg_carry_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, A, h0,
+                       wsf + sp.off_hend, wsf + sp.off_dsum, wsf + sp.off_h0, h_last, p.batch, sp.nseg, p.ED, p.N);
+    rc = check_launch();
+    if (rc != MPA_OK) return rc;
+    FwdParams p2 = p;
+    p2.nseg = sp.nseg; p2.seg_tiles = sp.seg_tiles;
+    p2.h0 = wsf + sp.off_h0; p2.hlast = nullptr;
+    return run(p2);
 }

@@ -71,7 +71,8 @@ class SelectiveScanFn(torch.autograd.Function):
     """Fused discretise -> scan -> readout with a hand-written backward kernel."""
 
     @staticmethod
-    def forward(ctx, x, delta, A, B, C, D, z, delta_bias, delta_softplus, h0, return_last_state):
+    def forward(ctx, x, delta, A, B, C, D, z, delta_bias, delta_softplus, h0, return_last_state,
+                need_grad=True):
         _require_gpu(x, delta, A, B, C, D, z, delta_bias, h0)
         lib = _lib.load()
         dt = x.dtype
@@ -96,8 +97,8 @@ class SelectiveScanFn(torch.autograd.Function):
         z_ = None if z is None else z.detach().to(dt)
         A_, D_, bias_, h0_ = _f32c(A), _f32c(D), _f32c(delta_bias), _f32c(h0)
         y = torch.empty((Bsz, L, ED), dtype=dt, device=x.device)
-        need_grad = any(t is not None and t.requires_grad
-                        for t in (x, delta, A, B, C, D, z, delta_bias))
+        # need_grad: checkpoints (and the pre-gate output) are written only for a backward pass;
+        # without them the library is also free to cut a long sequence into parallel segments
         flags = _lib.MPA_SSCAN_DELTA_SOFTPLUS if delta_softplus else 0
         shape = _sscan_shape(x_, delta_, B_, y, y, B_, N, flags, z_)
         ckpt = y_pre = None
@@ -159,7 +160,7 @@ class SelectiveScanFn(torch.autograd.Function):
         tx, td, tA, tB, tC, tD, tz, tb = ctx.in_dtypes
         return (dx.to(tx), ddelta.to(td), dA.to(tA), dB.to(tB), dC.to(tC), dD.to(tD),
                 None if dz is None else dz.to(tz), None if dbias is None else dbias.to(tb),
-                None, None, None)
+                None, None, None, None)
 
 
 def selective_scan_fn(x, delta, A, B, C, D, z=None, delta_bias=None, delta_softplus=False,
@@ -171,8 +172,12 @@ def selective_scan_fn(x, delta, A, B, C, D, z=None, delta_bias=None, delta_softp
     x, delta, z : (B, L, ED);  A : (ED, N);  B, C : (B, L, N);  D, delta_bias : (ED);
     h0 : optional (B, ED, N) initial state.  Returns y (B, L, ED) [, last state (B, ED, N)].
     """
+    # grad mode is off inside Function.forward and parameters keep requires_grad under no_grad,
+    # so whether a backward can follow is decided here
+    need_grad = torch.is_grad_enabled() and any(
+        t is not None and t.requires_grad for t in (x, delta, A, B, C, D, z, delta_bias))
     return SelectiveScanFn.apply(x, delta, A, B, C, D, z, delta_bias, bool(delta_softplus), h0,
-                                 bool(return_last_state))
+                                 bool(return_last_state), need_grad)
 
 
 def selective_scan(x, delta, A, B, C, D):

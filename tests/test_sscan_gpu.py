@@ -221,6 +221,62 @@ def test_time_outermost_memory_and_ragged_tail(pkg, dev):
     assert rel_err(y_exp, ref_exp) <= TOL[torch.float32]
 
 
+def _inference_case(pkg, dev, Bs, L, ED, N, dtype, seed, gated):
+    """forward without gradients (no checkpoints): y and the last state"""
+    inp = so.make_inputs(Bs, L, ED, N, seed=seed)
+    g = torch.Generator().manual_seed(seed + 1)
+    h0 = torch.randn(Bs, ED, N, generator=g)
+    z = torch.randn(Bs, L, ED, generator=g) if gated else None
+    raw = torch.randn(Bs, L, ED, generator=g) * 0.5 - 4.0
+    bias = torch.randn(ED, generator=g) * 0.3
+    q = lambda t: t.to(dtype)
+    d64 = lambda t: q(t).double()
+    delta = so.softplus_ref(d64(raw) + bias.double()) if gated else d64(inp["delta"])
+    yr, hl = so.selective_scan_ref(d64(inp["x"]), delta, inp["A"].double(), d64(inp["B"]), d64(inp["C"]),
+                                   inp["D"].double(), h0=h0.double(), return_last_state=True)
+    if gated:
+        yr = yr * (d64(z) * torch.sigmoid(d64(z)))
+    with torch.no_grad():
+        dv = lambda t: q(t).to(dev)
+        if gated:
+            y, hg = pkg.selective_scan_fn(dv(inp["x"]), dv(raw), inp["A"].to(dev), dv(inp["B"]), dv(inp["C"]),
+                                          inp["D"].to(dev), z=dv(z), delta_bias=bias.to(dev), delta_softplus=True,
+                                          h0=h0.to(dev), return_last_state=True)
+        else:
+            y, hg = pkg.selective_scan_fn(dv(inp["x"]), dv(inp["delta"]), inp["A"].to(dev), dv(inp["B"]),
+                                          dv(inp["C"]), inp["D"].to(dev), h0=h0.to(dev), return_last_state=True)
+    return y, hg, yr, hl
+
+
+@pytest.mark.parametrize("Bs,L,ED,N,nseg,gated", [
+    (1, 160, 64, 16, 3, False), (2, 100, 70, 16, 4, True), (1, 37, 130, 8, 2, False),
+    (1, 1000, 96, 16, 7, True), (3, 64, 64, 4, 4, False), (1, 16, 64, 16, 5, False), (1, 33, 5, 16, 64, True),
+])
+def test_segmented_forward_matches_oracle_and_single_pass(pkg, dev, Bs, L, ED, N, nseg, gated, monkeypatch):
+    # inference form (no checkpoints) with the sequence cut into segments that run side by side
+    monkeypatch.setenv("MPA_FWD_NSEG", str(nseg))
+    y, hg, yr, hl = _inference_case(pkg, dev, Bs, L, ED, N, torch.float32, 300 + L, gated)
+    assert rel_err(y, yr) <= TOL[torch.float32]
+    assert rel_err(hg, hl) <= TOL[torch.float32]
+    monkeypatch.setenv("MPA_FWD_NSEG", "1")
+    y1, h1, _, _ = _inference_case(pkg, dev, Bs, L, ED, N, torch.float32, 300 + L, gated)
+    assert rel_err(y, y1.double()) <= 1e-5 and rel_err(hg, h1.double()) <= 1e-5
+
+
+def test_segmented_forward_is_picked_for_a_single_long_sequence(pkg, dev, monkeypatch):
+    # batch 1, 24 channel groups, 4096 steps in bf16: the library cuts the sequence by itself
+    monkeypatch.delenv("MPA_FWD_NSEG", raising=False)
+    y, hg, yr, hl = _inference_case(pkg, dev, 1, 4096, 1536, 16, torch.bfloat16, 77, True)
+    assert rel_err(y, yr) <= TOL[torch.bfloat16]
+    assert rel_err(hg, hl) <= TOL[torch.float32]
+    big = torch.empty(1, 4096, 1536, dtype=torch.bfloat16, device=dev)
+    bc = torch.empty(1, 4096, 16, dtype=torch.bfloat16, device=dev)
+    shape = pkg.scan._sscan_shape(big, big, bc, big, big, bc, 16, 0)
+    import ctypes
+    need = pkg._lib.load().mpa_sscan_fwd_workspace_bytes(ctypes.byref(shape))
+    assert need > 2 * 10 * 1536 * 16 * 4  # room for the states of 10 segments
+
+
 def test_bitwise_reproducible(pkg, dev):
     inp = so.make_inputs(2, 130, 200, 16, seed=61)
     a = run_gpu_fwd_bwd(pkg, inp, dev)
