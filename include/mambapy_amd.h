@@ -169,12 +169,19 @@ size_t mpa_conv1d_bwd_workspace_bytes(const mpa_conv_shape* s);
  * d <= 2048 / 4096), weight (d) float32 or NULL (the muP variant has none), and its gradient:
  * dx (io_dtype) and dweight (d) float32, overwritten.  rstd (rows) float32 is an optional output.
  * Pointers to x, y, dy, dx must be 16-byte aligned.
+ *
+ * The residual add of the layer stack (mambapy/mamba.py:106-112: mixer(norm(x)) + x, read by the
+ * next layer's norm) can be folded in: with `residual` (rows x d, io_dtype) the forward writes
+ * sum_out = x + residual (rounded to io_dtype, as the separate add would be) and normalises that
+ * row; the backward then takes the sum as its `x` and `dsum`, the gradient that reaches the sum
+ * from its other users, and returns dx = (gradient through the norm) + dsum, which is the gradient
+ * of both x and residual.  residual, sum_out and dsum may be NULL (plain RMSNorm).
  */
-int mpa_rmsnorm_fwd(const void* x, const float* weight, void* y, float* rstd, int64_t rows, int64_t d,
-                    float eps, int32_t io_dtype, void* stream);
-int mpa_rmsnorm_bwd(const void* x, const float* weight, const void* dy, void* dx, float* dweight,
-                    int64_t rows, int64_t d, float eps, int32_t io_dtype, void* workspace,
-                    size_t workspace_bytes, void* stream);
+int mpa_rmsnorm_fwd(const void* x, const void* residual, const float* weight, void* y, void* sum_out,
+                    float* rstd, int64_t rows, int64_t d, float eps, int32_t io_dtype, void* stream);
+int mpa_rmsnorm_bwd(const void* x, const float* weight, const void* dy, const void* dsum, void* dx,
+                    float* dweight, int64_t rows, int64_t d, float eps, int32_t io_dtype,
+                    void* workspace, size_t workspace_bytes, void* stream);
 size_t mpa_rmsnorm_bwd_workspace_bytes(int64_t rows, int64_t d);
 
 /* ---- generic first-order scan -----------------------------------------------------------

@@ -7,14 +7,15 @@ submodule_search_locations=[".../mamba.py_amd"]), as `__graft_entry__.load_packa
 from . import _lib
 from .scan import PScan, pscan, selective_scan, selective_scan_fn, ssm_step, SelectiveScanFn
 from .conv import CausalConv1dFn, causal_conv1d_fn
-from .norm import RMSNormFn, rmsnorm_fn
+from .norm import AddRMSNormFn, RMSNormFn, add_rmsnorm_fn, rmsnorm_fn
 from .modules import Mamba, MambaBlock, MambaConfig, ResidualBlock, RMSNorm
 from .language_model import LM
 from .decode import GraphedDecoder
 from .patch import patch_mambapy
 
 __all__ = ["PScan", "pscan", "selective_scan", "selective_scan_fn", "ssm_step",
-           "SelectiveScanFn", "CausalConv1dFn", "causal_conv1d_fn", "RMSNormFn", "rmsnorm_fn", "Mamba", "MambaBlock", "MambaConfig", "ResidualBlock", "RMSNorm",
+           "SelectiveScanFn", "CausalConv1dFn", "causal_conv1d_fn", "RMSNormFn", "rmsnorm_fn",
+           "AddRMSNormFn", "add_rmsnorm_fn", "Mamba", "MambaBlock", "MambaConfig", "ResidualBlock", "RMSNorm",
            "LM", "GraphedDecoder", "patch_mambapy", "library_path", "library_version"]
 
 

@@ -83,8 +83,8 @@ def load():
     lib.mpa_conv1d_bwd_workspace_bytes.argtypes = [cp]
     lib.mpa_conv1d_bwd_workspace_bytes.restype = sz
     f32 = ctypes.c_float
-    lib.mpa_rmsnorm_fwd.argtypes = [vp] * 4 + [i64, i64, f32, i32, vp]
-    lib.mpa_rmsnorm_bwd.argtypes = [vp] * 5 + [i64, i64, f32, i32, vp, sz, vp]
+    lib.mpa_rmsnorm_fwd.argtypes = [vp] * 6 + [i64, i64, f32, i32, vp]
+    lib.mpa_rmsnorm_bwd.argtypes = [vp] * 6 + [i64, i64, f32, i32, vp, sz, vp]
     lib.mpa_rmsnorm_bwd_workspace_bytes.argtypes = [i64, i64]
     lib.mpa_rmsnorm_bwd_workspace_bytes.restype = sz
     for name in EXPORTS:

@@ -7,6 +7,11 @@
 // exchanges, and writes the scaled row; the second read of the row comes from cache.  The
 // kernels are bound by HBM: forward x in, y out; backward x, dy in, dx out, plus per-block
 // partial sums of dweight that a second kernel adds up in a fixed order.
+//
+// The residual add that precedes every norm of the layer stack (mambapy/mamba.py:106-112:
+// output = mixer(norm(x)) + x, then the next layer's norm reads it) can ride along: the forward
+// takes a second input, writes the sum (rounded to the I/O type, as the separate add would) and
+// normalises it; the backward adds the gradient that reaches the sum from its other users.
 #include "common.h"
 
 namespace mpa {
@@ -52,9 +57,11 @@ __device__ __forceinline__ float wave_sum(float v) {
 }
 
 // rows x d, contiguous rows; d a multiple of the vector width.  rstd (rows) is optional.
+// With `res`: the row that is normalised is round(x + res), also written to `sum_out`.
 template <typename IO>
-__global__ void __launch_bounds__(256) rmsnorm_fwd_kernel(const IO* __restrict__ x, const float* __restrict__ w,
-                                                          IO* __restrict__ y, float* __restrict__ rstd_out,
+__global__ void __launch_bounds__(256) rmsnorm_fwd_kernel(const IO* __restrict__ x, const IO* __restrict__ res,
+                                                          const float* __restrict__ w, IO* __restrict__ y,
+                                                          IO* __restrict__ sum_out, float* __restrict__ rstd_out,
                                                           int64_t rows, int d, float eps) {
     typedef RowVec<IO> V;
     const int lane = threadIdx.x & (kWave - 1);
@@ -63,10 +70,22 @@ __global__ void __launch_bounds__(256) rmsnorm_fwd_kernel(const IO* __restrict__
     const int nvec = d / V::kN;
     const typename V::T* xr = reinterpret_cast<const typename V::T*>(x + row * d);
     typename V::T* yr = reinterpret_cast<typename V::T*>(y + row * d);
+    const typename V::T* rr = reinterpret_cast<const typename V::T*>(res + row * d);
+    typename V::T* sr = reinterpret_cast<typename V::T*>(sum_out + row * d);
+    auto load_row = [&](int i, float (&f)[V::kN]) {
+        V::unpack(xr[i], f);
+        if (res) {
+            float g[V::kN];
+            V::unpack(rr[i], g);
+#pragma unroll
+            for (int j = 0; j < V::kN; ++j) f[j] = to_float(from_float<IO>(f[j] + g[j]));
+        }
+    };
     float ss = 0.0f;
     for (int i = lane; i < nvec; i += kWave) {
         float f[V::kN];
-        V::unpack(xr[i], f);
+        load_row(i, f);
+        if (res) sr[i] = V::pack(f);
 #pragma unroll
         for (int j = 0; j < V::kN; ++j) ss = __builtin_fmaf(f[j], f[j], ss);
     }
@@ -74,7 +93,7 @@ __global__ void __launch_bounds__(256) rmsnorm_fwd_kernel(const IO* __restrict__
     if (rstd_out && lane == 0) rstd_out[row] = rstd;
     for (int i = lane; i < nvec; i += kWave) {
         float f[V::kN], o[V::kN];
-        V::unpack(xr[i], f);
+        load_row(i, f);
 #pragma unroll
         for (int j = 0; j < V::kN; ++j) o[j] = f[j] * rstd * (w ? w[i * V::kN + j] : 1.0f);
         yr[i] = V::pack(o);
@@ -82,12 +101,14 @@ __global__ void __launch_bounds__(256) rmsnorm_fwd_kernel(const IO* __restrict__
 }
 
 // dx = rstd * (w*dy) - x * rstd^3 * mean(w*dy*x);  dweight[c] = sum_rows dy*x*rstd.
-// A wave walks kNormRowsPerWave rows; the dweight sums of a block (4 waves) go to
-// part[block][d] through LDS-free per-wave rows: part[(block*4 + wave)][d].
+// A wave walks kNormRowsPerWave rows and writes its dweight sums as one row of `part`.
+// `dres` (optional) is added to dx: the gradient that reaches the normalised row from its
+// other users (the residual stream).
 template <typename IO, int MAXV>
 __global__ void __launch_bounds__(256) rmsnorm_bwd_kernel(const IO* __restrict__ x, const float* __restrict__ w,
-                                                          const IO* __restrict__ dy, IO* __restrict__ dx,
-                                                          float* __restrict__ part, int64_t rows, int d, float eps) {
+                                                          const IO* __restrict__ dy, const IO* __restrict__ dres,
+                                                          IO* __restrict__ dx, float* __restrict__ part,
+                                                          int64_t rows, int d, float eps) {
     typedef RowVec<IO> V;
     const int lane = threadIdx.x & (kWave - 1);
     const int64_t wave = (int64_t)blockIdx.x * (blockDim.x / kWave) + (threadIdx.x / kWave);
@@ -103,6 +124,7 @@ __global__ void __launch_bounds__(256) rmsnorm_bwd_kernel(const IO* __restrict__
         const typename V::T* xr = reinterpret_cast<const typename V::T*>(x + row * d);
         const typename V::T* gr = reinterpret_cast<const typename V::T*>(dy + row * d);
         typename V::T* dr = reinterpret_cast<typename V::T*>(dx + row * d);
+        const typename V::T* qr = reinterpret_cast<const typename V::T*>(dres + row * d);
         float ss = 0.0f, sg = 0.0f;
 #pragma unroll
         for (int v = 0; v < MAXV; ++v) {
@@ -131,6 +153,12 @@ __global__ void __launch_bounds__(256) rmsnorm_bwd_kernel(const IO* __restrict__
                 for (int j = 0; j < V::kN; ++j) {
                     o[j] = __builtin_fmaf(g[j] * (w ? w[i * V::kN + j] : 1.0f), rstd, -f[j] * c);
                     dwacc[v][j] = __builtin_fmaf(g[j] * rstd, f[j], dwacc[v][j]);
+                }
+                if (dres) {
+                    float q[V::kN];
+                    V::unpack(qr[i], q);
+#pragma unroll
+                    for (int j = 0; j < V::kN; ++j) o[j] += q[j];
                 }
                 dr[i] = V::pack(o);
             }
@@ -179,20 +207,24 @@ static int64_t norm_waves(int64_t rows) { return (rows + kNormRowsPerWave - 1) /
 
 using namespace mpa;
 
-extern "C" int mpa_rmsnorm_fwd(const void* x, const float* weight, void* y, float* rstd, int64_t rows,
-                               int64_t d, float eps, int32_t io_dtype, void* stream) {
+extern "C" int mpa_rmsnorm_fwd(const void* x, const void* residual, const float* weight, void* y, void* sum_out,
+                               float* rstd, int64_t rows, int64_t d, float eps, int32_t io_dtype, void* stream) {
     int rc = norm_validate(rows, d, io_dtype);
     if (rc != MPA_OK) return rc;
-    if (!x || !y) return MPA_ERR_NULL_POINTER;
-    if (!aligned_to(x, 16) || !aligned_to(y, 16) || (weight && !aligned_to(weight, 4))) return MPA_ERR_MISALIGNED;
+    if (!x || !y || (residual && !sum_out)) return MPA_ERR_NULL_POINTER;
+    if (!aligned_to(x, 16) || !aligned_to(y, 16) || (weight && !aligned_to(weight, 4)) ||
+        (residual && (!aligned_to(residual, 16) || !aligned_to(sum_out, 16))))
+        return MPA_ERR_MISALIGNED;
     hipStream_t st = static_cast<hipStream_t>(stream);
     dim3 grid((unsigned)((rows + 3) / 4)), block(256);
     if (io_dtype == MPA_F32)
-        hipLaunchKernelGGL(rmsnorm_fwd_kernel<float>, grid, block, 0, st, static_cast<const float*>(x), weight,
-                           static_cast<float*>(y), rstd, rows, (int)d, eps);
+        hipLaunchKernelGGL(rmsnorm_fwd_kernel<float>, grid, block, 0, st, static_cast<const float*>(x),
+                           static_cast<const float*>(residual), weight, static_cast<float*>(y),
+                           static_cast<float*>(sum_out), rstd, rows, (int)d, eps);
     else
-        hipLaunchKernelGGL(rmsnorm_fwd_kernel<bf16_t>, grid, block, 0, st, static_cast<const bf16_t*>(x), weight,
-                           static_cast<bf16_t*>(y), rstd, rows, (int)d, eps);
+        hipLaunchKernelGGL(rmsnorm_fwd_kernel<bf16_t>, grid, block, 0, st, static_cast<const bf16_t*>(x),
+                           static_cast<const bf16_t*>(residual), weight, static_cast<bf16_t*>(y),
+                           static_cast<bf16_t*>(sum_out), rstd, rows, (int)d, eps);
     return check_launch();
 }
 
@@ -202,14 +234,15 @@ extern "C" size_t mpa_rmsnorm_bwd_workspace_bytes(int64_t rows, int64_t d) {
     return ((size_t)waves * d * sizeof(float) + 255) / 256 * 256;
 }
 
-extern "C" int mpa_rmsnorm_bwd(const void* x, const float* weight, const void* dy, void* dx, float* dweight,
-                               int64_t rows, int64_t d, float eps, int32_t io_dtype, void* workspace,
-                               size_t workspace_bytes, void* stream) {
+extern "C" int mpa_rmsnorm_bwd(const void* x, const float* weight, const void* dy, const void* dsum, void* dx,
+                               float* dweight, int64_t rows, int64_t d, float eps, int32_t io_dtype,
+                               void* workspace, size_t workspace_bytes, void* stream) {
     int rc = norm_validate(rows, d, io_dtype);
     if (rc != MPA_OK) return rc;
     if (!x || !dy || !dx) return MPA_ERR_NULL_POINTER;
     if (weight && (!dweight || !workspace)) return MPA_ERR_NULL_POINTER;
     if (!aligned_to(x, 16) || !aligned_to(dy, 16) || !aligned_to(dx, 16) || (weight && !aligned_to(weight, 4)) ||
+        (dsum && !aligned_to(dsum, 16)) ||
         (workspace && !aligned_to(workspace, 256)))
         return MPA_ERR_MISALIGNED;
     if (weight && workspace_bytes < mpa_rmsnorm_bwd_workspace_bytes(rows, d)) return MPA_ERR_WORKSPACE;
@@ -221,7 +254,8 @@ extern "C" int mpa_rmsnorm_bwd(const void* x, const float* weight, const void* d
     const int nv = (int)((d / vec + kWave - 1) / kWave);  // vectors per lane: 1..8
 #define MPA_NORM_CASE(IO_, MV_)                                                                               \
     hipLaunchKernelGGL((rmsnorm_bwd_kernel<IO_, MV_>), grid, block, 0, st, static_cast<const IO_*>(x), weight, \
-                       static_cast<const IO_*>(dy), static_cast<IO_*>(dx), part, rows, (int)d, eps)
+                       static_cast<const IO_*>(dy), static_cast<const IO_*>(dsum), static_cast<IO_*>(dx), part, \
+                       rows, (int)d, eps)
     if (io_dtype == MPA_F32) {
         if (nv <= 1) MPA_NORM_CASE(float, 1);
         else if (nv <= 2) MPA_NORM_CASE(float, 2);

@@ -17,7 +17,7 @@ import torch.nn as nn
 import torch.nn.functional as F
 
 from .conv import causal_conv1d_fn
-from .norm import rmsnorm_fn, rmsnorm_supported
+from .norm import add_rmsnorm_fn, rmsnorm_fn, rmsnorm_supported
 from .scan import selective_scan, selective_scan_fn, ssm_step
 
 
@@ -78,6 +78,15 @@ class RMSNorm(nn.Module):
             return rmsnorm_fn(x, None if self.use_mup else self.weight, self.eps)
         y = x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + self.eps)
         return y if self.use_mup else y * self.weight
+
+    def add_norm(self, x, residual):
+        """(norm(x + residual), x + residual); the add rides in the norm kernel when it can."""
+        if residual is None:
+            return self(x), x
+        if x.is_cuda and rmsnorm_supported(x) and residual.dtype == x.dtype:
+            return add_rmsnorm_fn(x, residual, None if self.use_mup else self.weight, self.eps)
+        total = x + residual
+        return self(total), total
 
 
 class MambaBlock(nn.Module):
@@ -266,27 +275,36 @@ class Mamba(nn.Module):
         self.layers = nn.ModuleList([ResidualBlock(config) for _ in range(config.n_layers)])
 
     def forward(self, x, return_caches: bool = False):
-        if not return_caches:
-            for layer in self.layers:
-                x = layer(x)
-            return x
+        # Same arithmetic as x = layer(x) for every layer, in another order of kernels: the add
+        # that ends layer i is done by the norm kernel that starts layer i+1 (pre-norm
+        # residual stream: `hidden` is the last mixer output, `residual` the running sum).
+        hidden, residual = x, None
         caches = []
         for layer in self.layers:
-            x, c = layer(x, return_cache=True)
-            caches.append(c)
-        return x, caches
+            normed, residual = layer.norm.add_norm(hidden, residual)
+            if return_caches:
+                hidden, c = layer.mixer(normed, return_cache=True)
+                caches.append(c)
+            else:
+                hidden = layer.mixer(normed)
+        x = hidden + residual if self.layers else x
+        return (x, caches) if return_caches else x
 
     def step(self, x, caches):
+        hidden, residual = x, None
         for i, layer in enumerate(self.layers):
-            x, caches[i] = layer.step(x, caches[i])
-        return x, caches
+            normed, residual = layer.norm.add_norm(hidden, residual)
+            hidden, caches[i] = layer.mixer.step(normed, caches[i])
+        return (hidden + residual if self.layers else x), caches
 
     def step_(self, x, caches):
         """In-place variant of step(): every (h, window) pair of `caches` is updated in place
         (h must be a float32 tensor, not None)."""
+        hidden, residual = x, None
         for layer, (h, window) in zip(self.layers, caches):
-            x = layer.step_(x, h, window)
-        return x
+            normed, residual = layer.norm.add_norm(hidden, residual)
+            hidden = layer.mixer.step_(normed, h, window)
+        return hidden + residual if self.layers else x
 
     def empty_caches(self, batch: int, device=None, dtype=None):
         """Fresh decode caches: h = None (zero state), zero conv window (mamba.py:344-346)."""

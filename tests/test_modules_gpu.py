@@ -46,6 +46,31 @@ def test_block_forward_backward_matches_float64_layer(pkg, dev, fused):
         assert rel_err(v.grad, pr[k].grad) <= 5e-4, k
 
 
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-5), (torch.bfloat16, 2e-2)])
+def test_stack_with_folded_residual_adds_equals_layer_by_layer(pkg, dev, dtype, tol):
+    # Mamba.forward folds every residual add into the next layer's norm kernel; the reference's
+    # order is x = layer(x) for each layer (mambapy/mamba.py:87-95, 106-112)
+    torch.manual_seed(5)
+    cfg = pkg.MambaConfig(d_model=64, n_layers=4)
+    model = pkg.Mamba(cfg).to(dev).to(dtype)
+    x = torch.randn(2, 40, 64, device=dev, dtype=dtype)
+    g = torch.randn(2, 40, 64, device=dev, dtype=dtype)
+    xa = x.clone().requires_grad_()
+    ya = model(xa)
+    ya.backward(g)
+    grads_a = {k: v.grad.clone() for k, v in model.named_parameters()}
+    model.zero_grad()
+    xb = x.clone().requires_grad_()
+    yb = xb
+    for layer in model.layers:
+        yb = layer(yb)
+    yb.backward(g)
+    assert rel_err(ya, yb.double()) <= tol
+    assert rel_err(xa.grad, xb.grad.double()) <= tol
+    for k, v in model.named_parameters():
+        assert rel_err(grads_a[k], v.grad.double()) <= 5 * tol, k
+
+
 def test_steps_equal_forward_and_prefill_handoff(pkg, dev):
     # mambapy/mamba.py:330-349: zero conv window + h=None reproduce the parallel forward
     torch.manual_seed(2)

@@ -46,3 +46,42 @@ def test_rmsnorm_module_uses_kernel_and_matches(pkg, dev):
     norm2 = pkg.RMSNorm(10).to(dev)
     x2 = torch.randn(3, 10, device=dev)
     assert rel_err(norm2(x2), so.rmsnorm_ref(x2.double(), norm2.weight.double(), norm2.eps)) <= TOL[torch.float32]
+
+
+@pytest.mark.parametrize("shape,dtype,with_w", [
+    ((2, 37, 768), torch.float32, True), ((3, 5, 64), torch.bfloat16, True), ((19, 2048), torch.float32, False),
+    ((2, 70, 1536), torch.bfloat16, True),
+])
+def test_add_rmsnorm_forward_backward(pkg, dev, shape, dtype, with_w):
+    # (norm(x + r), x + r) with both outputs used downstream: the gradient of x and of r is the
+    # gradient through the norm plus the one that reaches the sum directly
+    g = torch.Generator().manual_seed(7 + sum(shape))
+    x = (torch.randn(*shape, generator=g) * 1.5).to(dtype)
+    r = (torch.randn(*shape, generator=g) + 0.2).to(dtype)
+    w = (torch.randn(shape[-1], generator=g) * 0.5 + 1.0).to(dtype) if with_w else None
+    dy = torch.randn(*shape, generator=g).to(dtype)
+    dt = torch.randn(*shape, generator=g).to(dtype)
+    xr, rr = x.double().requires_grad_(), r.double().requires_grad_()
+    wr = None if w is None else w.double().requires_grad_()
+    # the kernel rounds the sum to the I/O type before it normalises it (as a separate add would)
+    tr = xr + rr
+    tr_q = tr + (tr.detach().to(dtype).double() - tr.detach())
+    yr = so.rmsnorm_ref(tr_q, wr, 1e-5)
+    (yr * dy.double()).sum().add((tr_q * dt.double()).sum()).backward()
+    xg, rg = x.to(dev).requires_grad_(), r.to(dev).requires_grad_()
+    wg = None if w is None else w.to(dev).requires_grad_()
+    y, total = pkg.add_rmsnorm_fn(xg, rg, wg, 1e-5)
+    torch.autograd.backward([y, total], [dy.to(dev), dt.to(dev)])
+    tol = TOL[dtype]
+    assert torch.equal(total.cpu(), (x.double() + r.double()).to(dtype))   # one rounding of the exact sum
+    assert rel_err(y, yr) <= tol
+    assert rel_err(xg.grad, xr.grad) <= tol and rel_err(rg.grad, rr.grad) <= tol
+    if w is not None:
+        assert rel_err(wg.grad, wr.grad) <= tol
+    # only the normalised output used: no gradient reaches the sum directly
+    xg2, rg2 = x.to(dev).requires_grad_(), r.to(dev).requires_grad_()
+    y2, _ = pkg.add_rmsnorm_fn(xg2, rg2, None if w is None else w.to(dev), 1e-5)
+    y2.backward(dy.to(dev))
+    xr2 = (x.double() + r.double()).to(dtype).double().requires_grad_()
+    so.rmsnorm_ref(xr2, None if w is None else w.double(), 1e-5).backward(dy.double())
+    assert rel_err(xg2.grad, xr2.grad) <= tol and torch.equal(xg2.grad, rg2.grad)
