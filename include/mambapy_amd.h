@@ -142,7 +142,9 @@ size_t mpa_sscan_bwd_workspace_bytes(const mpa_sscan_shape* s);
  * window_out optional (batch, dim, kernel-1): the last kernel-1 inputs, i.e. the cache to
  *            continue from with MambaBlock.step.
  * y has the y_* strides, dy too; dx the g_* strides; dweight (dim, kernel), dbias (dim) float32,
- * overwritten.  No gradient flows into window_in.
+ * overwritten.  No gradient flows into window_in.  window_out may equal window_in (the rolling
+ * cache of a decode loop, updated in place: every (batch, channel) row is read and written by
+ * one thread).
  */
 #define MPA_CONV_SILU 1
 typedef struct mpa_conv_shape {
@@ -211,7 +213,8 @@ int mpa_pscan_bwd(const mpa_pscan_shape* s, const void* A, const void* H, const 
  * Replaces the state update and readout of MambaBlock.ssm_step (mambapy/mamba.py:400-412)
  * for one token: h' = exp(delta*A)*h + delta*B*x ; y = C.h' + D*x, optionally
  * delta = softplus(delta + delta_bias) (mamba.py:398) and y *= silu(z) (mamba.py:373-375).
- *   x, delta, z, y : (batch, dim) io_dtype contiguous;  B, C : (batch, dstate) io_dtype,
+ *   x, delta, y : (batch, dim) io_dtype contiguous;  z : (batch, dim) with row stride z_stride (it
+ *   is a half of the in_proj output, mamba.py:356-357);  B, C : (batch, dstate) io_dtype,
  *   row stride bc_stride;  h_in, h_out : (batch, dim, dstate) float32 contiguous.
  * h_in == NULL means zeros (mamba.py:405-406).  h_out may equal h_in (in-place update);
  * with distinct buffers h_in is left untouched, which is the reference's behaviour
@@ -220,7 +223,8 @@ int mpa_pscan_bwd(const mpa_pscan_shape* s, const void* A, const void* H, const 
 int mpa_ssm_step(const void* x, const void* delta, const float* A, const void* B, const void* C,
                  const float* D, const void* z, const float* delta_bias, const float* h_in,
                  float* h_out, void* y, int64_t batch, int64_t dim, int64_t dstate,
-                 int64_t bc_stride, int32_t io_dtype, int32_t delta_softplus, void* stream);
+                 int64_t bc_stride, int64_t z_stride, int32_t io_dtype, int32_t delta_softplus,
+                 void* stream);
 
 #ifdef __cplusplus
 }

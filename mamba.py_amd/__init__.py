@@ -6,7 +6,7 @@ submodule_search_locations=[".../mamba.py_amd"]), as `__graft_entry__.load_packa
 """
 from . import _lib
 from .scan import PScan, pscan, selective_scan, selective_scan_fn, ssm_step, SelectiveScanFn
-from .conv import CausalConv1dFn, causal_conv1d_fn
+from .conv import CausalConv1dFn, causal_conv1d_fn, causal_conv1d_update
 from .norm import AddRMSNormFn, RMSNormFn, add_rmsnorm_fn, rmsnorm_fn
 from .modules import Mamba, MambaBlock, MambaConfig, ResidualBlock, RMSNorm
 from .language_model import LM
@@ -14,7 +14,7 @@ from .decode import GraphedDecoder
 from .patch import patch_mambapy
 
 __all__ = ["PScan", "pscan", "selective_scan", "selective_scan_fn", "ssm_step",
-           "SelectiveScanFn", "CausalConv1dFn", "causal_conv1d_fn", "RMSNormFn", "rmsnorm_fn",
+           "SelectiveScanFn", "CausalConv1dFn", "causal_conv1d_fn", "causal_conv1d_update", "RMSNormFn", "rmsnorm_fn",
            "AddRMSNormFn", "add_rmsnorm_fn", "Mamba", "MambaBlock", "MambaConfig", "ResidualBlock", "RMSNorm",
            "LM", "GraphedDecoder", "patch_mambapy", "library_path", "library_version"]
 

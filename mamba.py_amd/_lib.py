@@ -76,7 +76,7 @@ def load():
     pp = ctypes.POINTER(PscanShape)
     lib.mpa_pscan_fwd.argtypes = [pp] + [vp] * 4
     lib.mpa_pscan_bwd.argtypes = [pp] + [vp] * 6
-    lib.mpa_ssm_step.argtypes = [vp] * 11 + [i64] * 4 + [i32, i32, vp]
+    lib.mpa_ssm_step.argtypes = [vp] * 11 + [i64] * 5 + [i32, i32, vp]
     cp = ctypes.POINTER(ConvShape)
     lib.mpa_conv1d_fwd.argtypes = [cp] + [vp] * 7
     lib.mpa_conv1d_bwd.argtypes = [cp] + [vp] * 9 + [sz, vp]

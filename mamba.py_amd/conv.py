@@ -78,6 +78,29 @@ class CausalConv1dFn(torch.autograd.Function):
         return (dx, dw.view(wshape).to(wdtype), None if db is None else db.to(bdtype), None, None, None)
 
 
+def causal_conv1d_update(x, window, weight, bias=None, silu=True):
+    """One decode step of the convolution (mambapy/mamba.py:366-369, 379) in one kernel:
+    x : (B, ED) newest input (any row stride);  window : (B, ED, K-1) contiguous rolling cache of
+    the previous inputs, UPDATED IN PLACE (oldest dropped, x appended).  Returns
+    silu(conv) as (B, ED).  No autograd: decoding runs under torch.no_grad()."""
+    _require_gpu(x, window, weight, bias)
+    lib = _lib.load()
+    Bsz, ED = x.shape
+    K = weight.shape[-1]
+    if window.shape != (Bsz, ED, K - 1) or window.dtype != x.dtype or not window.is_contiguous():
+        raise RuntimeError("window must be a contiguous (B, ED, K-1) tensor of x's dtype")
+    x_ = x.detach().unsqueeze(1)
+    w_ = _f32c(weight).view(ED, K)
+    b_ = _f32c(bias)
+    y = torch.empty((Bsz, 1, ED), dtype=x.dtype, device=x.device)
+    shape = _conv_shape(x_, y, y, K, silu)
+    with torch.cuda.device(x.device):
+        rc = lib.mpa_conv1d_fwd(ctypes.byref(shape), _ptr(x_), _ptr(w_), _ptr(b_), _ptr(window), _ptr(y),
+                                _ptr(window), _stream(x.device))
+    _lib.check(rc, "mpa_conv1d_fwd")
+    return y[:, 0]
+
+
 def causal_conv1d_fn(x, weight, bias=None, window=None, silu=True, return_window=False):
     """x : (B, L, ED) (any strides);  weight : (ED, 1, K) or (ED, K), K in 2..4;  bias : (ED).
     window : optional (B, ED, K-1) inputs before step 0 (zeros if None).

@@ -25,6 +25,7 @@ struct StepParams {
     void* y;
     int batch, ED, N;
     int64_t bc_stride;
+    int64_t z_stride;  // row stride of z (elements)
     int softplus;
 };
 
@@ -71,7 +72,7 @@ __global__ void __launch_bounds__(256) ssm_step_kernel(const StepParams p) {
     }
     float yv = __builtin_fmaf(p.D[d], xv, acc);
     if (p.z) {
-        const float zv = load_as_float<IO>(p.z, row);
+        const float zv = load_as_float<IO>(p.z, b * p.z_stride + d);
         yv *= zv * sigmoid_f(zv);
     }
     store_from_float<IO>(p.y, row, yv);
@@ -103,7 +104,7 @@ __global__ void __launch_bounds__(256) ssm_step_quad_kernel(const StepParams p) 
     }
     const float xv = load_as_float<IO>(p.x, row);
     float dv = load_as_float<IO>(p.delta, row);
-    const float zv = p.z ? load_as_float<IO>(p.z, row) : 0.0f;
+    const float zv = p.z ? load_as_float<IO>(p.z, b * p.z_stride + d) : 0.0f;
     const float Dv = p.D[d];
     if (p.softplus) dv = softplus_f(dv + (p.dbias ? p.dbias[d] : 0.0f));
     const float dl2 = dv * kLog2e;
@@ -144,13 +145,13 @@ using namespace mpa;
 extern "C" int mpa_ssm_step(const void* x, const void* delta, const float* A, const void* B,
                             const void* C, const float* D, const void* z, const float* delta_bias,
                             const float* h_in, float* h_out, void* y, int64_t batch, int64_t dim,
-                            int64_t dstate, int64_t bc_stride, int32_t io_dtype,
+                            int64_t dstate, int64_t bc_stride, int64_t z_stride, int32_t io_dtype,
                             int32_t delta_softplus, void* stream) {
     if (!x || !delta || !A || !B || !C || !D || !h_out || !y) return MPA_ERR_NULL_POINTER;
     if (batch <= 0 || dim <= 0 || dstate <= 0 || batch * dim > (int64_t)1 << 40)
         return MPA_ERR_BAD_SHAPE;
     if (io_dtype != MPA_F32 && io_dtype != MPA_BF16) return MPA_ERR_BAD_DTYPE;
-    if (bc_stride < dstate) return MPA_ERR_BAD_STRIDE;
+    if (bc_stride < dstate || (z && z_stride < dim)) return MPA_ERR_BAD_STRIDE;
     if (!delta_softplus && delta_bias) return MPA_ERR_BAD_SHAPE;
     const size_t es = dtype_size(io_dtype);
     if (!aligned_to(x, es) || !aligned_to(delta, es) || !aligned_to(B, es) || !aligned_to(C, es) ||
@@ -164,6 +165,7 @@ extern "C" int mpa_ssm_step(const void* x, const void* delta, const float* A, co
     p.x = x; p.delta = delta; p.Bm = B; p.C = C; p.z = z; p.A = A; p.D = D; p.dbias = delta_bias;
     p.hin = h_in; p.hout = h_out; p.y = y;
     p.batch = (int)batch; p.ED = (int)dim; p.N = (int)dstate; p.bc_stride = bc_stride;
+    p.z_stride = z_stride;
     p.softplus = delta_softplus ? 1 : 0;
     const int64_t rows = batch * dim;
     dim3 grid((unsigned)((rows + 255) / 256));

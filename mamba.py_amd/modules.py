@@ -16,7 +16,7 @@ import torch
 import torch.nn as nn
 import torch.nn.functional as F
 
-from .conv import causal_conv1d_fn
+from .conv import causal_conv1d_fn, causal_conv1d_update
 from .norm import add_rmsnorm_fn, rmsnorm_fn, rmsnorm_supported
 from .scan import selective_scan, selective_scan_fn, ssm_step
 
@@ -142,7 +142,23 @@ class MambaBlock(nn.Module):
         return dlow, Bm, C
 
     def _A(self):
-        return -torch.exp(self.A_log.float())
+        """A = -exp(A_log) (mambapy/mamba.py:239).  Without autograd (decode, prefill) the value
+        is kept in one persistent buffer that is refreshed in place when A_log has changed, so
+        a token step does not spend two kernels per layer on it and a captured HIP graph keeps
+        reading the same memory."""
+        if torch.is_grad_enabled() and self.A_log.requires_grad:
+            return -torch.exp(self.A_log.float())
+        key = (self.A_log._version, self.A_log.data_ptr(), self.A_log.device)
+        if getattr(self, "_A_key", None) != key:
+            with torch.no_grad():
+                fresh = -torch.exp(self.A_log.detach().float())
+                buf = getattr(self, "_A_buf", None)
+                if buf is None or buf.shape != fresh.shape or buf.device != fresh.device:
+                    self._A_buf = fresh
+                else:
+                    buf.copy_(fresh)
+            self._A_key = key
+        return self._A_buf
 
     # -- training / prefill ---------------------------------------------------------------
     def forward(self, x, cache: Optional[Tuple] = None, return_cache: bool = False):
@@ -211,14 +227,20 @@ class MambaBlock(nn.Module):
         h, inputs = cache
         xz = self.in_proj(x)
         xin, z = xz.chunk(2, dim=1)
-        window = torch.cat([inputs, xin.unsqueeze(2)], dim=2)            # (B, ED, d_conv)
-        xc = (window * self.conv1d.weight[:, 0, :]).sum(-1)
-        if self.conv1d.bias is not None:
-            xc = xc + self.conv1d.bias
-        xs = F.silu(xc)
+        if 2 <= self.config.d_conv <= 4 and not torch.is_grad_enabled():
+            # convolution over (cache, newest input) + bias + silu and the new cache: one kernel
+            xs, window = causal_conv1d_fn(xin.unsqueeze(1), self.conv1d.weight, self.conv1d.bias,
+                                          window=inputs, return_window=True)
+            xs = xs[:, 0]
+        else:
+            full = torch.cat([inputs, xin.unsqueeze(2)], dim=2)          # (B, ED, d_conv)
+            xc = (full * self.conv1d.weight[:, 0, :]).sum(-1)
+            if self.conv1d.bias is not None:
+                xc = xc + self.conv1d.bias
+            xs, window = F.silu(xc), full[:, :, 1:]
         y, h = self.ssm_step(xs, h, z=z)
         out = self.out_proj(y)
-        return out, (h, window[:, :, 1:])
+        return out, (h, window)
 
     def ssm_step(self, x, h, z=None, inplace: bool = False):
         """x : (B, ED), h : (B, ED, N) or None -> (y, h'); mambapy/mamba.py:384-414.  With z
@@ -235,12 +257,16 @@ class MambaBlock(nn.Module):
         place.  Same arithmetic as step()."""
         xz = self.in_proj(x)
         xin, z = xz.chunk(2, dim=1)
-        full = torch.cat([window, xin.unsqueeze(2)], dim=2)              # (B, ED, d_conv)
-        xc = (full * self.conv1d.weight[:, 0, :]).sum(-1)
-        if self.conv1d.bias is not None:
-            xc = xc + self.conv1d.bias
-        y, _ = self.ssm_step(F.silu(xc), h, z=z, inplace=True)
-        window.copy_(full[:, :, 1:])
+        if 2 <= self.config.d_conv <= 4 and window.is_contiguous() and window.dtype == xin.dtype:
+            xs = causal_conv1d_update(xin, window, self.conv1d.weight, self.conv1d.bias)
+        else:
+            full = torch.cat([window, xin.unsqueeze(2)], dim=2)          # (B, ED, d_conv)
+            xc = (full * self.conv1d.weight[:, 0, :]).sum(-1)
+            if self.conv1d.bias is not None:
+                xc = xc + self.conv1d.bias
+            xs = F.silu(xc)
+            window.copy_(full[:, :, 1:])
+        y, _ = self.ssm_step(xs, h, z=z, inplace=True)
         return self.out_proj(y)
 
 

@@ -265,7 +265,7 @@ def ssm_step(x, delta, A, B, C, D, h=None, z=None, delta_bias=None, delta_softpl
     N = A.shape[-1]
     x_ = x.detach().contiguous()
     delta_ = delta.detach().to(dt).contiguous()
-    z_ = None if z is None else z.detach().to(dt).contiguous()
+    z_ = None if z is None else _rows_unit_stride(z.detach().to(dt))   # a half of in_proj's output
     B_ = _rows_unit_stride(B.detach().to(dt))
     C_ = _rows_unit_stride(C.detach().to(dt))
     if B_.stride(0) != C_.stride(0):
@@ -283,6 +283,7 @@ def ssm_step(x, delta, A, B, C, D, h=None, z=None, delta_bias=None, delta_softpl
     with torch.cuda.device(x.device):
         rc = lib.mpa_ssm_step(_ptr(x_), _ptr(delta_), _ptr(A_), _ptr(B_), _ptr(C_), _ptr(D_),
                               _ptr(z_), _ptr(bias_), _ptr(h), _ptr(h_out), _ptr(y), Bsz, ED, N,
-                              B_.stride(0), io, 1 if delta_softplus else 0, _stream(x.device))
+                              B_.stride(0), 0 if z_ is None else z_.stride(0), io,
+                              1 if delta_softplus else 0, _stream(x.device))
     _lib.check(rc, "mpa_ssm_step")
     return y, h_out

@@ -106,3 +106,24 @@ def test_conv_full_size_c4_layer_properties(pkg, dev):
         p1 = pkg.causal_conv1d_fn(x, w, None, silu=False).float()
         p2 = pkg.causal_conv1d_fn((2 * x.float()).to(torch.bfloat16), w, None, silu=False).float()
         assert rel_err(p2, 2 * p1) <= TOL[torch.bfloat16]
+
+
+@pytest.mark.parametrize("K,dtype", [(4, torch.float32), (3, torch.float32), (2, torch.bfloat16), (4, torch.bfloat16)])
+def test_decode_update_rolls_the_window_in_place(pkg, dev, K, dtype):
+    # mambapy/mamba.py:366-369, 379: conv over (cache, newest input), then the cache drops its oldest
+    g = torch.Generator().manual_seed(40 + K)
+    Bsz, ED = 3, 200
+    w = torch.randn(ED, 1, K, generator=g)
+    b = torch.randn(ED, generator=g)
+    window = torch.randn(Bsz, ED, K - 1, generator=g).to(dtype)
+    xz = torch.randn(Bsz, 2 * ED, generator=g).to(dtype)       # x is the first half of a wider row
+    win_dev = window.to(dev)
+    ref_win = window.double()
+    for _ in range(3):
+        x = xz[:, :ED]
+        want, ref_win = so.conv_window_step_ref(ref_win, x.double(), w.double(), b.double())
+        want = want * torch.sigmoid(want)
+        got = pkg.causal_conv1d_update(xz.to(dev)[:, :ED], win_dev, w.to(dev), b.to(dev))
+        assert rel_err(got, want) <= TOL[dtype]
+        assert torch.equal(win_dev.cpu().double(), ref_win)    # the cache holds inputs, bit for bit
+        xz = xz.roll(1, 0) * 0.5 + 0.1
