@@ -193,6 +193,68 @@ def bench_pscan(args, torch, pkg, dev):
     print(json.dumps(out))
 
 
+def bench_layer_kernels(args, torch, pkg, dev):
+    """The kernels either side of the scan in one layer, at the configs[4] layer shape (B=8,
+    L=4096, d_model=768, ED=1536, bf16): causal conv1d + bias + silu reading the x half of the
+    in_proj output in place, and RMSNorm with the residual add folded in; forward and backward
+    each, timed with HIP events on the launch stream, against the HBM roofline."""
+    Bsz, L, D, ED, K = 8, 4096, 768, 1536, 4
+    g = torch.Generator().manual_seed(1006)
+    bf = torch.bfloat16
+    # the x half of an in_proj output, as a leaf: a strided view, no slice node in the timed graph
+    xh = torch.randn(Bsz, L, 2 * ED, generator=g).to(bf).to(dev)[..., :ED].requires_grad_()
+    w = (torch.randn(ED, 1, K, generator=g) * 0.3).to(dev).requires_grad_()
+    b = torch.randn(ED, generator=g).to(dev).requires_grad_()
+    gy = torch.randn(Bsz, L, ED, generator=g).to(bf).to(dev)
+    h = torch.randn(Bsz, L, D, generator=g).to(bf).to(dev).requires_grad_()
+    r = torch.randn(Bsz, L, D, generator=g).to(bf).to(dev).requires_grad_()
+    nw = torch.ones(D, device=dev, requires_grad=True)
+    gn = torch.randn(Bsz, L, D, generator=g).to(bf).to(dev)
+    gt = torch.randn(Bsz, L, D, generator=g).to(bf).to(dev)
+    steps, warmup = max(5, args.steps // 2), 3
+
+    def step(ev=None):
+        for t in (xh, w, b, h, r, nw):
+            t.grad = None
+        rec = (lambda i: ev[i].record()) if ev else (lambda i: None)
+        rec(0)
+        y = pkg.causal_conv1d_fn(xh, w, b)
+        rec(1)
+        y.backward(gy)
+        rec(2)
+        n, tot = pkg.add_rmsnorm_fn(h, r, nw, 1e-5)
+        rec(3)
+        torch.autograd.backward([n, tot], [gn, gt])
+        rec(4)
+
+    t = _timed(torch, step, steps, warmup)
+    evs = [[torch.cuda.Event(enable_timing=True) for _ in range(5)] for _ in range(steps)]
+    for ev in evs:
+        step(ev)
+    torch.cuda.synchronize()
+    ms = [sum(e[i].elapsed_time(e[i + 1]) for e in evs) / steps for i in range(4)]
+    ce, ne = Bsz * L * ED * 2, Bsz * L * D * 2          # bytes of one conv / norm activation tensor
+    # conv: fwd x in, y out; bwd x, dy in, dx out.  norm+add: fwd x, residual in, y, sum out;
+    # bwd sum, dy, dsum in, dx out.
+    alg = [2 * ce, 3 * ce, 4 * ne, 4 * ne]
+    names = ["conv1d_fwd_kernel", "conv1d_bwd_kernel (+ finish)", "rmsnorm_fwd_kernel (+ residual add)",
+             "rmsnorm_bwd_kernel (+ finish)"]
+    per = [{"kernel": k, "ms": m, "algorithmic_bytes": a, "achieved": a / (m * 1e-3) / 1e9, "unit": "GB/s",
+            "frac": a / (m * 1e-3) / 1e9 / HBM_PEAK_GBS} for k, m, a in zip(names, ms, alg)]
+    slow = max(per, key=lambda e: e["ms"])
+    out = {
+        "metric": "conv1d + add-RMSNorm kernels fwd+bwd GB/s, mamba-130m layer shape B=8 L=4096 bf16",
+        "value": sum(alg) / t / 1e9, "unit": "GB/s", "higher_is_better": True,
+        "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": t * 1e3,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f32 arithmetic, bf16 I/O", "data": "synthetic (seeded)",
+        "config": {"workload": "configs[4] layer shape: conv over the x half of (8,4096,3072), norm of (8,4096,768)"},
+        "roofline": {"bound": "hbm", "kernel": slow["kernel"], "achieved": slow["achieved"], "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": slow["frac"], "traffic": None},
+        "kernels": per,
+    }
+    print(json.dumps(out))
+
+
 def bench_lm_forward(args, torch, pkg, dev, L):
     """configs[4]: random-init LM forward at the mamba-130m architecture, bf16 weights and
     activations, fp32 scan state, B=8, uniform-random token ids."""
@@ -227,7 +289,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS) + ["c3", "c4", "c4-3000", "pscan"],
+    ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS) + ["c3", "c4", "c4-3000", "pscan", "layer"],
                     help="c2 (default) is the headline workload; c3 = decode step, c4 = LM forward "
                          "(reported with their own metric, same one-line schema)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -251,6 +313,8 @@ def main():
         return bench_decode(args, torch, pkg, dev)
     if args.workload == "pscan":
         return bench_pscan(args, torch, pkg, dev)
+    if args.workload == "layer":
+        return bench_layer_kernels(args, torch, pkg, dev)
     if args.workload.startswith("c4"):
         return bench_lm_forward(args, torch, pkg, dev, 3000 if args.workload == "c4-3000" else 4096)
 

@@ -2,11 +2,13 @@
 // (mambapy/mamba.py:416-433; no weight under muP).
 //
 // The reference evaluates this as five elementwise / reduction kernels per call (pow, mean,
-// add + rsqrt, two multiplies), each a full pass over the activations.  Here one wave owns one
-// row: it reads the row with 16-byte loads, sums the squares across its lanes with lane
-// exchanges, and writes the scaled row; the second read of the row comes from cache.  The
-// kernels are bound by HBM: forward x in, y out; backward x, dy in, dx out, plus per-block
-// partial sums of dweight that a second kernel adds up in a fixed order.
+// add + rsqrt, two multiplies), each a full pass over the activations.  Here one wave owns a
+// row: it reads the row once with 16-byte loads into registers, sums across its lanes with six
+// DPP additions (no LDS round trips), and writes the result from the same registers.  The
+// kernels are bound by HBM, so they are organised to keep bytes in flight: the forward holds two
+// rows per wave at a time, the backward requests the next row before it works on the current
+// one.  Backward: dweight is summed per wave in registers, per block through LDS, and over the
+// blocks by a second kernel in a fixed order (no float atomics).
 //
 // The residual add that precedes every norm of the layer stack (mambapy/mamba.py:106-112:
 // output = mixer(norm(x)) + x, then the next layer's norm reads it) can ride along: the forward
@@ -16,7 +18,7 @@
 
 namespace mpa {
 
-constexpr int kNormRowsPerWave = 16;  // backward: rows walked by one wave (dweight partials per wave)
+constexpr int kNormBwdWaves = 8;  // waves per block of the backward kernel (one dweight partial per block)
 
 template <typename IO>
 struct RowVec;
@@ -50,93 +52,170 @@ struct RowVec<bf16_t> {
     }
 };
 
+// v + (v moved by the DPP control CTRL); rows outside ROW_MASK add zero
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ float dpp_add(float v) {
+    const int moved = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, ROW_MASK, 0xf, false);
+    return v + __builtin_bit_cast(float, moved);
+}
+// Sum over the 64 lanes, returned wave-uniform.  Four exchanges inside every row of 16 lanes
+// (after each, the partners hold the same partial sum, so the mirrors act as lane ^ 4 and
+// lane ^ 8), then lane 15 of row 0 / 2 into rows 1 / 3 and lane 31 into rows 2 and 3: lane 63
+// holds the total.
 __device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-    for (int m = 32; m >= 1; m >>= 1) v += __shfl_xor(v, m);
-    return v;
+    v = dpp_add<0xB1, 0xf>(v);   // quad_perm:[1,0,3,2]
+    v = dpp_add<0x4E, 0xf>(v);   // quad_perm:[2,3,0,1]
+    v = dpp_add<0x141, 0xf>(v);  // row_half_mirror
+    v = dpp_add<0x140, 0xf>(v);  // row_mirror
+    v = dpp_add<0x142, 0xa>(v);  // row_bcast:15
+    v = dpp_add<0x143, 0xc>(v);  // row_bcast:31
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
 }
 
-// rows x d, contiguous rows; d a multiple of the vector width.  rstd (rows) is optional.
-// With `res`: the row that is normalised is round(x + res), also written to `sum_out`.
-template <typename IO>
+// rows x d, contiguous rows; d a multiple of the vector width, at most MAXV vectors per lane.
+// A wave takes R consecutive rows and holds all of them in registers.  With `res` the row that
+// is normalised is round(x + res), also written to `sum_out`.  rstd (rows) is optional.
+template <typename IO, int MAXV, int R>
 __global__ void __launch_bounds__(256) rmsnorm_fwd_kernel(const IO* __restrict__ x, const IO* __restrict__ res,
                                                           const float* __restrict__ w, IO* __restrict__ y,
                                                           IO* __restrict__ sum_out, float* __restrict__ rstd_out,
                                                           int64_t rows, int d, float eps) {
     typedef RowVec<IO> V;
+    typedef typename V::T VT;
     const int lane = threadIdx.x & (kWave - 1);
-    const int64_t row = (int64_t)blockIdx.x * (blockDim.x / kWave) + (threadIdx.x / kWave);
-    if (row >= rows) return;
+    const int64_t row0 = ((int64_t)blockIdx.x * (blockDim.x / kWave) + (threadIdx.x / kWave)) * R;
+    if (row0 >= rows) return;
     const int nvec = d / V::kN;
-    const typename V::T* xr = reinterpret_cast<const typename V::T*>(x + row * d);
-    typename V::T* yr = reinterpret_cast<typename V::T*>(y + row * d);
-    const typename V::T* rr = reinterpret_cast<const typename V::T*>(res + row * d);
-    typename V::T* sr = reinterpret_cast<typename V::T*>(sum_out + row * d);
-    auto load_row = [&](int i, float (&f)[V::kN]) {
-        V::unpack(xr[i], f);
-        if (res) {
-            float g[V::kN];
-            V::unpack(rr[i], g);
+    VT xv[R][MAXV], rv[R][MAXV];
 #pragma unroll
-            for (int j = 0; j < V::kN; ++j) f[j] = to_float(from_float<IO>(f[j] + g[j]));
+    for (int r = 0; r < R; ++r) {
+        const int64_t row = row0 + r < rows ? row0 + r : rows - 1;  // a clamped copy is not stored
+        const VT* xr = reinterpret_cast<const VT*>(x + row * d);
+        const VT* rr = reinterpret_cast<const VT*>(res + row * d);
+#pragma unroll
+        for (int v = 0; v < MAXV; ++v) {
+            const int i = lane + v * kWave;
+            if (i < nvec) {
+                xv[r][v] = xr[i];
+                if (res) rv[r][v] = rr[i];
+            }
         }
-    };
-    float ss = 0.0f;
-    for (int i = lane; i < nvec; i += kWave) {
-        float f[V::kN];
-        load_row(i, f);
-        if (res) sr[i] = V::pack(f);
-#pragma unroll
-        for (int j = 0; j < V::kN; ++j) ss = __builtin_fmaf(f[j], f[j], ss);
     }
-    const float rstd = __builtin_amdgcn_rsqf(wave_sum(ss) / (float)d + eps);
-    if (rstd_out && lane == 0) rstd_out[row] = rstd;
-    for (int i = lane; i < nvec; i += kWave) {
-        float f[V::kN], o[V::kN];
-        load_row(i, f);
+    float wv[MAXV][V::kN];
 #pragma unroll
-        for (int j = 0; j < V::kN; ++j) o[j] = f[j] * rstd * (w ? w[i * V::kN + j] : 1.0f);
-        yr[i] = V::pack(o);
+    for (int v = 0; v < MAXV; ++v) {
+        const int i = lane + v * kWave;
+#pragma unroll
+        for (int j = 0; j < V::kN; ++j) wv[v][j] = (w && i < nvec) ? w[i * V::kN + j] : 1.0f;
+    }
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        if (row0 + r >= rows) break;
+        const int64_t row = row0 + r;
+        VT* yr = reinterpret_cast<VT*>(y + row * d);
+        VT* sr = reinterpret_cast<VT*>(sum_out + row * d);
+        float f[MAXV][V::kN];
+        float ss = 0.0f;
+#pragma unroll
+        for (int v = 0; v < MAXV; ++v) {
+            const int i = lane + v * kWave;
+            if (i < nvec) {
+                V::unpack(xv[r][v], f[v]);
+                if (res) {
+                    float g[V::kN];
+                    V::unpack(rv[r][v], g);
+#pragma unroll
+                    for (int j = 0; j < V::kN; ++j) f[v][j] = to_float(from_float<IO>(f[v][j] + g[j]));
+                    sr[i] = V::pack(f[v]);
+                }
+#pragma unroll
+                for (int j = 0; j < V::kN; ++j) ss = __builtin_fmaf(f[v][j], f[v][j], ss);
+            }
+        }
+        const float rstd = __builtin_amdgcn_rsqf(wave_sum(ss) / (float)d + eps);
+        if (rstd_out && lane == 0) rstd_out[row] = rstd;
+#pragma unroll
+        for (int v = 0; v < MAXV; ++v) {
+            const int i = lane + v * kWave;
+            if (i < nvec) {
+                float o[V::kN];
+#pragma unroll
+                for (int j = 0; j < V::kN; ++j) o[j] = f[v][j] * rstd * wv[v][j];
+                yr[i] = V::pack(o);
+            }
+        }
     }
 }
 
-// dx = rstd * (w*dy) - x * rstd^3 * mean(w*dy*x);  dweight[c] = sum_rows dy*x*rstd.
-// A wave walks kNormRowsPerWave rows and writes its dweight sums as one row of `part`.
-// `dres` (optional) is added to dx: the gradient that reaches the normalised row from its
-// other users (the residual stream).
+// dx = rstd * (w*dy) - x * rstd^3 * mean(w*dy*x) [+ dres];  dweight[c] = sum_rows dy*x*rstd.
+// A wave walks `rpw` consecutive rows, requesting row r+1 before it works on row r; its dweight
+// sums stay in registers, the kNormBwdWaves waves of a block add theirs through LDS and the
+// block writes one row of `part`.  `dres` (optional) is the gradient that reaches the
+// normalised row from its other users (the residual stream).  Rows of more than two vectors per
+// lane (LEAN) would not fit the register file that way: they are walked without the prefetch
+// and read the weight from cache instead of registers.
 template <typename IO, int MAXV>
-__global__ void __launch_bounds__(256) rmsnorm_bwd_kernel(const IO* __restrict__ x, const float* __restrict__ w,
-                                                          const IO* __restrict__ dy, const IO* __restrict__ dres,
-                                                          IO* __restrict__ dx, float* __restrict__ part,
-                                                          int64_t rows, int d, float eps) {
+__global__ void __launch_bounds__(kNormBwdWaves* kWave) rmsnorm_bwd_kernel(
+    const IO* __restrict__ x, const float* __restrict__ w, const IO* __restrict__ dy, const IO* __restrict__ dres,
+    IO* __restrict__ dx, float* __restrict__ part, int64_t rows, int d, float eps, int rpw) {
     typedef RowVec<IO> V;
+    typedef typename V::T VT;
+    extern __shared__ float sacc[];  // [kNormBwdWaves][d]
     const int lane = threadIdx.x & (kWave - 1);
-    const int64_t wave = (int64_t)blockIdx.x * (blockDim.x / kWave) + (threadIdx.x / kWave);
+    const int wib = wave_id();
+    const int64_t row_begin = ((int64_t)blockIdx.x * kNormBwdWaves + wib) * rpw;
+    const int64_t row_end = row_begin + rpw < rows ? row_begin + rpw : rows;
     const int nvec = d / V::kN;
-    float dwacc[MAXV][V::kN];
+    constexpr bool LEAN = MAXV > 2;
+    float wv[LEAN ? 1 : MAXV][V::kN], dwacc[MAXV][V::kN];
 #pragma unroll
-    for (int v = 0; v < MAXV; ++v)
+    for (int v = 0; v < MAXV; ++v) {
+        const int i = lane + v * kWave;
 #pragma unroll
-        for (int j = 0; j < V::kN; ++j) dwacc[v][j] = 0.0f;
-    for (int r = 0; r < kNormRowsPerWave; ++r) {
-        const int64_t row = wave * kNormRowsPerWave + r;
-        if (row >= rows) break;
-        const typename V::T* xr = reinterpret_cast<const typename V::T*>(x + row * d);
-        const typename V::T* gr = reinterpret_cast<const typename V::T*>(dy + row * d);
-        typename V::T* dr = reinterpret_cast<typename V::T*>(dx + row * d);
-        const typename V::T* qr = reinterpret_cast<const typename V::T*>(dres + row * d);
+        for (int j = 0; j < V::kN; ++j) {
+            if (!LEAN) wv[v][j] = (w && i < nvec) ? w[i * V::kN + j] : 1.0f;
+            dwacc[v][j] = 0.0f;
+        }
+    }
+    auto weights = [&](int v, int i, float (&wj)[V::kN]) {
+#pragma unroll
+        for (int j = 0; j < V::kN; ++j) wj[j] = LEAN ? (w ? w[i * V::kN + j] : 1.0f) : wv[LEAN ? 0 : v][j];
+    };
+    struct Raw {
+        VT x[MAXV], g[MAXV], q[MAXV];
+    };
+    auto load_row = [&](int64_t row, Raw& raw) {
+        const VT* xr = reinterpret_cast<const VT*>(x + row * d);
+        const VT* gr = reinterpret_cast<const VT*>(dy + row * d);
+        const VT* qr = reinterpret_cast<const VT*>(dres + row * d);
+#pragma unroll
+        for (int v = 0; v < MAXV; ++v) {
+            const int i = lane + v * kWave;
+            if (i < nvec) {
+                raw.x[v] = xr[i];
+                raw.g[v] = gr[i];
+                if (dres) raw.q[v] = qr[i];
+            }
+        }
+    };
+    Raw cur, nxt;
+    if (row_begin < row_end) load_row(row_begin, cur);
+    for (int64_t row = row_begin; row < row_end; ++row) {
+        if (!LEAN && row + 1 < row_end) load_row(row + 1, nxt);
+        VT* dr = reinterpret_cast<VT*>(dx + row * d);
         float ss = 0.0f, sg = 0.0f;
 #pragma unroll
         for (int v = 0; v < MAXV; ++v) {
             const int i = lane + v * kWave;
             if (i < nvec) {
-                float f[V::kN], g[V::kN];
-                V::unpack(xr[i], f);
-                V::unpack(gr[i], g);
+                float f[V::kN], g[V::kN], wj[V::kN];
+                V::unpack(cur.x[v], f);
+                V::unpack(cur.g[v], g);
+                weights(v, i, wj);
 #pragma unroll
                 for (int j = 0; j < V::kN; ++j) {
                     ss = __builtin_fmaf(f[j], f[j], ss);
-                    sg = __builtin_fmaf(g[j] * (w ? w[i * V::kN + j] : 1.0f), f[j], sg);
+                    sg = __builtin_fmaf(g[j] * wj[j], f[j], sg);
                 }
             }
         }
@@ -146,37 +225,49 @@ __global__ void __launch_bounds__(256) rmsnorm_bwd_kernel(const IO* __restrict__
         for (int v = 0; v < MAXV; ++v) {
             const int i = lane + v * kWave;
             if (i < nvec) {
-                float f[V::kN], g[V::kN], o[V::kN];
-                V::unpack(xr[i], f);
-                V::unpack(gr[i], g);
+                float f[V::kN], g[V::kN], wj[V::kN], o[V::kN];
+                V::unpack(cur.x[v], f);
+                V::unpack(cur.g[v], g);
+                weights(v, i, wj);
 #pragma unroll
                 for (int j = 0; j < V::kN; ++j) {
-                    o[j] = __builtin_fmaf(g[j] * (w ? w[i * V::kN + j] : 1.0f), rstd, -f[j] * c);
+                    o[j] = __builtin_fmaf(g[j] * wj[j], rstd, -f[j] * c);
                     dwacc[v][j] = __builtin_fmaf(g[j] * rstd, f[j], dwacc[v][j]);
                 }
                 if (dres) {
                     float q[V::kN];
-                    V::unpack(qr[i], q);
+                    V::unpack(cur.q[v], q);
 #pragma unroll
                     for (int j = 0; j < V::kN; ++j) o[j] += q[j];
                 }
                 dr[i] = V::pack(o);
             }
         }
-    }
-    if (part) {
-        float* pr = part + wave * d;
-#pragma unroll
-        for (int v = 0; v < MAXV; ++v) {
-            const int i = lane + v * kWave;
-            if (i < nvec)
-#pragma unroll
-                for (int j = 0; j < V::kN; ++j) pr[i * V::kN + j] = dwacc[v][j];
+        if (LEAN) {
+            if (row + 1 < row_end) load_row(row + 1, cur);
+        } else {
+            cur = nxt;
         }
+    }
+    if (!part) return;  // uniform over the grid
+    float* mine = sacc + wib * d;
+#pragma unroll
+    for (int v = 0; v < MAXV; ++v) {
+        const int i = lane + v * kWave;
+        if (i < nvec)
+#pragma unroll
+            for (int j = 0; j < V::kN; ++j) mine[i * V::kN + j] = dwacc[v][j];
+    }
+    __syncthreads();
+    for (int c = threadIdx.x; c < d; c += kNormBwdWaves * kWave) {
+        float s = sacc[c];
+#pragma unroll
+        for (int k = 1; k < kNormBwdWaves; ++k) s += sacc[k * d + c];
+        part[(int64_t)blockIdx.x * d + c] = s;
     }
 }
 
-// dweight[c] = sum over the per-wave partial rows, fixed order (32 columns x 32 row groups per block)
+// dweight[c] = sum over the per-block partial rows, fixed order (32 columns x 32 row groups per block)
 constexpr int kNormFinCols = 32, kNormFinRows = 32;
 __global__ void __launch_bounds__(1024) rmsnorm_bwd_finish_kernel(const float* part, float* dweight, int d,
                                                                   int64_t nparts) {
@@ -201,11 +292,66 @@ static int norm_validate(int64_t rows, int64_t d, int io_dtype) {
     return MPA_OK;
 }
 
-static int64_t norm_waves(int64_t rows) { return (rows + kNormRowsPerWave - 1) / kNormRowsPerWave; }
+// vectors per lane, rounded up to a power of two: 1, 2, 4, 8
+static int norm_maxv(int64_t d, int io_dtype) {
+    const int vec = io_dtype == MPA_BF16 ? 8 : 4;
+    const int nv = (int)((d / vec + kWave - 1) / kWave);
+    return nv <= 1 ? 1 : nv <= 2 ? 2 : nv <= 4 ? 4 : 8;
+}
+
+// Backward launch: rows per wave chosen for about 4096 waves (16 per CU) when the problem has
+// that many rows, at most 16 rows per wave; one dweight partial per block.
+struct NormBwdPlan {
+    int rpw;
+    int64_t blocks;
+};
+static NormBwdPlan norm_bwd_plan(int64_t rows) {
+    int64_t rpw = rows / 4096;
+    rpw = rpw < 1 ? 1 : rpw > 16 ? 16 : rpw;
+    const int64_t waves = (rows + rpw - 1) / rpw;
+    return NormBwdPlan{(int)rpw, (waves + kNormBwdWaves - 1) / kNormBwdWaves};
+}
+
+template <typename IO, int MAXV>
+static int launch_norm_fwd(const void* x, const void* res, const float* w, void* y, void* sum_out, float* rstd,
+                           int64_t rows, int d, float eps, hipStream_t st) {
+    constexpr int R = MAXV <= 2 ? 2 : 1;
+    const int64_t waves = (rows + R - 1) / R;
+    hipLaunchKernelGGL((rmsnorm_fwd_kernel<IO, MAXV, R>), dim3((unsigned)((waves + 3) / 4)), dim3(256), 0, st,
+                       static_cast<const IO*>(x), static_cast<const IO*>(res), w, static_cast<IO*>(y),
+                       static_cast<IO*>(sum_out), rstd, rows, d, eps);
+    return check_launch();
+}
+
+template <typename IO, int MAXV>
+static int launch_norm_bwd(const void* x, const float* w, const void* dy, const void* dsum, void* dx, float* part,
+                           int64_t rows, int d, float eps, hipStream_t st) {
+    const NormBwdPlan plan = norm_bwd_plan(rows);
+    const size_t lds = part ? (size_t)kNormBwdWaves * d * sizeof(float) : 0;
+    // the widest rows of this instantiation need more than the 64 KB a kernel gets by default
+    static const int attr_rc = allow_dynamic_lds(rmsnorm_bwd_kernel<IO, MAXV>,
+                                                 (size_t)kNormBwdWaves * MAXV * kWave * RowVec<IO>::kN * sizeof(float));
+    if (attr_rc != MPA_OK) return attr_rc;
+    hipLaunchKernelGGL((rmsnorm_bwd_kernel<IO, MAXV>), dim3((unsigned)plan.blocks), dim3(kNormBwdWaves * kWave), lds,
+                       st, static_cast<const IO*>(x), w, static_cast<const IO*>(dy), static_cast<const IO*>(dsum),
+                       static_cast<IO*>(dx), part, rows, d, eps, plan.rpw);
+    return check_launch();
+}
 
 }  // namespace mpa
 
 using namespace mpa;
+
+#define MPA_NORM_DISPATCH(FN, ...)                                                     \
+    (io_dtype == MPA_F32                                                               \
+         ? (maxv == 1   ? FN<float, 1>(__VA_ARGS__)                                    \
+            : maxv == 2 ? FN<float, 2>(__VA_ARGS__)                                    \
+            : maxv == 4 ? FN<float, 4>(__VA_ARGS__)                                    \
+                        : FN<float, 8>(__VA_ARGS__))                                   \
+         : (maxv == 1   ? FN<bf16_t, 1>(__VA_ARGS__)                                   \
+            : maxv == 2 ? FN<bf16_t, 2>(__VA_ARGS__)                                   \
+            : maxv == 4 ? FN<bf16_t, 4>(__VA_ARGS__)                                   \
+                        : FN<bf16_t, 8>(__VA_ARGS__)))
 
 extern "C" int mpa_rmsnorm_fwd(const void* x, const void* residual, const float* weight, void* y, void* sum_out,
                                float* rstd, int64_t rows, int64_t d, float eps, int32_t io_dtype, void* stream) {
@@ -216,22 +362,13 @@ extern "C" int mpa_rmsnorm_fwd(const void* x, const void* residual, const float*
         (residual && (!aligned_to(residual, 16) || !aligned_to(sum_out, 16))))
         return MPA_ERR_MISALIGNED;
     hipStream_t st = static_cast<hipStream_t>(stream);
-    dim3 grid((unsigned)((rows + 3) / 4)), block(256);
-    if (io_dtype == MPA_F32)
-        hipLaunchKernelGGL(rmsnorm_fwd_kernel<float>, grid, block, 0, st, static_cast<const float*>(x),
-                           static_cast<const float*>(residual), weight, static_cast<float*>(y),
-                           static_cast<float*>(sum_out), rstd, rows, (int)d, eps);
-    else
-        hipLaunchKernelGGL(rmsnorm_fwd_kernel<bf16_t>, grid, block, 0, st, static_cast<const bf16_t*>(x),
-                           static_cast<const bf16_t*>(residual), weight, static_cast<bf16_t*>(y),
-                           static_cast<bf16_t*>(sum_out), rstd, rows, (int)d, eps);
-    return check_launch();
+    const int maxv = norm_maxv(d, io_dtype);
+    return MPA_NORM_DISPATCH(launch_norm_fwd, x, residual, weight, y, sum_out, rstd, rows, (int)d, eps, st);
 }
 
 extern "C" size_t mpa_rmsnorm_bwd_workspace_bytes(int64_t rows, int64_t d) {
     if (rows <= 0 || d <= 0) return 0;
-    const int64_t waves = (norm_waves(rows) + 3) / 4 * 4;
-    return ((size_t)waves * d * sizeof(float) + 255) / 256 * 256;
+    return ((size_t)norm_bwd_plan(rows).blocks * d * sizeof(float) + 255) / 256 * 256;
 }
 
 extern "C" int mpa_rmsnorm_bwd(const void* x, const float* weight, const void* dy, const void* dsum, void* dx,
@@ -247,32 +384,11 @@ extern "C" int mpa_rmsnorm_bwd(const void* x, const float* weight, const void* d
         return MPA_ERR_MISALIGNED;
     if (weight && workspace_bytes < mpa_rmsnorm_bwd_workspace_bytes(rows, d)) return MPA_ERR_WORKSPACE;
     hipStream_t st = static_cast<hipStream_t>(stream);
-    const int64_t waves = norm_waves(rows);
-    dim3 grid((unsigned)((waves + 3) / 4)), block(256);
     float* part = weight ? static_cast<float*>(workspace) : nullptr;
-    const int vec = io_dtype == MPA_BF16 ? 8 : 4;
-    const int nv = (int)((d / vec + kWave - 1) / kWave);  // vectors per lane: 1..8
-#define MPA_NORM_CASE(IO_, MV_)                                                                               \
-    hipLaunchKernelGGL((rmsnorm_bwd_kernel<IO_, MV_>), grid, block, 0, st, static_cast<const IO_*>(x), weight, \
-                       static_cast<const IO_*>(dy), static_cast<const IO_*>(dsum), static_cast<IO_*>(dx), part, \
-                       rows, (int)d, eps)
-    if (io_dtype == MPA_F32) {
-        if (nv <= 1) MPA_NORM_CASE(float, 1);
-        else if (nv <= 2) MPA_NORM_CASE(float, 2);
-        else if (nv <= 4) MPA_NORM_CASE(float, 4);
-        else MPA_NORM_CASE(float, 8);
-    } else {
-        if (nv <= 1) MPA_NORM_CASE(bf16_t, 1);
-        else if (nv <= 2) MPA_NORM_CASE(bf16_t, 2);
-        else if (nv <= 4) MPA_NORM_CASE(bf16_t, 4);
-        else MPA_NORM_CASE(bf16_t, 8);
-    }
-#undef MPA_NORM_CASE
-    rc = check_launch();
+    const int maxv = norm_maxv(d, io_dtype);
+    rc = MPA_NORM_DISPATCH(launch_norm_bwd, x, weight, dy, dsum, dx, part, rows, (int)d, eps, st);
     if (rc != MPA_OK || !weight) return rc;
-    // rows of the partial buffer beyond the last wave of a partially filled block were written
-    // by waves that own no row (all zeros), so every one of the grid's waves counts
-    hipLaunchKernelGGL(rmsnorm_bwd_finish_kernel, dim3((unsigned)((d + kNormFinCols - 1) / kNormFinCols)), dim3(1024), 0, st, part, dweight,
-                       (int)d, (int64_t)grid.x * 4);
+    hipLaunchKernelGGL(rmsnorm_bwd_finish_kernel, dim3((unsigned)((d + kNormFinCols - 1) / kNormFinCols)),
+                       dim3(1024), 0, st, part, dweight, (int)d, norm_bwd_plan(rows).blocks);
     return check_launch();
 }
