@@ -24,7 +24,7 @@
 
 namespace mpa {
 
-constexpr int kConvSpan = 64;   // steps per lane
+constexpr int kConvSpan = 64;   // steps per lane (doubled when the problem still fills the chip, see conv_span)
 constexpr int kConvGroup = 16;  // steps loaded together
 constexpr int kConvMaxK = 4;
 
@@ -38,7 +38,7 @@ struct ConvParams {
     const void* dy;
     void* dx;
     float* part;         // [B][nspan][K+1][ED]
-    int batch, L, ED, K, nspan;
+    int batch, L, ED, K, nspan, span;
     int silu;
     int64_t x_sb, x_sl, x_sd;
     int64_t y_sb, y_sl, y_sd;
@@ -58,7 +58,7 @@ __global__ void __launch_bounds__(256) conv1d_fwd_kernel(const ConvParams p) {
     const int d = blockIdx.x * blockDim.x + threadIdx.x;
     if (d >= p.ED) return;
     const int b = blockIdx.z;
-    const int t0 = blockIdx.y * kConvSpan;
+    const int t0 = blockIdx.y * p.span;
     const int K = p.K;
     const IO* xrow = static_cast<const IO*>(p.x) + b * p.x_sb + (int64_t)d * p.x_sd;
     const IO* wrow = p.win ? static_cast<const IO*>(p.win) + ((int64_t)b * p.ED + d) * (K - 1) : nullptr;
@@ -75,7 +75,7 @@ __global__ void __launch_bounds__(256) conv1d_fwd_kernel(const ConvParams p) {
     float h2 = conv_input<IO>(p, xrow, wrow, t0 - 2);
     float h3 = conv_input<IO>(p, xrow, wrow, t0 - 3);
 
-    const int tend = min(t0 + kConvSpan, p.L);
+    const int tend = min(t0 + p.span, p.L);
     IO cur[kConvGroup], nxt[kConvGroup];
     auto load_group = [&](int tg, IO (&dst)[kConvGroup]) {
         // steps beyond the sequence are clamped (valid memory); their results are not stored
@@ -113,7 +113,7 @@ __global__ void __launch_bounds__(256) conv1d_bwd_kernel(const ConvParams p) {
     const int d = blockIdx.x * blockDim.x + threadIdx.x;
     if (d >= p.ED) return;
     const int b = blockIdx.z;
-    const int t0 = blockIdx.y * kConvSpan;
+    const int t0 = blockIdx.y * p.span;
     const int K = p.K;
     const IO* xrow = static_cast<const IO*>(p.x) + b * p.x_sb + (int64_t)d * p.x_sd;
     const IO* wrow = p.win ? static_cast<const IO*>(p.win) + ((int64_t)b * p.ED + d) * (K - 1) : nullptr;
@@ -134,7 +134,7 @@ __global__ void __launch_bounds__(256) conv1d_bwd_kernel(const ConvParams p) {
     float g1 = 0.0f, g2 = 0.0f, g3 = 0.0f;
     float dw[kConvMaxK] = {0.0f, 0.0f, 0.0f, 0.0f}, db = 0.0f;
 
-    const int tend = min(t0 + kConvSpan, p.L);        // dweight / dbias / dx cover [t0, tend)
+    const int tend = min(t0 + p.span, p.L);           // dweight / dbias / dx cover [t0, tend)
     const int twalk = min(tend + kConvMaxK - 1, p.L + kConvMaxK - 1);
     IO cx[kConvGroup], cy[kConvGroup], nx[kConvGroup], ny[kConvGroup];
     auto load_group = [&](int tg, IO (&dx_)[kConvGroup], IO (&dy_)[kConvGroup]) {
@@ -231,10 +231,18 @@ static int conv_validate(const mpa_conv_shape* s) {
     return MPA_OK;
 }
 
+// Steps per lane: longer spans mean fewer halo reads and fewer dweight partials, shorter spans
+// more waves; 128 steps when that still leaves 16 waves per CU.
+static int conv_span(const mpa_conv_shape* s) {
+    const int64_t waves128 = s->batch * ((s->seqlen + 2 * kConvSpan - 1) / (2 * kConvSpan)) * ((s->dim + kWave - 1) / kWave);
+    return waves128 >= 4096 ? 2 * kConvSpan : kConvSpan;
+}
+
 static ConvParams conv_params(const mpa_conv_shape* s) {
     ConvParams p{};
     p.batch = (int)s->batch; p.L = (int)s->seqlen; p.ED = (int)s->dim; p.K = s->kernel;
-    p.nspan = (p.L + kConvSpan - 1) / kConvSpan;
+    p.span = conv_span(s);
+    p.nspan = (p.L + p.span - 1) / p.span;
     p.silu = (s->flags & MPA_CONV_SILU) ? 1 : 0;
     p.x_sb = s->x_sb; p.x_sl = s->x_sl; p.x_sd = s->x_sd;
     p.y_sb = s->y_sb; p.y_sl = s->y_sl; p.y_sd = s->y_sd;
@@ -272,7 +280,8 @@ extern "C" int mpa_conv1d_fwd(const mpa_conv_shape* s, const void* x, const floa
 
 extern "C" size_t mpa_conv1d_bwd_workspace_bytes(const mpa_conv_shape* s) {
     if (conv_validate(s) != MPA_OK) return 0;
-    const size_t nspan = (size_t)(s->seqlen + kConvSpan - 1) / kConvSpan;
+    const size_t span = (size_t)conv_span(s);
+    const size_t nspan = ((size_t)s->seqlen + span - 1) / span;
     return ((size_t)s->batch * nspan * (kConvMaxK + 1) * s->dim * sizeof(float) + 255) / 256 * 256;
 }
 
