@@ -301,6 +301,27 @@ def test_chunk_split_consistency_with_carried_state(pkg, dev):
     assert rel_err(h2, h_full) <= 1e-6
 
 
+def test_long_sequence_fp32_and_segmented_inference(pkg, dev, monkeypatch):
+    # 50 000 steps, far beyond the benchmark shapes (the reference materialises (B, L, ED, N)
+    # tensors and pads L to a power of two, pscan.py:165-174): forward + backward
+    # against the float64 C oracle, then the same forward without gradients, which the library
+    # cuts into parallel segments by itself (one batch row, two channel groups)
+    monkeypatch.delenv("MPA_FWD_NSEG", raising=False)
+    inp = so.make_inputs(1, 50000, 96, 16, seed=4242)
+    ref = c_oracle.sscan_fwd_bwd(**inp)
+    got = run_gpu_fwd_bwd(pkg, inp, dev)
+    _check(got, ref, TOL[torch.float32], "L=50000")
+    with torch.no_grad():
+        y = pkg.selective_scan_fn(*[inp[k].to(dev) for k in ("x", "delta", "A", "B", "C", "D")])
+    assert rel_err(y, ref["y"]) <= TOL[torch.float32]
+    # zero-length and zero-batch inputs are rejected, not undefined
+    for shape in ((1, 0, 8), (0, 4, 8)):
+        x = torch.zeros(*shape, device=dev)
+        bc = torch.zeros(shape[0], shape[1], 16, device=dev)
+        with pytest.raises(RuntimeError):
+            pkg.selective_scan(x, x, inp["A"][:8].to(dev), bc, bc, inp["D"][:8].to(dev))
+
+
 def test_config1_full_size_fp32(pkg, dev):
     # configs[1]: B=8, L=2048, ED=1536, N=16 float32, against the float64 C oracle
     inp = so.make_inputs(8, 2048, 1536, 16, seed=1001)
