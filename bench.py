@@ -49,7 +49,7 @@ def cpu_baseline(workload, torch, so):
     forward + backward, float32, all host threads) on a slice of the workload's channels:
     channels are independent, so the slice is the same work per channel."""
     B, L, ED, N, _, seed, _ = WORKLOADS[workload]
-    ed = min(ED, 128 if workload != "c0" else ED)
+    ed = min(ED, 512 if workload != "c0" else ED)
     bs = min(B, 2)
     threads = int(os.environ.get("OMP_NUM_THREADS") or os.cpu_count() or 1)
     torch.set_num_threads(threads)
@@ -64,7 +64,7 @@ def cpu_baseline(workload, torch, so):
 
     once()
     reps, t0 = 0, time.perf_counter()
-    while reps < 3 or (time.perf_counter() - t0 < 6.0 and reps < 20):
+    while reps < 3 or (time.perf_counter() - t0 < 12.0 and reps < 60):  # about 12 s of CPU work
         once()
         reps += 1
     dt = (time.perf_counter() - t0) / reps
