@@ -116,6 +116,21 @@ def test_reference_test_distribution_randn_A_and_delta(pkg, dev):
     _check(got, ref, TOL[torch.float32], "randn A/delta")
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_sum_backward_convention_of_the_reference_tests(pkg, dev, dtype):
+    # tests/compare_mambapy_cuda.py:49-53 of the reference backpropagates y.sum(): the upstream
+    # gradient is an expanded (stride-0) tensor of ones
+    inp = so.make_inputs(2, 300, 192, 16, seed=77, dtype=dtype)
+    inp["dy"] = torch.ones_like(inp["x"])
+    ref = c_oracle.sscan_fwd_bwd(**inp)
+    names = ("x", "delta", "A", "B", "C", "D")
+    args = [inp[k].to(dev).requires_grad_() for k in names]
+    y = pkg.selective_scan(*args)
+    y.sum().backward()
+    got = dict(y=y.detach(), **{k: a.grad for k, a in zip(GRAD_KEYS, args)})
+    _check(got, ref, TOL[dtype], "y.sum().backward()")
+
+
 def test_gate_softplus_bias_h0_and_last_state(pkg, dev):
     Bs, L, ED, N = 2, 90, 80, 16
     inp = so.make_inputs(Bs, L, ED, N, seed=51)
