@@ -119,14 +119,6 @@ __device__ __forceinline__ int wave_id() {
 
 typedef float f16v __attribute__((ext_vector_type(16)));
 
-// B/C reach the scan waves in sub-tiles of kSS steps; two sub-tiles (the one in use and the
-// one in flight) must fit the scalar register file, so a sub-tile holds 32 floats (64 at 32
-// states per lane).
-template <int NS>
-struct BcPack {
-    static constexpr int kSS = NS >= 16 ? 1 : 16 / NS;
-};
-
 // COUNT consecutive floats through the scalar cache into SGPRs (the address is wave-uniform)
 template <int COUNT>
 __device__ __forceinline__ void scalar_load(const float* src, float (&dst)[COUNT]) {

@@ -21,6 +21,11 @@
 //    (fmac_bcast), so B and C cost no extra instructions and no scalar registers.  Above that
 //    a small pre-pass packs them as float32 in the order each scan wave consumes them and the
 //    scan waves fetch them with scalar loads into SGPRs.
+//  * The only parallel axes are batch * dim/64 workgroups and the states inside them.  When a
+//    launch without checkpoints (inference) would cover a fraction of the chip, the sequence is
+//    cut into segments that run side by side: a first pass finds every segment's end state from
+//    zero and its sum of delta, seg_carry_kernel chains them, a second pass is the normal
+//    kernel from the true initial states (see seg_plan).
 //  * Both channel-contiguous and time-contiguous ((B,ED,L) memory) operands are read and
 //    written coalesced: a service thread owns 4 consecutive steps of one channel, and the
 //    thread -> (channel, step group) map follows the unit-stride axis.
