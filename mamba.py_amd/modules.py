@@ -63,6 +63,32 @@ class MambaConfig:
             self.mup_width_mult = self.d_model / self.mup_base_width
 
 
+def _frozen_f32(owner, key, p, fn=None):
+    """float32 form of a small parameter (optionally fn(parameter)) for the kernels that take
+    float32 constants.  Inside autograd the parameter itself is returned and the conversion is
+    part of the graph.  Outside it (decode, prefill) the converted value is kept in one
+    persistent buffer per (module, key) that is refreshed in place when the parameter has
+    changed: a forward pass then spends no kernels on these conversions and a captured HIP graph
+    keeps reading the same memory."""
+    if p is None:
+        return None
+    if torch.is_grad_enabled() and p.requires_grad:
+        return p if fn is None else fn(p)
+    if fn is None and p.dtype == torch.float32:
+        return p
+    cache = owner.__dict__.setdefault("_f32_cache", {})
+    tag = (p._version, p.data_ptr(), p.device)
+    hit = cache.get(key)
+    if hit is None or hit[0] != tag:
+        with torch.no_grad():
+            fresh = p.detach().float() if fn is None else fn(p.detach())
+            if hit is not None and hit[1].shape == fresh.shape and hit[1].device == fresh.device:
+                hit[1].copy_(fresh)
+                fresh = hit[1]
+        cache[key] = (tag, fresh)
+    return cache[key][1]
+
+
 class RMSNorm(nn.Module):
     """x * rsqrt(mean(x^2) + eps) [* weight]  (mambapy/mamba.py:416-433; no gain under muP)."""
 
@@ -73,9 +99,12 @@ class RMSNorm(nn.Module):
         if not use_mup:
             self.weight = nn.Parameter(torch.ones(d_model))
 
+    def _w(self):
+        return None if self.use_mup else _frozen_f32(self, "weight", self.weight)
+
     def forward(self, x):
         if x.is_cuda and rmsnorm_supported(x):
-            return rmsnorm_fn(x, None if self.use_mup else self.weight, self.eps)
+            return rmsnorm_fn(x, self._w(), self.eps)
         y = x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + self.eps)
         return y if self.use_mup else y * self.weight
 
@@ -84,7 +113,7 @@ class RMSNorm(nn.Module):
         if residual is None:
             return self(x), x
         if x.is_cuda and rmsnorm_supported(x) and residual.dtype == x.dtype:
-            return add_rmsnorm_fn(x, residual, None if self.use_mup else self.weight, self.eps)
+            return add_rmsnorm_fn(x, residual, self._w(), self.eps)
         total = x + residual
         return self(total), total
 
@@ -142,23 +171,17 @@ class MambaBlock(nn.Module):
         return dlow, Bm, C
 
     def _A(self):
-        """A = -exp(A_log) (mambapy/mamba.py:239).  Without autograd (decode, prefill) the value
-        is kept in one persistent buffer that is refreshed in place when A_log has changed, so
-        a token step does not spend two kernels per layer on it and a captured HIP graph keeps
-        reading the same memory."""
-        if torch.is_grad_enabled() and self.A_log.requires_grad:
-            return -torch.exp(self.A_log.float())
-        key = (self.A_log._version, self.A_log.data_ptr(), self.A_log.device)
-        if getattr(self, "_A_key", None) != key:
-            with torch.no_grad():
-                fresh = -torch.exp(self.A_log.detach().float())
-                buf = getattr(self, "_A_buf", None)
-                if buf is None or buf.shape != fresh.shape or buf.device != fresh.device:
-                    self._A_buf = fresh
-                else:
-                    buf.copy_(fresh)
-            self._A_key = key
-        return self._A_buf
+        """A = -exp(A_log) in float32 (mambapy/mamba.py:239)."""
+        return _frozen_f32(self, "A", self.A_log, lambda t: -torch.exp(t.float()))
+
+    def _D(self):
+        return _frozen_f32(self, "D", self.D)
+
+    def _dt_bias(self):
+        return _frozen_f32(self, "dt_bias", self.dt_proj.bias)
+
+    def _conv_wb(self):
+        return (_frozen_f32(self, "conv_w", self.conv1d.weight), _frozen_f32(self, "conv_b", self.conv1d.bias))
 
     # -- training / prefill ---------------------------------------------------------------
     def forward(self, x, cache: Optional[Tuple] = None, return_cache: bool = False):
@@ -173,10 +196,11 @@ class MambaBlock(nn.Module):
         if 2 <= K <= 4:
             # causal depthwise convolution + bias + silu in one kernel, reading the x half of
             # the projection in place (no transposes) and returning the decode window
+            cw, cb = self._conv_wb()
             if return_cache:
-                xs, window = causal_conv1d_fn(xin, self.conv1d.weight, self.conv1d.bias, return_window=True)
+                xs, window = causal_conv1d_fn(xin, cw, cb, return_window=True)
             else:
-                xs = causal_conv1d_fn(xin, self.conv1d.weight, self.conv1d.bias)
+                xs = causal_conv1d_fn(xin, cw, cb)
         else:
             xc = self.conv1d(xin.transpose(1, 2))[:, :, :L]
             xs = F.silu(xc).transpose(1, 2)                  # (B, L, ED), unit stride along L
@@ -200,13 +224,13 @@ class MambaBlock(nn.Module):
         """(B, L, ED) -> (B, L, ED): projections to (delta, B, C), then the fused scan
         (mambapy/mamba.py:236-272); with z the result is already gated, y * silu(z), as on the
         reference's fused path (mamba.py:259-260, 225-227)."""
-        A, D = self._A(), self.D.float()
+        A, D = self._A(), self._D()
         dlow, Bm, C = self._split_projection(self.x_proj(x))
         # (B, L, ED) with unit stride along ED, the layout of x: the reference forms the transposed
         # product (mamba.py:247) only because its fused backend wants (B, ED, L)
         delta = F.linear(dlow, self.dt_proj.weight)
         if self.config.fused_softplus:
-            return selective_scan_fn(x, delta, A, Bm, C, D, z=z, delta_bias=self.dt_proj.bias,
+            return selective_scan_fn(x, delta, A, Bm, C, D, z=z, delta_bias=self._dt_bias(),
                                      delta_softplus=True, return_last_state=return_last_state)
         delta = F.softplus(delta + self.dt_proj.bias)
         return selective_scan_fn(x, delta, A, Bm, C, D, z=z, return_last_state=return_last_state)
@@ -229,8 +253,7 @@ class MambaBlock(nn.Module):
         xin, z = xz.chunk(2, dim=1)
         if 2 <= self.config.d_conv <= 4 and not torch.is_grad_enabled():
             # convolution over (cache, newest input) + bias + silu and the new cache: one kernel
-            xs, window = causal_conv1d_fn(xin.unsqueeze(1), self.conv1d.weight, self.conv1d.bias,
-                                          window=inputs, return_window=True)
+            xs, window = causal_conv1d_fn(xin.unsqueeze(1), *self._conv_wb(), window=inputs, return_window=True)
             xs = xs[:, 0]
         else:
             full = torch.cat([inputs, xin.unsqueeze(2)], dim=2)          # (B, ED, d_conv)
@@ -247,8 +270,8 @@ class MambaBlock(nn.Module):
         the gate y*silu(z) is applied inside the kernel; inplace=True updates h itself."""
         dlow, Bm, C = self._split_projection(self.x_proj(x))
         raw = F.linear(dlow, self.dt_proj.weight)                        # bias added in-kernel
-        y, h_new = ssm_step(x, raw, self._A(), Bm, C, self.D.float(), h, z=z,
-                            delta_bias=self.dt_proj.bias, delta_softplus=True, inplace=inplace)
+        y, h_new = ssm_step(x, raw, self._A(), Bm, C, self._D(), h, z=z,
+                            delta_bias=self._dt_bias(), delta_softplus=True, inplace=inplace)
         return y, h_new
 
     def step_(self, x, h, window):
@@ -258,7 +281,7 @@ class MambaBlock(nn.Module):
         xz = self.in_proj(x)
         xin, z = xz.chunk(2, dim=1)
         if 2 <= self.config.d_conv <= 4 and window.is_contiguous() and window.dtype == xin.dtype:
-            xs = causal_conv1d_update(xin, window, self.conv1d.weight, self.conv1d.bias)
+            xs = causal_conv1d_update(xin, window, *self._conv_wb())
         else:
             full = torch.cat([window, xin.unsqueeze(2)], dim=2)          # (B, ED, d_conv)
             xc = (full * self.conv1d.weight[:, 0, :]).sum(-1)
