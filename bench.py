@@ -283,6 +283,66 @@ def bench_layer_kernels(args, torch, pkg, dev):
     print(json.dumps(out))
 
 
+def bench_generate(args, torch, pkg, dev):
+    """Generation with the mamba-130m architecture (random-init, bf16): one prefill of a 512-token
+    prompt, then 128 greedy tokens, (a) with LM.step per token, (b) with the step replayed as a
+    HIP graph, and, for scale, (c) the reference's way of generating (mambapy/lm.py:119-155: the
+    whole sequence goes through forward again for every new token), timed on 8 tokens."""
+    vocab, Lp, new = 50280, 512, 128
+    cfg = pkg.MambaConfig(d_model=768, n_layers=24, d_state=16)
+    torch.manual_seed(1007)
+    model = pkg.LM(cfg, vocab, pad_vocab_size_multiple=8).to(dev).to(torch.bfloat16).eval()
+    rows = {}
+    for Bsz in (1, 64):
+        prompt = torch.randint(0, vocab, (Bsz, Lp), generator=torch.Generator().manual_seed(1007)).to(dev)
+
+        def eager():
+            return model.generate(prompt, new)
+
+        def graphed():
+            logits, caches = model.prefill(prompt)
+            dec = graphed.dec
+            for (h, w), (h0, w0) in zip(dec.caches, caches):
+                h.copy_(h0)
+                w.copy_(w0)
+            out = []
+            for _ in range(new):
+                nxt = logits.argmax(-1)
+                out.append(nxt)
+                logits = dec(nxt)
+            return out
+
+        def rerun():
+            seq = prompt
+            for _ in range(8):
+                logits = model(seq)[:, -1]
+                seq = torch.cat([seq, logits.argmax(-1, keepdim=True)], 1)
+            return seq
+
+        with torch.no_grad():
+            _, caches = model.prefill(prompt)
+            graphed.dec = pkg.GraphedDecoder(model, caches)
+            t_pre = _timed(torch, lambda: model.prefill(prompt), 5, 2)
+            t_eager = _timed(torch, eager, 2, 1)
+            t_graph = _timed(torch, graphed, 3, 1)
+            t_rerun = _timed(torch, rerun, 2, 1) / 8
+        rows[Bsz] = {"prefill_ms": t_pre * 1e3,
+                     "eager_step_tokens_per_s": Bsz * new / (t_eager - t_pre),
+                     "graphed_step_tokens_per_s": Bsz * new / (t_graph - t_pre),
+                     "ms_per_token_step_graphed": (t_graph - t_pre) / new * 1e3,
+                     "rerun_forward_tokens_per_s": Bsz / t_rerun}
+    out = {
+        "metric": "generated tokens/s, mamba-130m architecture, 512-token prompt + 128 new tokens, batch 64",
+        "value": rows[64]["graphed_step_tokens_per_s"], "unit": "tokens/s", "higher_is_better": True,
+        "n_gpus": 1, "steps": 3, "warmup": 1, "ms_per_step": rows[64]["ms_per_token_step_graphed"],
+        "scaling": "weak", "vs_baseline": None, "dtype": "bf16 weights/activations, f32 scan state",
+        "data": "synthetic (random-init weights, uniform-random prompt)",
+        "config": {"workload": "prefill once + one state-update step per token (HIP graph); batch 1 and 64"},
+        "batch_1": rows[1], "batch_64": rows[64],
+    }
+    print(json.dumps(out))
+
+
 def bench_lm_forward(args, torch, pkg, dev, L):
     """configs[4]: random-init LM forward at the mamba-130m architecture, bf16 weights and
     activations, fp32 scan state, B=8, uniform-random token ids."""
@@ -317,7 +377,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS) + ["c3", "c4", "c4-3000", "pscan", "layer"],
+    ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS) + ["c3", "c4", "c4-3000", "pscan", "layer", "generate"],
                     help="c2 (default) is the headline workload; c3 = decode step, c4 = LM forward "
                          "(reported with their own metric, same one-line schema)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -343,6 +403,8 @@ def main():
         return bench_pscan(args, torch, pkg, dev)
     if args.workload == "layer":
         return bench_layer_kernels(args, torch, pkg, dev)
+    if args.workload == "generate":
+        return bench_generate(args, torch, pkg, dev)
     if args.workload.startswith("c4"):
         return bench_lm_forward(args, torch, pkg, dev, 3000 if args.workload == "c4-3000" else 4096)
 
