@@ -586,7 +586,10 @@ __global__ void __launch_bounds__(256) seg_carry_kernel(const float* __restrict_
         segh0[row * per_b + dn] = h;
         const float* ds = dsum + row * (kTile / 4) * ED + d;
         const float sd = (ds[0] + ds[ED]) + (ds[2 * (int64_t)ED] + ds[3 * (int64_t)ED]);
-        h = __builtin_fmaf(fast_exp2(a2 * sd), h, hend[row * per_b + dn]);
+        // (a zero state stays out of the product: with A > 0 the factor can overflow, and 0 * inf
+        // is not what the step-by-step recurrence computes)
+        const float e = hend[row * per_b + dn];
+        h = h == 0.0f ? e : __builtin_fmaf(fast_exp2(a2 * sd), h, e);
     }
     if (hlast) hlast[i] = h;
 }

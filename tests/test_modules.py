@@ -14,9 +14,13 @@ def test_config_derived_values(pkg):
 def test_parameter_count_known_answer(pkg):
     # examples/example_e2e_training.ipynb cell 5 of the reference: d_model=16, n_layers=4,
     # vocab 9 with a TIED head has 13 664 parameters; this LM keeps the head untied (lm.py:41)
-    m = pkg.LM(pkg.MambaConfig(d_model=16, n_layers=4), 9)
+    import json
+    import os
+    with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "reference_vectors.json")) as f:
+        g = json.load(f)["param_count"]
+    m = pkg.LM(pkg.MambaConfig(d_model=g["d_model"], n_layers=g["n_layers"]), g["vocab_size"])
     n = sum(p.numel() for p in m.parameters())
-    assert n - m.lm_head.weight.numel() == 13664
+    assert g["parameters"] == 13664 and n - m.lm_head.weight.numel() == g["parameters"]
 
 
 def test_state_dict_keys_match_reference_layout(pkg):

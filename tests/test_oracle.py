@@ -1,7 +1,9 @@
 """Pins the CPU oracle (oracle/) against the reference's own known-answer vectors and
 against what the mathematics fixes, so that a plausible mistake in the oracle (a dropped
 term, a wrong sign or index, a transposed operand) fails here.  Runs without a GPU."""
+import json
 import math
+import os
 
 import pytest
 import torch
@@ -9,6 +11,10 @@ import torch
 from oracle import c_oracle, scan_oracle as so
 
 torch.set_default_dtype(torch.float32)
+
+
+with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "reference_vectors.json")) as _f:
+    GOLDEN = json.load(_f)
 
 
 def _as4d(v):
@@ -19,26 +25,27 @@ def _as4d(v):
 
 def test_reference_cumsum_vector_1234():
     # docs/pscan.ipynb cells 5, 8, 11: cumsum([1,2,3,4]) = [1,3,6,10]  (A == 1)
-    X = _as4d([1, 2, 3, 4])
+    X = _as4d(GOLDEN["cumsum_1234"]["X"])
     A = torch.ones_like(X)
-    want = [1, 3, 6, 10]
+    want = GOLDEN["cumsum_1234"]["H"]
+    assert want == [1, 3, 6, 10]
     assert so.linear_recurrence(A, X).flatten().tolist() == want
     assert so.pscan_blelloch(A, X).flatten().tolist() == want
 
 
 def test_reference_upsweep_vector():
     # docs/pscan.ipynb cell 43: up-sweep only of [1..8] leaves [1,3,3,10,5,11,7,36]
-    X = _as4d([1, 2, 3, 4, 5, 6, 7, 8])
+    X = _as4d(GOLDEN["upsweep_1_to_8"]["X"])
     A = torch.ones_like(X)
     so.blelloch_upsweep_(A, X)
-    assert X.flatten().tolist() == [1, 3, 3, 10, 5, 11, 7, 36]
+    assert X.flatten().tolist() == GOLDEN["upsweep_1_to_8"]["X_after_upsweep"]
 
 
 def test_reference_padded_scan_vector():
     # docs/tests.ipynb cell 1: inclusive scan with a zero-padded tail
-    X = _as4d([5, 1, 2, 3, 4, 5, 6, 7, 8, 0, 0, 0, 0, 0, 0, 0])
+    X = _as4d(GOLDEN["padded_scan"]["X"])
     A = torch.ones_like(X)
-    want = [5, 6, 8, 11, 15, 20, 26, 33, 41] + [41] * 7
+    want = GOLDEN["padded_scan"]["H"]
     H = X.clone()
     so.blelloch_scan_(A.clone(), H)
     assert H.flatten().tolist() == want
@@ -47,7 +54,7 @@ def test_reference_padded_scan_vector():
 
 def test_next_pow2_matches_reference_table():
     # mambapy/pscan.py:13-18 : 64->64, 3000->4096, 4097->8192, 1->1
-    assert [so.next_pow2(v) for v in (1, 2, 3, 64, 3000, 4096, 4097)] == [1, 2, 4, 64, 4096, 4096, 8192]
+    assert [so.next_pow2(v) for v in GOLDEN["next_pow2"]["in"]] == GOLDEN["next_pow2"]["out"]
 
 
 # ---- closed forms and brute force -----------------------------------------------------

@@ -29,10 +29,13 @@ def test_pscan_forward_backward_fp32(pkg, dev, Bs, L, D, N):
 
 def test_pscan_reference_golden_vectors(pkg, dev):
     # docs/pscan.ipynb cells 5/8/11 and docs/tests.ipynb cell 1 (A == 1: cumulative sums)
-    X = torch.tensor([1., 2., 3., 4.], device=dev).reshape(1, 4, 1, 1)
-    assert pkg.pscan(torch.ones_like(X), X).flatten().tolist() == [1, 3, 6, 10]
-    X = torch.tensor([5., 1, 2, 3, 4, 5, 6, 7, 8, 0, 0, 0, 0, 0, 0, 0], device=dev).reshape(1, 16, 1, 1)
-    assert pkg.pscan(torch.ones_like(X), X).flatten().tolist() == [5, 6, 8, 11, 15, 20, 26, 33, 41] + [41] * 7
+    import json
+    import os
+    with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "reference_vectors.json")) as f:
+        golden = json.load(f)
+    for key in ("cumsum_1234", "padded_scan"):
+        X = torch.tensor(golden[key]["X"], dtype=torch.float32, device=dev).reshape(1, -1, 1, 1)
+        assert pkg.pscan(torch.ones_like(X), X).flatten().tolist() == golden[key]["H"]
 
 
 def test_pscan_inputs_untouched_and_strided_views(pkg, dev):
