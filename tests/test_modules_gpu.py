@@ -116,6 +116,27 @@ def test_lm_forward_generate_and_bf16(pkg, dev):
         assert l16.dtype == torch.bfloat16 and rel_err(l16, logits) <= 5e-2
 
 
+def test_lm_full_size_causality_and_prefill_handoff_bf16(pkg, dev):
+    # configs[4] at full size (24 layers, d_model 768, vocab 50280, B=8, bf16): properties that
+    # do not need an oracle of that size.  (1) Causality: the logits of the first 3000 positions
+    # do not depend on what follows, and L=3000 (ragged tiles, no power-of-two padding) must
+    # give what the first 3000 positions of L=4096 give.  (2) Prefill of 4095 tokens + one
+    # decode step reproduces position 4095 of the parallel forward.
+    torch.manual_seed(1004)
+    cfg = pkg.MambaConfig(d_model=768, n_layers=24, d_state=16)
+    model = pkg.LM(cfg, 50280, pad_vocab_size_multiple=8).to(dev).to(torch.bfloat16).eval()
+    ids = torch.randint(0, 50280, (8, 4096), generator=torch.Generator().manual_seed(1004)).to(dev)
+    with torch.no_grad():
+        full = model(ids)
+        part = model(ids[:, :3000])
+        assert rel_err(part, full[:, :3000].double()) <= 2e-2
+        del part
+        last, caches = model.prefill(ids[:, :4095])
+        assert rel_err(last, full[:, 4094].double()) <= 2e-2
+        nxt, _ = model.step(ids[:, 4095], caches)
+        assert rel_err(nxt, full[:, 4095].double()) <= 2e-2
+
+
 def test_softplus_path_without_gate_full_gradients(pkg, dev):
     # delta = softplus(raw + bias) inside the kernel, no gate: the fast backward path
     Bs, L, ED, N = 2, 150, 128, 16
