@@ -121,3 +121,25 @@ def test_step_config3_shape(pkg, dev):
     y, hn = pkg.ssm_step(x.to(dev), dl.to(dev), inp["A"].to(dev), Bm.to(dev), C.to(dev),
                          inp["D"].to(dev), h.to(dev))
     assert rel_err(y, yr) <= TOL[torch.float32] and rel_err(hn, hr) <= TOL[torch.float32]
+
+
+def test_config3_256_steps_equal_one_scan_with_carried_state(pkg, dev):
+    # configs[3] at full size: 256 in-place decode steps from a random state (batch 64, ED=5120,
+    # N=16) must give what one scan over the same 256 positions with that initial state gives
+    # (mambapy/mamba.py:344-346), outputs and final state
+    Bs, T, ED, N = 64, 256, 5120, 16
+    inp = so.make_inputs(Bs, T, ED, N, seed=1003)
+    g = torch.Generator().manual_seed(8)
+    h0 = torch.randn(Bs, ED, N, generator=g)
+    d = {k: v.to(dev) for k, v in inp.items()}
+    with torch.no_grad():
+        y_scan, h_scan = pkg.selective_scan_fn(d["x"], d["delta"], d["A"], d["B"], d["C"], d["D"],
+                                               h0=h0.to(dev), return_last_state=True)
+        h = h0.to(dev).clone()
+        ys = []
+        for t in range(T):
+            y, _ = pkg.ssm_step(d["x"][:, t], d["delta"][:, t], d["A"], d["B"][:, t], d["C"][:, t], d["D"], h,
+                                inplace=True)
+            ys.append(y)
+    assert rel_err(torch.stack(ys, 1), y_scan.double()) <= TOL[torch.float32]
+    assert rel_err(h, h_scan.double()) <= TOL[torch.float32]
