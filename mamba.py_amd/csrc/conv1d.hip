@@ -20,6 +20,8 @@
 //     dpre = dy * silu'(pre), dx[t] = sum_k w[k] * dpre[t + K-1-k], and keeps per-lane sums of
 //     dweight / dbias over its span; spans and batch rows are then summed by a second kernel
 //     in a fixed order (no floating-point atomics).
+#include <type_traits>
+
 #include "common.h"
 
 namespace mpa {
@@ -145,13 +147,14 @@ __global__ void __launch_bounds__(256) conv1d_bwd_kernel(const ConvParams p) {
             dy_[j] = dyrow[(int64_t)tc * p.y_sl];
         }
     };
-    load_group(t0, cx, cy);
-    for (int tg = t0; tg < twalk; tg += kConvGroup) {
-        if (tg + kConvGroup < twalk) load_group(tg + kConvGroup, nx, ny);
+    // one group of kConvGroup steps; EDGE = the group touches the start or the end of the span or of
+    // the sequence (the others need no predicate: every step is live, counted and stored)
+    auto walk_group = [&](auto edge_c, int tg) {
+        constexpr bool EDGE = decltype(edge_c)::value;
 #pragma unroll
         for (int j = 0; j < kConvGroup; ++j) {
             const int t = tg + j;
-            const bool live = t < p.L;  // steps past the sequence contribute dpre = 0
+            const bool live = !EDGE || t < p.L;  // steps past the sequence contribute dpre = 0
             const float xv = live ? to_float(cx[j]) : 0.0f;
             float pre = __builtin_fmaf(wk[3], xv, bv);
             pre = __builtin_fmaf(wk[2], h1, pre);
@@ -162,7 +165,7 @@ __global__ void __launch_bounds__(256) conv1d_bwd_kernel(const ConvParams p) {
                 const float s = sigmoid_f(pre);
                 g *= s * __builtin_fmaf(pre, 1.0f - s, 1.0f);
             }
-            if (t < tend) {
+            if (!EDGE || t < tend) {
                 dw[3] = __builtin_fmaf(g, xv, dw[3]);
                 dw[2] = __builtin_fmaf(g, h1, dw[2]);
                 dw[1] = __builtin_fmaf(g, h2, dw[1]);
@@ -172,7 +175,7 @@ __global__ void __launch_bounds__(256) conv1d_bwd_kernel(const ConvParams p) {
             // dx[t-3] = w[K-1]*dpre[t-3] + w[K-2]*dpre[t-2] + w[K-3]*dpre[t-1] + w[K-4]*dpre[t]
             const float dxv = __builtin_fmaf(wk[3], g3, __builtin_fmaf(wk[2], g2, __builtin_fmaf(wk[1], g1, wk[0] * g)));
             const int tx = t - (kConvMaxK - 1);
-            if (tx >= t0 && tx < tend) dxrow[(int64_t)tx * p.g_sl] = from_float<IO>(dxv);
+            if (!EDGE || (tx >= t0 && tx < tend)) dxrow[(int64_t)tx * p.g_sl] = from_float<IO>(dxv);
             g3 = g2;
             g2 = g1;
             g1 = g;
@@ -180,6 +183,14 @@ __global__ void __launch_bounds__(256) conv1d_bwd_kernel(const ConvParams p) {
             h2 = h1;
             h1 = xv;
         }
+    };
+    load_group(t0, cx, cy);
+    for (int tg = t0; tg < twalk; tg += kConvGroup) {
+        if (tg + kConvGroup < twalk) load_group(tg + kConvGroup, nx, ny);
+        if (tg > t0 && tg + kConvGroup <= tend)
+            walk_group(std::false_type{}, tg);
+        else
+            walk_group(std::true_type{}, tg);
 #pragma unroll
         for (int j = 0; j < kConvGroup; ++j) {
             cx[j] = nx[j];
