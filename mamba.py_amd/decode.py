@@ -26,6 +26,10 @@ class GraphedDecoder:
              LM.prefill(...) or Mamba.empty_caches(...); h may be None (zero state).  The
              decoder copies them into its own buffers.
     The returned tensor is the decoder's output buffer: it is overwritten by the next call.
+    Weights are read from the model's own tensors at replay time, except the float32 forms of
+    the small parameters (A, D, biases, conv and norm weights), which live in per-module buffers
+    that an eager forward/step refreshes in place after a weight update; build a new decoder
+    (or run one eager step) after changing those.
     """
 
     def __init__(self, model, caches, warmup: int = 2):
