@@ -363,3 +363,58 @@ def test_errors_are_reported_not_undefined(pkg, dev):
                            g["C"].double(), g["D"])
     with pytest.raises(RuntimeError):
         pkg.selective_scan(inp["x"], inp["delta"], inp["A"], inp["B"], inp["C"], inp["D"])  # CPU
+
+
+@pytest.mark.parametrize("seed", range(40))
+def test_random_shapes_layouts_and_options(pkg, dev, seed):
+    # seeded sweep over ragged shapes, both memory layouts, fp32 / bf16, gate + softplus + bias, initial
+    # state: forward, last state and every gradient against the float64 definition
+    import random
+    rnd = random.Random(1234 + seed)
+    Bs, L = rnd.randint(1, 3), rnd.choice([1, 2, 15, 16, 17, 31, 33, 47, 64, 65, 100, 129, 200])
+    ED = rnd.choice([1, 3, 31, 63, 64, 65, 96, 128, 130, 200])
+    N = rnd.choice([1, 2, 4, 7, 8, 12, 15, 16, 16, 16, 16, 24, 32, 64])
+    dtype = rnd.choice([torch.float32, torch.float32, torch.bfloat16])
+    gated, tmajor, with_h0 = rnd.random() < 0.5, rnd.random() < 0.4, rnd.random() < 0.5
+    inp = so.make_inputs(Bs, L, ED, N, seed=9000 + seed, dtype=dtype)
+    g = torch.Generator().manual_seed(9100 + seed)
+    z = torch.randn(Bs, L, ED, generator=g).to(dtype)
+    raw = (torch.randn(Bs, L, ED, generator=g) * 0.5 - 4.0).to(dtype)
+    bias = torch.randn(ED, generator=g) * 0.3
+    h0 = torch.randn(Bs, ED, N, generator=g) if with_h0 else None
+    f64 = lambda t: t.double().requires_grad_()
+    x, dl, A, Bm, C, D = map(f64, (inp["x"], raw if gated else inp["delta"], inp["A"], inp["B"], inp["C"], inp["D"]))
+    zz, bb = f64(z), f64(bias)
+    delta = so.softplus_ref(dl + bb) if gated else dl
+    yr, hl = so.selective_scan_ref(x, delta, A, Bm, C, D, h0=None if h0 is None else h0.double(),
+                                   return_last_state=True)
+    if gated:
+        yr = yr * (zz * torch.sigmoid(zz))
+    yr.backward(inp["dy"].double())
+    ref = dict(y=yr, hl=hl, dx=x.grad, ddelta=dl.grad, dA=A.grad, dB=Bm.grad, dC=C.grad, dD=D.grad)
+    if gated:
+        ref.update(dz=zz.grad, dbias=bb.grad)
+
+    def lay(t):  # (B, L, ED) values in (B, ED, L) memory, the layout MambaBlock.forward produces
+        t = t.to(dev)
+        return t.transpose(1, 2).contiguous().transpose(1, 2) if tmajor else t
+    gx = lay(inp["x"]).requires_grad_()
+    gd = lay(raw if gated else inp["delta"]).requires_grad_()
+    gz = lay(z).requires_grad_()
+    gA, gB, gC, gD, gb = (t.to(dev).requires_grad_() for t in (inp["A"], inp["B"], inp["C"], inp["D"], bias))
+    kw = dict(z=gz, delta_bias=gb, delta_softplus=True) if gated else {}
+    y, hg = pkg.selective_scan_fn(gx, gd, gA, gB, gC, gD, h0=None if h0 is None else h0.to(dev),
+                                  return_last_state=True, **kw)
+    y.backward(inp["dy"].to(dev))
+    got = dict(y=y, hl=hg, dx=gx.grad, ddelta=gd.grad, dA=gA.grad, dB=gB.grad, dC=gC.grad, dD=gD.grad)
+    if gated:
+        got.update(dz=gz.grad, dbias=gb.grad)
+    tol = TOL[dtype]
+    what = f"B{Bs} L{L} ED{ED} N{N} {dtype} gated={gated} tmajor={tmajor} h0={with_h0}"
+    for k in ref:
+        scale = ref[k].abs().max().item()
+        if scale == 0.0:
+            assert got[k].abs().max().item() == 0.0, f"{what}: {k}"
+            continue
+        e = rel_err(got[k], ref[k])
+        assert e <= (TOL[torch.float32] if k == "hl" and dtype == torch.float32 else tol), f"{what}: {k} rel err {e:.3e}"
