@@ -127,3 +127,20 @@ def test_decode_update_rolls_the_window_in_place(pkg, dev, K, dtype):
         assert rel_err(got, want) <= TOL[dtype]
         assert torch.equal(win_dev.cpu().double(), ref_win)    # the cache holds inputs, bit for bit
         xz = xz.roll(1, 0) * 0.5 + 0.1
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_conv_random_sweep(pkg, dev, seed):
+    # seeded sweep: ragged lengths around the 64/128-step spans, channel counts around the
+    # wave width, every tap count, strided input, decode window, with and without silu / bias
+    import random
+    rnd = random.Random(77 + seed)
+    Bsz = rnd.randint(1, 3)
+    L = rnd.choice([1, 2, 3, 5, 63, 64, 65, 127, 128, 129, 191, 200, 257, 300])
+    ED = rnd.choice([1, 5, 63, 64, 65, 128, 200, 256, 257])
+    K = rnd.choice([2, 3, 4])
+    dtype = rnd.choice([torch.float32, torch.float32, torch.bfloat16])
+    got, ref = _case(pkg, dev, Bsz, L, ED, K, dtype, 5000 + seed, strided=rnd.random() < 0.5,
+                     window=rnd.random() < 0.5, silu=rnd.random() < 0.7, bias=rnd.random() < 0.8)
+    for k in ref:
+        assert rel_err(got[k], ref[k]) <= TOL[dtype], f"B{Bsz} L{L} ED{ED} K{K} {dtype}: {k}"

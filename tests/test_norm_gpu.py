@@ -85,3 +85,45 @@ def test_add_rmsnorm_forward_backward(pkg, dev, shape, dtype, with_w):
     xr2 = (x.double() + r.double()).to(dtype).double().requires_grad_()
     so.rmsnorm_ref(xr2, None if w is None else w.double(), 1e-5).backward(dy.double())
     assert rel_err(xg2.grad, xr2.grad) <= tol and torch.equal(xg2.grad, rg2.grad)
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_rmsnorm_random_sweep(pkg, dev, seed):
+    # seeded sweep over row counts (around the rows-per-wave and waves-per-block boundaries) and
+    # every supported width class (1, 2, 4, 8 vectors per lane), with and without the residual
+    import random
+    rnd = random.Random(300 + seed)
+    dtype = rnd.choice([torch.float32, torch.bfloat16])
+    vec = 4 if dtype == torch.float32 else 8
+    d = vec * rnd.choice([1, 3, 16, 64, 65, 96, 128, 200, 256, 300, 512])
+    rows = rnd.choice([1, 2, 7, 8, 9, 63, 64, 65, 257, 1000, 4097, 9000])
+    with_res, with_w = rnd.random() < 0.5, rnd.random() < 0.8
+    g = torch.Generator().manual_seed(seed)
+    x = (torch.randn(rows, d, generator=g) * 1.3).to(dtype)
+    r = torch.randn(rows, d, generator=g).to(dtype)
+    w = (torch.randn(d, generator=g) * 0.5 + 1.0) if with_w else None
+    dy = torch.randn(rows, d, generator=g).to(dtype)
+    dt = torch.randn(rows, d, generator=g).to(dtype)
+    xr, rr = x.double().requires_grad_(), r.double().requires_grad_()
+    wr = None if w is None else w.double().requires_grad_()
+    tr = xr + rr if with_res else xr
+    tq = tr + (tr.detach().to(dtype).double() - tr.detach()) if with_res else tr
+    yr = so.rmsnorm_ref(tq, wr, 1e-5)
+    loss = (yr * dy.double()).sum() + ((tq * dt.double()).sum() if with_res else 0.0)
+    loss.backward()
+    xg, rg = x.to(dev).requires_grad_(), r.to(dev).requires_grad_()
+    wg = None if w is None else w.to(dev).requires_grad_()
+    if with_res:
+        y, total = pkg.add_rmsnorm_fn(xg, rg, wg, 1e-5)
+        torch.autograd.backward([y, total], [dy.to(dev), dt.to(dev)])
+    else:
+        y = pkg.rmsnorm_fn(xg, wg, 1e-5)
+        y.backward(dy.to(dev))
+    tol = TOL[dtype]
+    what = f"rows {rows} d {d} {dtype} res={with_res} w={with_w}"
+    assert rel_err(y, yr) <= tol, what
+    assert rel_err(xg.grad, xr.grad) <= tol, what
+    if with_res:
+        assert rel_err(rg.grad, rr.grad) <= tol, what
+    if with_w:
+        assert rel_err(wg.grad, wr.grad) <= tol, what
