@@ -143,3 +143,42 @@ def test_config3_256_steps_equal_one_scan_with_carried_state(pkg, dev):
             ys.append(y)
     assert rel_err(torch.stack(ys, 1), y_scan.double()) <= TOL[torch.float32]
     assert rel_err(h, h_scan.double()) <= TOL[torch.float32]
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_step_random_sweep(pkg, dev, seed):
+    # seeded sweep of the decode step: every d_state class of the kernel (4*Q lanes-per-row form, the
+    # one-lane-per-row forms), B / C / z as slices of wider rows, gate + softplus + bias, fresh and
+    # carried state, fp32 and bf16 vectors
+    import random
+    rnd = random.Random(900 + seed)
+    Bs, ED = rnd.choice([1, 2, 5, 64]), rnd.choice([1, 7, 64, 65, 130, 256])
+    N = rnd.choice([1, 2, 3, 4, 8, 12, 16, 16, 16, 24, 32, 64])
+    dtype = rnd.choice([torch.float32, torch.bfloat16])
+    gated, with_h = rnd.random() < 0.6, rnd.random() < 0.7
+    g = torch.Generator().manual_seed(seed)
+    xz = torch.randn(Bs, 2 * ED, generator=g).to(dtype)            # z is the second half of a wider row
+    x, z = torch.randn(Bs, ED, generator=g).to(dtype), xz[:, ED:]
+    raw = (torch.randn(Bs, ED, generator=g) * 0.5 - 3.0).to(dtype)
+    dbc = torch.randn(Bs, 5 + 2 * N, generator=g).to(dtype)        # B and C as slices of one projection
+    Bm, C = dbc[:, 5:5 + N], dbc[:, 5 + N:]
+    A = -torch.rand(ED, N, generator=g) * 4
+    D, bias = torch.randn(ED, generator=g), torch.randn(ED, generator=g) * 0.3
+    h = torch.randn(Bs, ED, N, generator=g) if with_h else None
+    delta = so.softplus_ref(raw.double() + bias.double()) if gated else raw.double().abs() * 0.05
+    yr, hr = so.ssm_step_ref(x.double(), delta, A.double(), Bm.double(), C.double(), D.double(),
+                             None if h is None else h.double())
+    if gated:
+        yr = yr * (z.double() * torch.sigmoid(z.double()))
+        y, hn = pkg.ssm_step(x.to(dev), raw.to(dev), A.to(dev), dbc.to(dev)[:, 5:5 + N], dbc.to(dev)[:, 5 + N:],
+                             D.to(dev), None if h is None else h.to(dev), z=xz.to(dev)[:, ED:],
+                             delta_bias=bias.to(dev), delta_softplus=True)
+    else:
+        dl = (raw.double().abs() * 0.05).to(dtype)
+        yr, hr = so.ssm_step_ref(x.double(), dl.double(), A.double(), Bm.double(), C.double(), D.double(),
+                                 None if h is None else h.double())
+        y, hn = pkg.ssm_step(x.to(dev), dl.to(dev), A.to(dev), dbc.to(dev)[:, 5:5 + N], dbc.to(dev)[:, 5 + N:],
+                             D.to(dev), None if h is None else h.to(dev))
+    what = f"B{Bs} ED{ED} N{N} {dtype} gated={gated} h={with_h}"
+    assert rel_err(y, yr) <= TOL[dtype], what
+    assert rel_err(hn, hr) <= TOL[torch.float32], what
