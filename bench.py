@@ -458,7 +458,8 @@ def main():
     gbs = (fwd_b + bwd_b) / (ms_per_step * 1e-3) / 1e9
     bwd_gbs = bwd_b / (bwd_ms * 1e-3) / 1e9
     out = {
-        "metric": "selective-scan fwd+bwd GB/s (% HBM peak) + tokens/s, 1.4b layer L=4096",
+        "metric": "selective-scan fwd+bwd GB/s (% HBM peak) + tokens/s, "
+                  + ("1.4b layer L=4096" if args.workload == "c2" else desc),
         "value": gbs, "unit": "GB/s",
         "pct_hbm_peak": 100.0 * gbs / HBM_PEAK_GBS,
         "tokens_per_s": B * L / (ms_per_step * 1e-3),
