@@ -5,6 +5,8 @@
 #include <stdint.h>
 #include <stdlib.h>
 
+#include <atomic>
+
 #include "../../include/mambapy_amd.h"
 
 namespace mpa {
@@ -170,7 +172,8 @@ int launch_pack_bc(const mpa_sscan_shape* s, const void* B, const void* C, float
                    int steps_per_subtile, hipStream_t st);
 
 // Kernels may use more LDS than the 64 KB a static __shared__ array can hold (gfx950 has
-// 160 KB per CU), so they take dynamic LDS; the limit is raised once per kernel.
+// 160 KB per CU), so they take dynamic LDS; the limit is raised once per kernel and device (the
+// attribute belongs to the kernel's code object on the device that is current).
 template <typename K>
 inline int allow_dynamic_lds(K kernel, size_t bytes) {
     if (bytes > 160 * 1024) return MPA_ERR_BAD_SHAPE;
@@ -180,5 +183,19 @@ inline int allow_dynamic_lds(K kernel, size_t bytes) {
                ? MPA_OK
                : MPA_ERR_LAUNCH;
 }
+// One per launch site: remembers on which devices the limit of that site's kernel has been raised.
+struct LdsLimitOnce {
+    static constexpr int kMaxDevices = 64;
+    std::atomic<bool> done[kMaxDevices] = {};
+    template <typename K>
+    int ensure(K kernel, size_t bytes) {
+        int dev = -1;
+        if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return MPA_ERR_LAUNCH;
+        if (done[dev].load(std::memory_order_acquire)) return MPA_OK;
+        const int rc = allow_dynamic_lds(kernel, bytes);
+        if (rc == MPA_OK) done[dev].store(true, std::memory_order_release);
+        return rc;
+    }
+};
 
 }  // namespace mpa

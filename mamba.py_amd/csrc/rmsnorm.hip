@@ -329,7 +329,8 @@ static int launch_norm_bwd(const void* x, const float* w, const void* dy, const 
     const NormBwdPlan plan = norm_bwd_plan(rows);
     const size_t lds = part ? (size_t)kNormBwdWaves * d * sizeof(float) : 0;
     // the widest rows of this instantiation need more than the 64 KB a kernel gets by default
-    static const int attr_rc = allow_dynamic_lds(rmsnorm_bwd_kernel<IO, MAXV>,
+    static LdsLimitOnce lds_limit;
+    const int attr_rc = lds_limit.ensure(rmsnorm_bwd_kernel<IO, MAXV>,
                                                  (size_t)kNormBwdWaves * MAXV * kWave * RowVec<IO>::kN * sizeof(float));
     if (attr_rc != MPA_OK) return attr_rc;
     hipLaunchKernelGGL((rmsnorm_bwd_kernel<IO, MAXV>), dim3((unsigned)plan.blocks), dim3(kNormBwdWaves * kWave), lds,

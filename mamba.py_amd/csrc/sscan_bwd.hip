@@ -442,7 +442,8 @@ static int launch_bwd(const BwdParams& p, hipStream_t stream) {
     dim3 grid((p.ED + kWave - 1) / kWave, p.batch);
     dim3 block(NW * kWave);
     constexpr size_t lds = sizeof(float) * BwdLds<NS, NW>::floats(HAS_Z);
-    static const int attr_rc = allow_dynamic_lds(sscan_bwd_kernel<IO, NS, NW, HAS_Z>, lds);
+    static LdsLimitOnce lds_limit;
+    const int attr_rc = lds_limit.ensure(sscan_bwd_kernel<IO, NS, NW, HAS_Z>, lds);
     if (attr_rc != MPA_OK) return attr_rc;
     hipLaunchKernelGGL((sscan_bwd_kernel<IO, NS, NW, HAS_Z>), grid, block, lds, stream, p);
     return check_launch();

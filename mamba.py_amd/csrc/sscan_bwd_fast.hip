@@ -669,7 +669,8 @@ static int launch_fast(const BwdParams& p, hipStream_t stream) {
     dim3 block((NW + kSvc) * kWave);
     constexpr size_t lds = sizeof(float) * BwdFastLds<NS, NW>::floats;
     static_assert(lds <= 160 * 1024, "LDS budget");
-    static const int attr_rc = allow_dynamic_lds(sscan_bwd_fast_kernel<IO, NS, NW, HAS_Z>, lds);
+    static LdsLimitOnce lds_limit;
+    const int attr_rc = lds_limit.ensure(sscan_bwd_fast_kernel<IO, NS, NW, HAS_Z>, lds);
     if (attr_rc != MPA_OK) return attr_rc;
     hipLaunchKernelGGL((sscan_bwd_fast_kernel<IO, NS, NW, HAS_Z>), grid, block, lds, stream, p);
     return check_launch();

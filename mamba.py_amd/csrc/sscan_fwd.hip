@@ -634,7 +634,8 @@ static int launch_fwd(const FwdParams& p, hipStream_t stream) {
     dim3 grid((p.ED + kWave - 1) / kWave, p.batch * (p.nseg > 1 ? p.nseg : 1));
     dim3 block((NW + kService) * kWave);
     constexpr size_t lds = sizeof(float) * FwdLds<NS, NW>::floats;
-    static const int attr_rc = allow_dynamic_lds(sscan_fwd_kernel<IO, NS, NW, HAS_Z>, lds);
+    static LdsLimitOnce lds_limit;
+    const int attr_rc = lds_limit.ensure(sscan_fwd_kernel<IO, NS, NW, HAS_Z>, lds);
     if (attr_rc != MPA_OK) return attr_rc;
     hipLaunchKernelGGL((sscan_fwd_kernel<IO, NS, NW, HAS_Z>), grid, block, lds, stream, p);
     return check_launch();
