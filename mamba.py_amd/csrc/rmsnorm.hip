@@ -285,7 +285,7 @@ __global__ void __launch_bounds__(1024) rmsnorm_bwd_finish_kernel(const float* p
 }
 
 static int norm_validate(int64_t rows, int64_t d, int io_dtype) {
-    if (rows <= 0 || d <= 0 || rows > (int64_t)1 << 40) return MPA_ERR_BAD_SHAPE;
+    if (rows <= 0 || d <= 0 || rows > (int64_t)1 << 31) return MPA_ERR_BAD_SHAPE;  // one wave per one or two rows
     if (io_dtype != MPA_F32 && io_dtype != MPA_BF16) return MPA_ERR_BAD_DTYPE;
     const int vec = io_dtype == MPA_BF16 ? 8 : 4;
     if (d % vec != 0 || d / vec > 8 * kWave) return MPA_ERR_BAD_SHAPE;  // d <= 4096 (bf16) / 2048 (f32)
