@@ -235,6 +235,7 @@ static int conv_validate(const mpa_conv_shape* s) {
     if (s->batch <= 0 || s->seqlen <= 0 || s->dim <= 0 || s->batch > 65535) return MPA_ERR_BAD_SHAPE;
     if (s->kernel < 2 || s->kernel > kConvMaxK) return MPA_ERR_BAD_SHAPE;
     if (s->seqlen > (int64_t)1 << 30 || s->dim > (int64_t)1 << 30) return MPA_ERR_BAD_SHAPE;
+    if ((s->seqlen + kConvSpan - 1) / kConvSpan > 65535) return MPA_ERR_BAD_SHAPE;  // spans are the grid's y axis
     if (s->io_dtype != MPA_F32 && s->io_dtype != MPA_BF16) return MPA_ERR_BAD_DTYPE;
     const int64_t st[] = {s->x_sb, s->x_sl, s->x_sd, s->y_sb, s->y_sl, s->y_sd, s->g_sb, s->g_sl, s->g_sd};
     for (int64_t v : st)
