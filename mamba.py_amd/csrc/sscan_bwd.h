@@ -21,8 +21,9 @@ struct BwdParams {
     void* dx;
     void* ddelta;
     void* dz;
-    float* partB;   // [CG][batch][L][N]
-    float* partC;   // [CG][batch][L][N]
+    float* partB;   // [CG] groups of [batch][L][N], part_gs floats apart
+    float* partC;   // same layout
+    int64_t part_gs;  // distance between the partials of two channel groups (see bwd_workspace)
     float* partA;   // [batch][ED][N]
     float* partD;   // [batch][ED]
     float* partDb;  // [batch][ED]  (ddelta_bias)

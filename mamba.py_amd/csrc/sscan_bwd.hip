@@ -277,7 +277,7 @@ __global__ void __launch_bounds__(NW* kWave) sscan_bwd_kernel(const BwdParams p)
                     const int n = w * NS + (o % NS);
                     if (part == 0 && t < p.L && n < p.N) {
                         float* dst = (o < NS) ? p.partB : p.partC;
-                        dst[(((int64_t)cg * p.batch + b) * p.L + t) * p.N + n] = s;
+                        dst[cg * p.part_gs + ((int64_t)b * p.L + t) * p.N + n] = s;
                     }
                     wave_lds_sync();
                 }
@@ -381,25 +381,66 @@ __global__ void __launch_bounds__(NW* kWave) sscan_bwd_kernel(const BwdParams p)
 }
 
 // Sums the partial buffers: dB/dC over channel groups, dA/dD/ddelta_bias over the batch.
-template <typename IO>
+// V = 4: d_state is a multiple of 4, a thread sums four consecutive states with 16-byte loads.
+template <typename IO, int V>
 __global__ void __launch_bounds__(256) sscan_bwd_finish_kernel(
     const float* partB, const float* partC, const float* partA, const float* partD,
-    const float* partDb, void* dB, void* dC, float* dA, float* dD, float* dDb, int CG, int batch,
-    int L, int ED, int N, int64_t dbc_sb, int64_t dbc_sl) {
+    const float* partDb, void* dB, void* dC, float* dA, float* dD, float* dDb, int CG, int64_t gs,
+    int batch, int L, int ED, int N, int64_t dbc_sb, int64_t dbc_sl) {
     const int64_t bln = (int64_t)batch * L * N;
     const int64_t edn = (int64_t)ED * N;
-    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < bln) {
-        float sb = 0.0f, sc = 0.0f;
-        for (int g = 0; g < CG; ++g) {
-            sb += partB[g * bln + i];
-            sc += partC[g * bln + i];
+    const int64_t nbc = bln / V;  // threads of the dB/dC part
+    const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t i = t - nbc + bln;  // index into the dA / dD parts, as if V were 1
+    if (t < nbc) {
+        float sb[V], sc[V];
+#pragma unroll
+        for (int v = 0; v < V; ++v) sb[v] = sc[v] = 0.0f;
+        // eight groups per round: all sixteen loads are issued before the first sum (the kernel is
+        // bound by memory latency, not by instructions); the order of the additions is fixed
+        constexpr int kRound = 8;
+        for (int g0 = 0; g0 < CG; g0 += kRound) {
+            if constexpr (V == 4) {
+                float4 b4[kRound], c4[kRound];
+#pragma unroll
+                for (int r = 0; r < kRound; ++r) {
+                    const int g = g0 + r < CG ? g0 + r : CG - 1;  // clamped copies are not added
+                    b4[r] = *reinterpret_cast<const float4*>(partB + g * gs + 4 * t);
+                    c4[r] = *reinterpret_cast<const float4*>(partC + g * gs + 4 * t);
+                }
+#pragma unroll
+                for (int r = 0; r < kRound; ++r) {
+                    if (g0 + r < CG) {
+                        sb[0] += b4[r].x; sb[1] += b4[r].y; sb[2] += b4[r].z; sb[3] += b4[r].w;
+                        sc[0] += c4[r].x; sc[1] += c4[r].y; sc[2] += c4[r].z; sc[3] += c4[r].w;
+                    }
+                }
+            } else {
+                float b1[kRound], c1[kRound];
+#pragma unroll
+                for (int r = 0; r < kRound; ++r) {
+                    const int g = g0 + r < CG ? g0 + r : CG - 1;
+                    b1[r] = partB[g * gs + t];
+                    c1[r] = partC[g * gs + t];
+                }
+#pragma unroll
+                for (int r = 0; r < kRound; ++r) {
+                    if (g0 + r < CG) {
+                        sb[0] += b1[r];
+                        sc[0] += c1[r];
+                    }
+                }
+            }
         }
-        const int n = (int)(i % N);
-        const int64_t bt = i / N;
+        const int64_t e = V * t;
+        const int n = (int)(e % N);
+        const int64_t bt = e / N;
         const int64_t off = (bt / L) * dbc_sb + (bt % L) * dbc_sl + n;
-        store_from_float<IO>(dB, off, sb);
-        store_from_float<IO>(dC, off, sc);
+#pragma unroll
+        for (int v = 0; v < V; ++v) {
+            store_from_float<IO>(dB, off + v, sb[v]);
+            store_from_float<IO>(dC, off + v, sc[v]);
+        }
     } else if (i < bln + edn) {
         const int64_t j = i - bln;
         float s = 0.0f;
@@ -418,7 +459,7 @@ __global__ void __launch_bounds__(256) sscan_bwd_finish_kernel(
 }
 
 struct BwdWorkspace {
-    size_t offB, offC, offA, offD, offDb, total;
+    size_t offB, offC, offA, offD, offDb, total, group_stride;
 };
 
 static BwdWorkspace bwd_workspace(const mpa_sscan_shape* s) {
@@ -428,9 +469,14 @@ static BwdWorkspace bwd_workspace(const mpa_sscan_shape* s) {
     const size_t be = (size_t)s->batch * s->dim;
     auto up = [](size_t v) { return (v + 63) / 64 * 64; };  // 256-byte granules of floats
     BwdWorkspace w;
+    // The partial sums of the channel groups for one (batch, step, state) are written at the same
+    // time by different workgroups and read together by the finish kernel.  batch*L*N floats is
+    // often a power of two (1 MiB at the headline shape), which would put all of them on the same
+    // memory channel: an odd number of 256-byte lines between groups spreads them.
+    w.group_stride = up(bln) + 17 * 64;
     w.offB = 0;
-    w.offC = w.offB + up(cg * bln);
-    w.offA = w.offC + up(cg * bln);
+    w.offC = w.offB + cg * w.group_stride;
+    w.offA = w.offC + cg * w.group_stride;
     w.offD = w.offA + up(ben);
     w.offDb = w.offD + up(be);
     w.total = (w.offDb + up(be)) * sizeof(float);
@@ -503,6 +549,7 @@ extern "C" int mpa_sscan_bwd(const mpa_sscan_shape* s, const void* x, const void
     p.ypre = z ? y_pregate : nullptr;
     p.dbias = delta_bias; p.h0 = h0; p.ckpt = h_ckpt; p.dx = dx; p.ddelta = ddelta; p.dz = dz;
     p.partB = wsf + ws.offB; p.partC = wsf + ws.offC; p.partA = wsf + ws.offA;
+    p.part_gs = (int64_t)ws.group_stride;
     p.partD = wsf + ws.offD; p.partDb = wsf + ws.offDb;
     p.batch = (int)s->batch; p.L = (int)s->seqlen; p.ED = (int)s->dim; p.N = (int)s->dstate;
     p.nchunks = (p.L + kTile - 1) / kTile;
@@ -532,15 +579,21 @@ extern "C" int mpa_sscan_bwd(const mpa_sscan_shape* s, const void* x, const void
     if (rc != MPA_OK) return rc;
 
     const int cg = (p.ED + kWave - 1) / kWave;
-    const int64_t total = (int64_t)p.batch * p.L * p.N + (int64_t)p.ED * p.N + p.ED;
+    // the partial buffers start on 256-byte granules, so rows of four states are 16-byte aligned
+    const int vec = p.N % 4 == 0 ? 4 : 1;
+    const int64_t total = (int64_t)p.batch * p.L * p.N / vec + (int64_t)p.ED * p.N + p.ED;
     dim3 fgrid((unsigned)((total + 255) / 256));
-    if (s->io_dtype == MPA_F32)
-        hipLaunchKernelGGL(sscan_bwd_finish_kernel<float>, fgrid, dim3(256), 0, st, p.partB, p.partC,
-                           p.partA, p.partD, softplus && ddelta_bias ? p.partDb : nullptr, dB, dC, dA, dD,
-                           ddelta_bias, cg, p.batch, p.L, p.ED, p.N, s->dbc_sb, s->dbc_sl);
-    else
-        hipLaunchKernelGGL(sscan_bwd_finish_kernel<bf16_t>, fgrid, dim3(256), 0, st, p.partB, p.partC,
-                           p.partA, p.partD, softplus && ddelta_bias ? p.partDb : nullptr, dB, dC, dA, dD,
-                           ddelta_bias, cg, p.batch, p.L, p.ED, p.N, s->dbc_sb, s->dbc_sl);
+#define MPA_FINISH(IO_, V_)                                                                                    \
+    hipLaunchKernelGGL((sscan_bwd_finish_kernel<IO_, V_>), fgrid, dim3(256), 0, st, p.partB, p.partC, p.partA, \
+                       p.partD, softplus && ddelta_bias ? p.partDb : nullptr, dB, dC, dA, dD, ddelta_bias, cg,  \
+                       p.part_gs, p.batch, p.L, p.ED, p.N, s->dbc_sb, s->dbc_sl)
+    if (s->io_dtype == MPA_F32) {
+        if (vec == 4) MPA_FINISH(float, 4);
+        else MPA_FINISH(float, 1);
+    } else {
+        if (vec == 4) MPA_FINISH(bf16_t, 4);
+        else MPA_FINISH(bf16_t, 1);
+    }
+#undef MPA_FINISH
     return check_launch();
 }

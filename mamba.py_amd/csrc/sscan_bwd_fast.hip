@@ -217,7 +217,7 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
         const int fw_i = ((sw >> 1) * kWave + lane) * kFw;  // index inside the [kTile][NP] half
         const int fw_tt = fw_i / NP, fw_n = fw_i % NP;
         const int fw_e = (fw_tt * 2 + fw_which) * NP + fw_n;  // index inside the dB|dC tile in LDS
-        float* const fw_base = (fw_which ? p.partC : p.partB) + ((int64_t)cg * p.batch + b) * p.L * p.N;
+        float* const fw_base = (fw_which ? p.partC : p.partB) + cg * p.part_gs + (int64_t)b * p.L * p.N;
         const uint32_t fw_off = ((uint32_t)fw_tt * (uint32_t)p.N + (uint32_t)fw_n) * 4u;
         const bool fw_vec = p.N == NP;  // rows of the partial buffers are then aligned for vector stores
 
