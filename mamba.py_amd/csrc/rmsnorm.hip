@@ -5,8 +5,8 @@
 // add + rsqrt, two multiplies), each a full pass over the activations.  Here one wave owns a
 // row: it reads the row once with 16-byte loads into registers, sums across its lanes with six
 // DPP additions (no LDS round trips), and writes the result from the same registers.  The
-// kernels are bound by HBM, so they are organised to keep bytes in flight: the forward holds two
-// rows per wave at a time, the backward requests the next row before it works on the current
+// kernels are bound by HBM, so they are organised to keep bytes in flight: the forward holds four
+// rows per wave at a time (two: 37 us, four: 34 us at 32768 x 768 bfloat16), the backward requests the next row before it works on the current
 // one.  Backward: dweight is summed per wave in registers, per block through LDS, and over the
 // blocks by a second kernel in a fixed order (no float atomics).
 //
@@ -315,7 +315,7 @@ static NormBwdPlan norm_bwd_plan(int64_t rows) {
 template <typename IO, int MAXV>
 static int launch_norm_fwd(const void* x, const void* res, const float* w, void* y, void* sum_out, float* rstd,
                            int64_t rows, int d, float eps, hipStream_t st) {
-    constexpr int R = MAXV <= 2 ? 2 : 1;
+    constexpr int R = MAXV <= 2 ? 4 : 1;
     const int64_t waves = (rows + R - 1) / R;
     hipLaunchKernelGGL((rmsnorm_fwd_kernel<IO, MAXV, R>), dim3((unsigned)((waves + 3) / 4)), dim3(256), 0, st,
                        static_cast<const IO*>(x), static_cast<const IO*>(res), w, static_cast<IO*>(y),
