@@ -418,3 +418,37 @@ def test_random_shapes_layouts_and_options(pkg, dev, seed):
             continue
         e = rel_err(got[k], ref[k])
         assert e <= (TOL[torch.float32] if k == "hl" and dtype == torch.float32 else tol), f"{what}: {k} rel err {e:.3e}"
+
+
+def test_config2_shape_gated_softplus_bf16_channel_slice(pkg, dev):
+    # The fused form a Mamba layer actually calls (gate + softplus + bias) at the headline shape,
+    # B=4, L=4096, ED=4096, N=16, bf16 I/O.  Channels are independent, so y, dx, ddelta, dz and
+    # the per-channel gradients dA, dD, dbias of a 16-channel slice of the full-size run must
+    # match the float64 oracle run on that slice alone (dB/dC sum over all channels and are
+    # covered at full size by the ungated test above).
+    Bs, L, ED, N, S = 4, 4096, 4096, 16, 16
+    dt = torch.bfloat16
+    inp = so.make_inputs(Bs, L, ED, N, seed=1002, dtype=dt)
+    g = torch.Generator().manual_seed(2002)
+    z = torch.randn(Bs, L, ED, generator=g).to(dt)
+    raw = (torch.randn(Bs, L, ED, generator=g) * 0.5 - 4.0).to(dt)
+    bias = torch.randn(ED, generator=g) * 0.3
+    t = lambda v: v.to(dev).requires_grad_()
+    gx, gr, gA, gB, gC, gD, gz, gb = map(t, (inp["x"], raw, inp["A"], inp["B"], inp["C"], inp["D"], z, bias))
+    y = pkg.selective_scan_fn(gx, gr, gA, gB, gC, gD, z=gz, delta_bias=gb, delta_softplus=True)
+    y.backward(inp["dy"].to(dev))
+    sl = slice(1016, 1016 + S)  # a slice that straddles two 64-channel groups (boundary at 1024)
+    f64 = lambda v: v.double().requires_grad_()
+    x, r, A, Dd, zz, bb = map(f64, (inp["x"][..., sl], raw[..., sl], inp["A"][sl], inp["D"][sl], z[..., sl], bias[sl]))
+    Bm, C = inp["B"].double(), inp["C"].double()
+    yr = so.selective_scan_ref(x, so.softplus_ref(r + bb), A, Bm, C, Dd)
+    yr = yr * (zz * torch.sigmoid(zz))
+    yr.backward(inp["dy"][..., sl].double())
+    tol = TOL[dt]
+    assert rel_err(y[..., sl], yr) <= tol
+    assert rel_err(gx.grad[..., sl], x.grad) <= tol
+    assert rel_err(gr.grad[..., sl], r.grad) <= tol
+    assert rel_err(gz.grad[..., sl], zz.grad) <= tol
+    assert rel_err(gA.grad[sl], A.grad) <= tol
+    assert rel_err(gD.grad[sl], Dd.grad) <= tol
+    assert rel_err(gb.grad[sl], bb.grad) <= tol
