@@ -127,3 +127,22 @@ def test_rmsnorm_random_sweep(pkg, dev, seed):
         assert rel_err(rg.grad, rr.grad) <= tol, what
     if with_w:
         assert rel_err(wg.grad, wr.grad) <= tol, what
+
+
+def test_add_rmsnorm_configs4_layer_shape_bf16(pkg, dev):
+    # the norm of configs[4] at full size: (8, 4096, 768) bf16 with the residual add, forward and backward
+    g = torch.Generator().manual_seed(1004)
+    shape, dtype = (8, 4096, 768), torch.bfloat16
+    x, r, dy, dt = (torch.randn(*shape, generator=g).to(dtype) for _ in range(4))
+    w = torch.randn(768, generator=g) * 0.2 + 1.0
+    xr, rr, wr = x.double().requires_grad_(), r.double().requires_grad_(), w.double().requires_grad_()
+    tr = xr + rr
+    tq = tr + (tr.detach().to(dtype).double() - tr.detach())
+    yr = so.rmsnorm_ref(tq, wr, 1e-5)
+    ((yr * dy.double()).sum() + (tq * dt.double()).sum()).backward()
+    xg, rg, wg = x.to(dev).requires_grad_(), r.to(dev).requires_grad_(), w.to(dev).requires_grad_()
+    y, total = pkg.add_rmsnorm_fn(xg, rg, wg, 1e-5)
+    torch.autograd.backward([y, total], [dy.to(dev), dt.to(dev)])
+    tol = TOL[dtype]
+    assert rel_err(y, yr) <= tol and rel_err(xg.grad, xr.grad) <= tol and rel_err(wg.grad, wr.grad) <= tol
+    assert torch.equal(xg.grad, rg.grad)
