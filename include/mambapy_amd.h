@@ -12,7 +12,9 @@
  *   - io_dtype selects the storage type of x, delta, B, C, z, y, dy and of their
  *     gradients; A, D, delta_bias, the recurrent state and every accumulation are float32;
  *   - the return value is MPA_OK or one of the MPA_ERR_* codes; nothing is thrown.
- * All entry points are reentrant and keep no global state.
+ * All entry points are reentrant and keep no global state: nothing is read from the
+ * environment, every choice the library makes is a function of the arguments (the
+ * workspace queries and the calls they size therefore always agree).
  */
 #ifndef MAMBAPY_AMD_H
 #define MAMBAPY_AMD_H
@@ -24,7 +26,7 @@
 extern "C" {
 #endif
 
-#define MPA_VERSION 100 /* major*10000 + minor*100 + patch */
+#define MPA_VERSION 200 /* major*10000 + minor*100 + patch */
 
 enum mpa_status {
     MPA_OK = 0,
@@ -66,11 +68,30 @@ typedef struct mpa_sscan_shape {
     int64_t g_sb, g_sl, g_sd;
     int64_t bc_sb, bc_sl;
     int64_t dbc_sb, dbc_sl;
+    /* Launch plan.  0 = chosen by the library from the shape (the normal case); a caller that
+     * tunes or tests may pin the decomposition.  The same values must be given to a call and
+     * to the workspace query that sizes it. */
+    int32_t plan_states_per_lane; /* states of d_state kept by one lane: a power of two */
+    int32_t plan_segments;        /* pieces the sequence is cut into (1 = never cut) */
+    int32_t plan_flags;           /* bit set of MPA_PLAN_* */
+    int32_t reserved;             /* 0 */
 } mpa_sscan_shape;
 
 /* delta = softplus(delta + delta_bias) is applied inside the kernel (mamba.py:264-265);
  * without the flag `delta` is used as given and delta_bias must be NULL. */
 #define MPA_SSCAN_DELTA_SOFTPLUS 1
+/* The recurrence runs from the last step to the first: h[t] = a[t]*h[t+1] + ..., h0 is the
+ * state before step seqlen-1 and h_last the state after step 0.  Equal to flipping x, delta,
+ * z, B, C along time, scanning, and flipping y back, which is how the reference's
+ * bidirectional block obtains its backward direction (mambapy/vim.py:228-261: xz.flip([1])
+ * in, y_b.flip([1]) out) at the price of those copies. */
+#define MPA_SSCAN_REVERSE 2
+
+/* mpa_sscan_bwd: use the general backward kernel even where the fast one applies. */
+#define MPA_PLAN_BWD_GENERAL 1
+/* Test hook: the bounded waits inside the kernels behave as if they had run out (see
+ * mpa_sscan_bwd); every kernel still runs to its end. */
+#define MPA_PLAN_EXPIRE_WAITS 2
 
 int mpa_version(void);
 /* Host string naming the GPU architecture the kernels were compiled for ("gfx950"). */
@@ -94,6 +115,10 @@ const char* mpa_status_string(int status);
  *   y_pregate  optional, only with z: the output before the gate (C.h + D*x), io_dtype, strides
  *            of y.  mpa_sscan_bwd needs it on its fast path; NULL when no gradient is needed.
  *   workspace  scratch of mpa_sscan_fwd_workspace_bytes() bytes.
+ * When batch * dim/64 workgroups would cover a fraction of the chip, the sequence is cut into
+ * segments that run side by side (end states of all segments from zero, a carry pass, then the
+ * real pass from the true initial states); checkpoints, h_last and y are the same as without the
+ * cut up to float32 rounding.
  */
 int mpa_sscan_fwd(const mpa_sscan_shape* s, const void* x, const void* delta, const float* A,
                   const void* B, const void* C, const float* D, const void* z,
@@ -105,9 +130,10 @@ int mpa_sscan_fwd(const mpa_sscan_shape* s, const void* x, const void* delta, co
 int64_t mpa_sscan_ckpt_elems(const mpa_sscan_shape* s);
 
 /* Bytes of the scratch `workspace` of mpa_sscan_fwd (256-byte aligned; holds B and C
- * repacked as float32 in the order the scan waves read them; contents are dead after the
- * call). */
-size_t mpa_sscan_fwd_workspace_bytes(const mpa_sscan_shape* s);
+ * repacked as float32 in the order the scan waves read them, or the per-segment states of a
+ * cut sequence; contents are dead after the call).  with_ckpt = 1 for a call that passes
+ * h_ckpt, 0 for one that does not (the two are cut differently). */
+size_t mpa_sscan_fwd_workspace_bytes(const mpa_sscan_shape* s, int with_ckpt);
 
 /* ---- fused selective scan, backward -----------------------------------------------------
  * Replaces what autograd records for mamba.py:284-293 plus PScan.backward
@@ -120,6 +146,11 @@ size_t mpa_sscan_fwd_workspace_bytes(const mpa_sscan_shape* s);
  * given.  y_pregate (strides of dy) is what the forward call wrote for the same inputs; with z
  * and y_pregate == NULL the pre-gate output is recomputed by a slower, more general kernel.
  * `workspace` needs mpa_sscan_bwd_workspace_bytes() bytes, 256-byte aligned.
+ * d_state up to MPA_MAX_DSTATE.  Short batches of long sequences are cut into segments as in
+ * the forward call (the carry runs from the end).
+ * One kernel waits, with a bound, for a counter in shared memory; the wait cannot run out
+ * unless the hardware scheduler misbehaves, and if it ever does the call does not return clean
+ * numbers: every element of dA, dD (and ddelta_bias) is then NaN.
  */
 int mpa_sscan_bwd(const mpa_sscan_shape* s, const void* x, const void* delta, const float* A,
                   const void* B, const void* C, const float* D, const void* z,

@@ -11,6 +11,9 @@ LIB_PATH = os.path.join(_HERE, "csrc", "libmambapy_amd.so")
 
 MPA_F32, MPA_BF16 = 0, 1
 MPA_SSCAN_DELTA_SOFTPLUS = 1
+MPA_SSCAN_REVERSE = 2
+MPA_PLAN_BWD_GENERAL = 1
+MPA_PLAN_EXPIRE_WAITS = 2
 MPA_CONV_SILU = 1
 MPA_CKPT_STEPS = 16
 MPA_MAX_DSTATE = 256
@@ -27,7 +30,8 @@ class SscanShape(ctypes.Structure):
                [("io_dtype", ctypes.c_int32), ("flags", ctypes.c_int32)] + \
                [(n, ctypes.c_int64) for n in (
                    "u_sb", "u_sl", "u_sd", "z_sb", "z_sl", "z_sd", "d_sb", "d_sl", "d_sd", "y_sb", "y_sl", "y_sd",
-                   "g_sb", "g_sl", "g_sd", "bc_sb", "bc_sl", "dbc_sb", "dbc_sl")]
+                   "g_sb", "g_sl", "g_sd", "bc_sb", "bc_sl", "dbc_sb", "dbc_sl")] + \
+               [(n, ctypes.c_int32) for n in ("plan_states_per_lane", "plan_segments", "plan_flags", "reserved")]
 
 
 class ConvShape(ctypes.Structure):
@@ -66,7 +70,7 @@ def load():
     lib.mpa_status_string.argtypes = [ctypes.c_int]
     sp = ctypes.POINTER(SscanShape)
     lib.mpa_sscan_fwd.argtypes = [sp] + [vp] * 14 + [sz, vp]
-    lib.mpa_sscan_fwd_workspace_bytes.argtypes = [sp]
+    lib.mpa_sscan_fwd_workspace_bytes.argtypes = [sp, ctypes.c_int]
     lib.mpa_sscan_fwd_workspace_bytes.restype = sz
     lib.mpa_sscan_ckpt_elems.argtypes = [sp]
     lib.mpa_sscan_ckpt_elems.restype = i64

@@ -163,7 +163,7 @@ inline size_t dtype_size(int dt) { return dt == MPA_BF16 ? 2 : 4; }
 
 // states owned by one lane of a scan wave, chosen from the problem size so that the launch
 // fills the 1024 SIMDs of the chip (the only parallel axes are batch*dim and d_state)
-int pick_states_per_lane(int64_t batch, int64_t dim, int64_t dstate, int ns_max, const char* env);
+int pick_states_per_lane(int64_t batch, int64_t dim, int64_t dstate, int ns_max, int pinned);
 int padded_states(int64_t n);
 int validate_shape(const mpa_sscan_shape* s);
 // B and C repacked as float32 for scalar loads (see pack_bc_kernel in sscan_fwd.hip)

@@ -24,9 +24,17 @@ struct BwdParams {
     float* partB;   // [CG] groups of [batch][L][N], part_gs floats apart
     float* partC;   // same layout
     int64_t part_gs;  // distance between the partials of two channel groups (see bwd_workspace)
-    float* partA;   // [batch][ED][N]
-    float* partD;   // [batch][ED]
-    float* partDb;  // [batch][ED]  (ddelta_bias)
+    float* partA;   // [rows][ED][N]   rows = batch * nseg
+    float* partD;   // [rows][ED]
+    float* partDb;  // [rows][ED]  (ddelta_bias)
+    // sequence cut into nseg segments of seg_tiles tiles, counted from the END of the forward
+    // walk (the order in which the backward visits them); ag0 [rows][ED][N] = a*g flowing into
+    // every segment from the one visited before it (NULL = zeros: not cut)
+    const float* ag0;
+    int nseg, seg_tiles;
+    int* status;       // device word: set to 1 when a bounded wait inside the kernel runs out
+    int expire_waits;  // test hook: treat every bounded wait as run out
+    int reverse;       // the forward walk ran from the last physical step to the first
     int batch, L, ED, N, nchunks;
     int softplus;
     int in_tmajor, dy_tmajor, out_tmajor;

@@ -18,6 +18,7 @@
 // steps; over channel groups, batch and time by deterministic partial buffers that a small
 // second kernel sums (no floating-point atomics: results are bitwise reproducible).
 #include "sscan_bwd.h"
+#include "sscan_fwd.h"
 
 namespace mpa {
 
@@ -111,17 +112,22 @@ __global__ void __launch_bounds__(NW* kWave) sscan_bwd_kernel(const BwdParams p)
         }
     };
 
+    // c counts the tiles in the order of the forward walk (the index of their checkpoints) and tt
+    // the steps inside a tile likewise; with a reverse walk both are mirrored in memory
+    const bool rev = p.reverse != 0;
+    auto first_step = [&](int c) { return (rev ? p.nchunks - 1 - c : c) * kTile; };
+    auto phys_step = [&](int tt) { return rev ? kTile - 1 - tt : tt; };
+
     auto prefetch = [&](int c) {
-        const int t0 = c * kTile;
-        const int tl = min(kTile, p.L - t0);
+        const int t0 = first_step(c);
 #pragma unroll
         for (int k = 0; k < EPT; ++k) {
             const int idx = tid + k * NT;
             int tt, cc;
             elem_map(idx, p.in_tmajor, tt, cc);
             float xv = 0.0f, dv = 0.0f, dyv = 0.0f, zv = 0.0f;
-            if (idx < kTile * kWave && tt < tl && d0 + cc < p.ED) {
-                const int64_t t = t0 + tt;
+            if (idx < kTile * kWave && t0 + phys_step(tt) < p.L && d0 + cc < p.ED) {
+                const int64_t t = t0 + phys_step(tt);
                 const int64_t ch = d0 + cc;
                 xv = load_as_float<IO>(p.x, b * p.u_sb + t * p.u_sl + ch * p.u_sd);
                 dv = load_as_float<IO>(p.delta, b * p.d_sb + t * p.d_sl + ch * p.d_sd);
@@ -138,8 +144,8 @@ __global__ void __launch_bounds__(NW* kWave) sscan_bwd_kernel(const BwdParams p)
             const int idx = tid + k * NT;
             const int tt = idx / NP, n = idx % NP;
             float bv = 0.0f, cv = 0.0f;
-            if (idx < kTile * NP && tt < tl && n < p.N) {
-                const int64_t off = b * p.bc_sb + (int64_t)(t0 + tt) * p.bc_sl + n;
+            if (idx < kTile * NP && t0 + phys_step(tt) < p.L && n < p.N) {
+                const int64_t off = b * p.bc_sb + (int64_t)(t0 + phys_step(tt)) * p.bc_sl + n;
                 bv = load_as_float<IO>(p.Bm, off);
                 cv = load_as_float<IO>(p.C, off);
             }
@@ -163,7 +169,7 @@ __global__ void __launch_bounds__(NW* kWave) sscan_bwd_kernel(const BwdParams p)
 
     // sDelta holds the delta the recurrence uses (after softplus); the raw value that the
     // softplus derivative needs is recomputed from it: sigmoid(raw) = 1 - exp(-softplus(raw))
-    auto stage = [&](int tl) {
+    auto stage = [&](int t0) {
 #pragma unroll
         for (int k = 0; k < EPT; ++k) {
             const int idx = tid + k * NT;
@@ -171,7 +177,7 @@ __global__ void __launch_bounds__(NW* kWave) sscan_bwd_kernel(const BwdParams p)
             elem_map(idx, p.in_tmajor, tt, cc);
             if (idx < kTile * kWave) {
                 float dv = rDl[k];
-                const bool live = (tt < tl && d0 + cc < p.ED);
+                const bool live = (t0 + phys_step(tt) < p.L && d0 + cc < p.ED);
                 if (p.softplus && live) dv = softplus_f(dv + (p.dbias ? p.dbias[d0 + cc] : 0.0f));
                 float dyv = rDy[k];
                 if (HAS_Z) {
@@ -200,12 +206,11 @@ __global__ void __launch_bounds__(NW* kWave) sscan_bwd_kernel(const BwdParams p)
     const int last = p.nchunks - 1;
     prefetch(last);
     for (int c = last; c >= 0; --c) {
-        const int t0 = c * kTile;
-        const int tl = min(kTile, p.L - t0);
+        const int t0 = first_step(c);
         float h[NS];
         // a tail chunk was prefetched with zero padding (delta = 0: a = 1, u = 0; dy = 0),
         // which makes the padded steps exact no-ops in both sweeps
-        stage(tl);
+        stage(t0);
 #pragma unroll
         for (int i = 0; i < NS; ++i) h[i] = rH[i];
         __syncthreads();
@@ -273,7 +278,7 @@ __global__ void __launch_bounds__(NW* kWave) sscan_bwd_kernel(const BwdParams p)
 #pragma unroll
                     for (int m = 1; m < LPR; m *= 2) s += __shfl_xor(s, m, kWave);
                     const int rs = row / (2 * NS), o = row % (2 * NS);
-                    const int t = t0 + tt + rs;
+                    const int t = t0 + phys_step(tt + rs);
                     const int n = w * NS + (o % NS);
                     if (part == 0 && t < p.L && n < p.N) {
                         float* dst = (o < NS) ? p.partB : p.partC;
@@ -297,7 +302,7 @@ __global__ void __launch_bounds__(NW* kWave) sscan_bwd_kernel(const BwdParams p)
                     cc = idx % kWave;
                 }
                 const int tt = seg * PS + ts;
-                if (idx < PS * kWave && tt < tl && d0 + cc < p.ED) {
+                if (idx < PS * kWave && t0 + phys_step(tt) < p.L && d0 + cc < p.ED) {
                     float gB = 0.0f, dd = 0.0f;
 #pragma unroll
                     for (int ww = 0; ww < NW; ++ww) {
@@ -308,7 +313,7 @@ __global__ void __launch_bounds__(NW* kWave) sscan_bwd_kernel(const BwdParams p)
                     const float dv = sDelta[0][tt][cc];
                     const float dyg = sDy[0][tt][cc];  // dy, already gated when HAS_Z
                     const float Dv = p.D[d0 + cc];
-                    const int64_t t = t0 + tt;
+                    const int64_t t = t0 + phys_step(tt);
                     const int64_t ch = d0 + cc;
                     const float dxv = __builtin_fmaf(dv, gB, Dv * dyg);
                     float ddv = __builtin_fmaf(xv, gB, dd * kLn2);
@@ -380,13 +385,15 @@ __global__ void __launch_bounds__(NW* kWave) sscan_bwd_kernel(const BwdParams p)
     }
 }
 
-// Sums the partial buffers: dB/dC over channel groups, dA/dD/ddelta_bias over the batch.
-// V = 4: d_state is a multiple of 4, a thread sums four consecutive states with 16-byte loads.
+// Sums the partial buffers: dB/dC over channel groups, dA/dD/ddelta_bias over the rows of the
+// main launch (batch rows, or their segments).  V = 4: d_state is a multiple of 4, a thread sums
+// four consecutive states with 16-byte loads.  `status` is the word the main kernel sets when one
+// of its bounded waits ran out: the parameter gradients are then NaN, never silently wrong.
 template <typename IO, int V>
 __global__ void __launch_bounds__(256) sscan_bwd_finish_kernel(
     const float* partB, const float* partC, const float* partA, const float* partD,
     const float* partDb, void* dB, void* dC, float* dA, float* dD, float* dDb, int CG, int64_t gs,
-    int batch, int L, int ED, int N, int64_t dbc_sb, int64_t dbc_sl) {
+    int batch, int rows, int L, int ED, int N, int64_t dbc_sb, int64_t dbc_sl, const int* status) {
     const int64_t bln = (int64_t)batch * L * N;
     const int64_t edn = (int64_t)ED * N;
     const int64_t nbc = bln / V;  // threads of the dB/dC part
@@ -444,31 +451,51 @@ __global__ void __launch_bounds__(256) sscan_bwd_finish_kernel(
     } else if (i < bln + edn) {
         const int64_t j = i - bln;
         float s = 0.0f;
-        for (int bb = 0; bb < batch; ++bb) s += partA[bb * edn + j];
-        dA[j] = s;
+        for (int bb = 0; bb < rows; ++bb) s += partA[bb * edn + j];
+        dA[j] = *status ? __builtin_nanf("") : s;
     } else if (i < bln + edn + ED) {
         const int64_t j = i - bln - edn;
         float s = 0.0f, sdb = 0.0f;
-        for (int bb = 0; bb < batch; ++bb) {
+        for (int bb = 0; bb < rows; ++bb) {
             s += partD[(int64_t)bb * ED + j];
             if (dDb) sdb += partDb[(int64_t)bb * ED + j];
         }
-        dD[j] = s;
-        if (dDb) dDb[j] = sdb;
+        const bool failed = *status != 0;
+        dD[j] = failed ? __builtin_nanf("") : s;
+        if (dDb) dDb[j] = failed ? __builtin_nanf("") : sdb;
     }
 }
 
+// states per lane of the backward kernels (at most 4) and, for that choice, how a thin launch
+// is cut: half of the CUs or fewer covered (the first pass of a cut costs a quarter of the second)
+static constexpr int kBwdThin = 2;
+static int bwd_states_per_lane(const mpa_sscan_shape* s) {
+    const int ns = pick_states_per_lane(s->batch, s->dim, s->dstate, 4, s->plan_states_per_lane);
+    return ns < 0 ? 4 : ns;
+}
+// The cut exists on the fast kernel only, i.e. up to 16 states.
+static SegPlan bwd_seg_plan(const mpa_sscan_shape* s) {
+    const int ns = bwd_states_per_lane(s);
+    if (s->dstate > 16 || !bwd_fast_supported(ns, padded_states(s->dstate) / ns) ||
+        (s->plan_flags & MPA_PLAN_BWD_GENERAL))
+        return SegPlan{1, 0, 0, 0, 0, 0};
+    return seg_plan(s, ns, kBwdThin);
+}
+
 struct BwdWorkspace {
-    size_t offB, offC, offA, offD, offDb, total, group_stride;
+    size_t offB, offC, offA, offD, offDb, offStatus, offSeg, total, group_stride;
+    SegPlan seg;
 };
 
 static BwdWorkspace bwd_workspace(const mpa_sscan_shape* s) {
+    BwdWorkspace w;
+    w.seg = bwd_seg_plan(s);
+    const size_t rows = (size_t)s->batch * w.seg.nseg;
     const size_t cg = (size_t)(s->dim + kWave - 1) / kWave;
     const size_t bln = (size_t)s->batch * s->seqlen * s->dstate;
-    const size_t ben = (size_t)s->batch * s->dim * s->dstate;
-    const size_t be = (size_t)s->batch * s->dim;
+    const size_t ren = rows * s->dim * s->dstate;
+    const size_t re = rows * s->dim;
     auto up = [](size_t v) { return (v + 63) / 64 * 64; };  // 256-byte granules of floats
-    BwdWorkspace w;
     // The partial sums of the channel groups for one (batch, step, state) are written at the same
     // time by different workgroups and read together by the finish kernel.  batch*L*N floats is
     // often a power of two (1 MiB at the headline shape), which would put all of them on the same
@@ -477,11 +504,16 @@ static BwdWorkspace bwd_workspace(const mpa_sscan_shape* s) {
     w.offB = 0;
     w.offC = w.offB + cg * w.group_stride;
     w.offA = w.offC + cg * w.group_stride;
-    w.offD = w.offA + up(ben);
-    w.offDb = w.offD + up(be);
-    w.total = (w.offDb + up(be)) * sizeof(float);
+    w.offD = w.offA + up(ren);
+    w.offDb = w.offD + up(re);
+    w.offStatus = w.offDb + up(re);
+    w.offSeg = w.offStatus + 64;
+    w.total = (w.offSeg + up(w.seg.floats)) * sizeof(float);
     return w;
 }
+
+// one word set to zero without a memset node (a caller may be capturing a HIP graph)
+__global__ void clear_status_kernel(int* status) { *status = 0; }
 
 template <typename IO, int NS, int NW, bool HAS_Z>
 static int launch_bwd(const BwdParams& p, hipStream_t stream) {
@@ -525,7 +557,6 @@ extern "C" int mpa_sscan_bwd(const mpa_sscan_shape* s, const void* x, const void
                              void* stream) {
     int rc = validate_shape(s);
     if (rc != MPA_OK) return rc;
-    if (s->dstate > 64) return MPA_ERR_BAD_SHAPE;  // backward keeps <= 4 states per lane
     if (!x || !delta || !A || !B || !C || !D || !dy || !h_ckpt || !dx || !ddelta || !dA || !dB ||
         !dC || !dD || !workspace)
         return MPA_ERR_NULL_POINTER;
@@ -551,6 +582,10 @@ extern "C" int mpa_sscan_bwd(const mpa_sscan_shape* s, const void* x, const void
     p.partB = wsf + ws.offB; p.partC = wsf + ws.offC; p.partA = wsf + ws.offA;
     p.part_gs = (int64_t)ws.group_stride;
     p.partD = wsf + ws.offD; p.partDb = wsf + ws.offDb;
+    p.status = reinterpret_cast<int*>(wsf + ws.offStatus);
+    p.expire_waits = (s->plan_flags & MPA_PLAN_EXPIRE_WAITS) ? 1 : 0;
+    p.reverse = (s->flags & MPA_SSCAN_REVERSE) ? 1 : 0;
+    p.nseg = 1;
     p.batch = (int)s->batch; p.L = (int)s->seqlen; p.ED = (int)s->dim; p.N = (int)s->dstate;
     p.nchunks = (p.L + kTile - 1) / kTile;
     p.softplus = softplus ? 1 : 0;
@@ -564,12 +599,39 @@ extern "C" int mpa_sscan_bwd(const mpa_sscan_shape* s, const void* x, const void
     p.out_tmajor = (s->g_sd != 1 && s->g_sl == 1) ? 1 : 0;
 
     const int np = padded_states(s->dstate);
-    int ns = pick_states_per_lane(s->batch, s->dim, s->dstate, 4, "MPA_BWD_NS");
-    if (ns < 0) ns = 4;
+    const int ns = bwd_states_per_lane(s);
     const int nw = np / ns;
     hipStream_t st = static_cast<hipStream_t>(stream);
-    const char* force_general = getenv("MPA_BWD_GENERAL");
-    if ((!z || p.ypre) && bwd_fast_supported(ns, nw) && !(force_general && force_general[0] == '1')) {
+    hipLaunchKernelGGL(clear_status_kernel, dim3(1), dim3(1), 0, st, p.status);
+    const bool fast = (!z || p.ypre) && bwd_fast_supported(ns, nw) && !(s->plan_flags & MPA_PLAN_BWD_GENERAL);
+    int rows = p.batch;
+    if (fast) {
+        if (ws.seg.nseg > 1) {
+            // Sequence cut into segments that run side by side.  The reverse recurrence
+            // ag[t] = a[t] * (ag[t+1] + C[t]*dy[t]) is linear in its state like the forward one,
+            // so the forward kernel in its carry mode, walking against the forward direction,
+            // finds every segment's end value from zero and its sum of delta; seg_carry_kernel
+            // chains them into the value that flows into each segment.
+            float* seg = wsf + ws.offSeg;
+            FwdParams g{};
+            g.x = dy; g.delta = delta; g.z = z; g.A = A; g.D = D; g.dbias = delta_bias;
+            g.Bm = C; g.C = C; g.bc_sb = s->bc_sb; g.bc_sl = s->bc_sl;
+            g.hlast = seg + ws.seg.off_hend; g.dsum = seg + ws.seg.off_dsum;
+            g.nseg = ws.seg.nseg; g.seg_tiles = ws.seg.seg_tiles;
+            g.batch = p.batch; g.L = p.L; g.ED = p.ED; g.N = p.N; g.nchunks = p.nchunks;
+            g.softplus = p.softplus; g.reverse = p.reverse ? 0 : 1;
+            g.u_sb = s->y_sb; g.u_sl = s->y_sl; g.u_sd = s->y_sd;
+            g.z_sb = s->z_sb; g.z_sl = s->z_sl; g.z_sd = s->z_sd;
+            g.d_sb = s->d_sb; g.d_sl = s->d_sl; g.d_sd = s->d_sd;
+            g.in_tmajor = (s->d_sd != 1 && s->d_sl == 1) ? 1 : 0;
+            rc = launch_fwd_any(g, s->io_dtype, ns, nw, kGCarry, st);
+            if (rc != MPA_OK) return rc;
+            rc = launch_seg_carry(A, nullptr, seg + ws.seg.off_hend, seg + ws.seg.off_dsum, seg + ws.seg.off_h0,
+                                  nullptr, p.batch, ws.seg.nseg, p.ED, p.N, st);
+            if (rc != MPA_OK) return rc;
+            p.nseg = ws.seg.nseg; p.seg_tiles = ws.seg.seg_tiles; p.ag0 = seg + ws.seg.off_h0;
+            rows = p.batch * p.nseg;
+        }
         rc = launch_bwd_fast(p, ns, nw, s->io_dtype, st);
     } else if (s->io_dtype == MPA_F32)
         rc = z ? dispatch_bwd<float, true>(p, ns, nw, st) : dispatch_bwd<float, false>(p, ns, nw, st);
@@ -586,7 +648,7 @@ extern "C" int mpa_sscan_bwd(const mpa_sscan_shape* s, const void* x, const void
 #define MPA_FINISH(IO_, V_)                                                                                    \
     hipLaunchKernelGGL((sscan_bwd_finish_kernel<IO_, V_>), fgrid, dim3(256), 0, st, p.partB, p.partC, p.partA, \
                        p.partD, softplus && ddelta_bias ? p.partDb : nullptr, dB, dC, dA, dD, ddelta_bias, cg,  \
-                       p.part_gs, p.batch, p.L, p.ED, p.N, s->dbc_sb, s->dbc_sl)
+                       p.part_gs, p.batch, rows, p.L, p.ED, p.N, s->dbc_sb, s->dbc_sl, p.status)
     if (s->io_dtype == MPA_F32) {
         if (vec == 4) MPA_FINISH(float, 4);
         else MPA_FINISH(float, 1);

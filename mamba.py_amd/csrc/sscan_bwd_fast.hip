@@ -137,17 +137,30 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
 
     const int lane = threadIdx.x & (kWave - 1);
     const int w = wave_id();
-    const int b = blockIdx.y;
+    // Row of the launch: a batch row, or one segment of it.  Tiles of the row are counted from
+    // the end of the forward walk: tile k of the row is backward-walk tile k0 + k.
+    const int bs = blockIdx.y;
+    int b = bs, k0 = 0, ntiles = p.nchunks;
+    if (p.nseg > 1) {
+        b = bs / p.nseg;
+        k0 = (bs - b * p.nseg) * p.seg_tiles;
+        ntiles = min(p.seg_tiles, p.nchunks - k0);
+    }
     const int cg = blockIdx.x;
     const int d0 = cg * kWave;
-    const int ntiles = p.nchunks;
     const int cmax = min(kWave, p.ED - d0) - 1;  // last valid channel of the group
+    const bool rev = p.reverse != 0;
+    const int last_chunk = p.nchunks - 1;
+    const bool ragged_seq = p.nchunks * kTile > p.L;
     // dD / ddelta_bias partials [2][4][kWave]: written once at the very end, into the delta
     // buffer that no tile uses any more
     float* const sDD = sDl + (ntiles & 3) * kTileF;
 
-    // tile index k counts from the END of the sequence: tile k covers chunk c = ntiles-1-k
-    auto chunk_of = [&](int k) { return ntiles - 1 - k; };
+    // tile k of the row is walk tile c of the forward pass (the index of its checkpoint), which
+    // covers physical chunk c, or last_chunk - c when the forward walk ran in reverse; inside a
+    // tile walk step s is physical step s or kTile-1-s
+    auto chunk_of = [&](int k) { return last_chunk - (k0 + k); };
+    auto phys_of = [&](int c) { return rev ? last_chunk - c : c; };
 
     if (w >= NW) {
         // ================================ service waves ================================
@@ -161,18 +174,22 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
 
         // ---- input side: item -> (channel, step group), offsets that never change ----
         const int ci = p.in_tmajor ? item / NQ : item % kWave;
-        const int qi = p.in_tmajor ? item % NQ : item / kWave;
+        const int qi = p.in_tmajor ? item % NQ : item / kWave;  // walk step group of the item
+        // its physical step group (recomputed where it is used: not kept alive across the tiles)
+        auto qp_now = [&]() { return rev ? NQ - 1 - qi : qi; };
+        const int qp = qp_now();
+        auto jw = [&](int j) { return (uint32_t)(rev ? 3 - j : j); };  // walk step j of an item -> physical
         const bool ci_ok = ci <= cmax;
         const int cic = min(ci, cmax);
         const float bias = p.dbias ? p.dbias[d0 + cic] : 0.0f;
         IO* const dzg = static_cast<IO*>(p.dz) + (b * p.g_sb + (int64_t)d0 * p.g_sd);
-        // byte offset of the item's first step (one vector register per tensor); its other three
-        // steps are one row stride further each, which goes into the scalar offset of the access
-        const uint32_t offx = ((uint32_t)(4 * qi) * (uint32_t)p.u_sl + (uint32_t)cic * (uint32_t)p.u_sd) * kES;
-        const uint32_t offd = ((uint32_t)(4 * qi) * (uint32_t)p.d_sl + (uint32_t)cic * (uint32_t)p.d_sd) * kES;
-        const uint32_t offy = ((uint32_t)(4 * qi) * (uint32_t)p.y_sl + (uint32_t)cic * (uint32_t)p.y_sd) * kES;
-        const uint32_t offzi = ((uint32_t)(4 * qi) * (uint32_t)p.z_sl + (uint32_t)cic * (uint32_t)p.z_sd) * kES;
-        const uint32_t offz = ((uint32_t)(4 * qi) * (uint32_t)p.g_sl + (uint32_t)cic * (uint32_t)p.g_sd) * kES;  // dz
+        // byte offset of the item's lowest physical step (one vector register per tensor); walk
+        // step j of the item is jw(j) row strides further, which goes into the scalar offset
+        const uint32_t offx = ((uint32_t)(4 * qp) * (uint32_t)p.u_sl + (uint32_t)cic * (uint32_t)p.u_sd) * kES;
+        const uint32_t offd = ((uint32_t)(4 * qp) * (uint32_t)p.d_sl + (uint32_t)cic * (uint32_t)p.d_sd) * kES;
+        const uint32_t offy = ((uint32_t)(4 * qp) * (uint32_t)p.y_sl + (uint32_t)cic * (uint32_t)p.y_sd) * kES;
+        const uint32_t offzi = ((uint32_t)(4 * qp) * (uint32_t)p.z_sl + (uint32_t)cic * (uint32_t)p.z_sd) * kES;
+        const uint32_t offz = ((uint32_t)(4 * qp) * (uint32_t)p.g_sl + (uint32_t)cic * (uint32_t)p.g_sd) * kES;  // dz
         const uint32_t sx = (uint32_t)p.u_sl * kES, sd = (uint32_t)p.d_sl * kES, sy = (uint32_t)p.y_sl * kES;
         const uint32_t sz = (uint32_t)p.z_sl * kES, sg = (uint32_t)p.g_sl * kES;
         // tensor origins of this (batch row, channel group)
@@ -183,11 +200,10 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
         const IO* const ypb = static_cast<const IO*>(p.ypre) + (b * p.y_sb + (int64_t)d0 * p.y_sd);
         const IO* const Bb = static_cast<const IO*>(p.Bm) + b * p.bc_sb;
         const IO* const Cb = static_cast<const IO*>(p.C) + b * p.bc_sb;
-        // Loads of a ragged tile run past the sequence end.  That is harmless (the values are
-        // masked at staging) as long as the address is inside the tensor: the ragged tile is
+        // Loads of the ragged chunk run past the sequence end.  That is harmless (the values are
+        // masked at staging) as long as the address is inside the tensor: the ragged chunk is
         // read through windows that end with the tensor's last element, whatever the strides
         // (out-of-window loads return zero).
-        const bool ragged_end = ntiles * kTile > p.L;
         // B/C of a tile: kTile * NP elements each, kBcPer per service thread, step fastest
         constexpr int kBcPer = NP * kTile / (kSvc * kWave);
         static_assert(NP * kTile % (kSvc * kWave) == 0, "whole elements per thread");
@@ -196,17 +212,19 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
 #pragma unroll
         for (int r = 0; r < kBcPer; ++r) {
             const int e = item + r * (kSvc * kWave);
-            bct[r] = e % kTile;
+            bct[r] = e % kTile;  // walk step
             bcn[r] = e / kTile;
-            offbc[r] = ((uint32_t)bct[r] * (uint32_t)p.bc_sl + (uint32_t)min(bcn[r], p.N - 1)) * kES;
+            offbc[r] = ((uint32_t)(rev ? kTile - 1 - bct[r] : bct[r]) * (uint32_t)p.bc_sl +
+                        (uint32_t)min(bcn[r], p.N - 1)) * kES;
         }
 
         // ---- output side: item -> (channel, step group) ----
         const int co = p.out_tmajor ? item / NQ : item % kWave;
         const int qo = p.out_tmajor ? item % NQ : item / kWave;
+        const int qpo = rev ? NQ - 1 - qo : qo;
         const bool co_ok = co <= cmax;
         const float Dr = p.D[d0 + min(co, cmax)];
-        const uint32_t offg = ((uint32_t)(4 * qo) * (uint32_t)p.g_sl + (uint32_t)min(co, cmax) * (uint32_t)p.g_sd) * kES;
+        const uint32_t offg = ((uint32_t)(4 * qpo) * (uint32_t)p.g_sl + (uint32_t)min(co, cmax) * (uint32_t)p.g_sd) * kES;
         IO* const dxg = static_cast<IO*>(p.dx) + (b * p.g_sb + (int64_t)d0 * p.g_sd);
         IO* const ddg = static_cast<IO*>(p.ddelta) + (b * p.g_sb + (int64_t)d0 * p.g_sd);
         // dB/dC forwarding: kFw consecutive states of one (step, dB|dC) per thread
@@ -215,10 +233,11 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
         // (even service waves forward dB, odd ones dC, so that the destination is wave-uniform)
         const int fw_which = sw & 1;
         const int fw_i = ((sw >> 1) * kWave + lane) * kFw;  // index inside the [kTile][NP] half
-        const int fw_tt = fw_i / NP, fw_n = fw_i % NP;
+        const int fw_tt = fw_i / NP, fw_n = fw_i % NP;        // walk step, state
+        const int fw_tp = rev ? kTile - 1 - fw_tt : fw_tt;    // physical step inside the chunk
         const int fw_e = (fw_tt * 2 + fw_which) * NP + fw_n;  // index inside the dB|dC tile in LDS
         float* const fw_base = (fw_which ? p.partC : p.partB) + cg * p.part_gs + (int64_t)b * p.L * p.N;
-        const uint32_t fw_off = ((uint32_t)fw_tt * (uint32_t)p.N + (uint32_t)fw_n) * 4u;
+        const uint32_t fw_off = ((uint32_t)fw_tp * (uint32_t)p.N + (uint32_t)fw_n) * 4u;
         const bool fw_vec = p.N == NP;  // rows of the partial buffers are then aligned for vector stores
 
         float dDacc = 0.0f, dDb = 0.0f;
@@ -230,18 +249,18 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
             // tiles beyond the last one are clamped to it; steps beyond the sequence end are read
             // as whatever follows inside the tensor (or zero past its end) and masked at staging
             const int k = min(kk, ntiles - 1);
-            const int c = chunk_of(k);
-            const IO* xk = xb + (int64_t)c * kTile * p.u_sl;
-            const IO* dk = db + (int64_t)c * kTile * p.d_sl;
-            const IO* yk = yb + (int64_t)c * kTile * p.y_sl;
-            const IO* zk = zb + (int64_t)c * kTile * p.z_sl;
-            const IO* ypk = ypb + (int64_t)c * kTile * p.y_sl;
-            const IO* Bk = Bb + (int64_t)c * kTile * p.bc_sl;
-            const IO* Ck = Cb + (int64_t)c * kTile * p.bc_sl;
+            const int pc = phys_of(chunk_of(k));
+            const IO* xk = xb + (int64_t)pc * kTile * p.u_sl;
+            const IO* dk = db + (int64_t)pc * kTile * p.d_sl;
+            const IO* yk = yb + (int64_t)pc * kTile * p.y_sl;
+            const IO* zk = zb + (int64_t)pc * kTile * p.z_sl;
+            const IO* ypk = ypb + (int64_t)pc * kTile * p.y_sl;
+            const IO* Bk = Bb + (int64_t)pc * kTile * p.bc_sl;
+            const IO* Ck = Cb + (int64_t)pc * kTile * p.bc_sl;
             uint32_t wx = 0xffffffffu, wd = wx, wy = wx, wz = wx, wbc = wx;
-            if (ragged_end && c == ntiles - 1) {
-                // elements from this tile's origin to one past the tensor's last element
-                const int64_t tb = (int64_t)c * kTile;
+            if (ragged_seq && pc == last_chunk) {
+                // elements from this chunk's origin to one past the tensor's last element
+                const int64_t tb = (int64_t)pc * kTile;
                 auto left = [&](int64_t sb_, int64_t sl_, int64_t sd_, int64_t width) {
                     const int64_t end = (p.batch - 1) * sb_ + (p.L - 1) * sl_ + (width - 1) * sd_ + 1;
                     return window_bytes(end, b * sb_ + tb * sl_ + (int64_t)d0 * sd_, kES);
@@ -254,12 +273,12 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
             }
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                raw.x[j] = ld_off(xk, offx, j * sx, wx);
-                raw.d[j] = ld_off(dk, offd, j * sd, wd);
-                raw.y[j] = ld_off(yk, offy, j * sy, wy);
+                raw.x[j] = ld_off(xk, offx, jw(j) * sx, wx);
+                raw.d[j] = ld_off(dk, offd, jw(j) * sd, wd);
+                raw.y[j] = ld_off(yk, offy, jw(j) * sy, wy);
                 if constexpr (HAS_Z) {
-                    raw.z[j] = ld_off(zk, offzi, j * sz, wz);
-                    raw.yp[j] = ld_off(ypk, offy, j * sy, wy);
+                    raw.z[j] = ld_off(zk, offzi, jw(j) * sz, wz);
+                    raw.yp[j] = ld_off(ypk, offy, jw(j) * sy, wy);
                 }
             }
 #pragma unroll
@@ -269,7 +288,7 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
             }
         };
         auto stage_tile = [&](int k, const Raw& raw) {
-            const int c = chunk_of(k);
+            const int pc = phys_of(chunk_of(k));
             float xv[4], dv[4], yv[4];
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
@@ -292,25 +311,25 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
                     yv[j] *= zv * sg;
                 }
             }
-            const bool ragged = !group_full || (c + 1) * kTile > p.L;
+            const bool ragged = !group_full || (ragged_seq && pc == last_chunk);
             if constexpr (HAS_Z) {
-                IO* dzk = dzg + (int64_t)c * kTile * p.g_sl;
+                IO* dzk = dzg + (int64_t)pc * kTile * p.g_sl;
                 if (!ragged) {
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) st_off(dzk, offz, from_float<IO>(dzv[j]), j * sg);
+                    for (int j = 0; j < 4; ++j) st_off(dzk, offz, from_float<IO>(dzv[j]), jw(j) * sg);
                 } else {
-                    const int t0 = c * kTile + 4 * qi;
+                    const int t0 = pc * kTile + 4 * qp_now();
                     for (int j = 0; j < 4; ++j)
-                        if (ci_ok && t0 + j < p.L) st_off(dzk, offz, from_float<IO>(dzv[j]), j * sg);
+                        if (ci_ok && t0 + (int)jw(j) < p.L) st_off(dzk, offz, from_float<IO>(dzv[j]), jw(j) * sg);
                 }
             }
             if (ragged) {
                 // padding (beyond the sequence or the channel count): delta = 0, u = 0, dy = 0
                 // make the step an exact no-op in both sweeps
-                const int t0 = c * kTile + 4 * qi;
+                const int t0 = pc * kTile + 4 * qp_now();
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
-                    const bool ok = ci_ok && t0 + j < p.L;
+                    const bool ok = ci_ok && t0 + (int)jw(j) < p.L;
                     xv[j] = ok ? xv[j] : 0.0f;
                     dv[j] = ok ? dv[j] : 0.0f;
                     yv[j] = ok ? yv[j] : 0.0f;
@@ -333,7 +352,7 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
             }
         };
         auto reduce_tile = [&](int k) {
-            const int c = chunk_of(k);
+            const int pc = phys_of(chunk_of(k));
             float4 gB = make_float4(0.f, 0.f, 0.f, 0.f), dd = gB;
 #pragma unroll
             for (int ww = 0; ww < NW; ++ww) {
@@ -372,28 +391,29 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
                     dDb += dv[j];
                 }
             }
-            IO* dxk = dxg + (int64_t)c * kTile * p.g_sl;
-            IO* ddk = ddg + (int64_t)c * kTile * p.g_sl;
-            float* fwk = fw_base + (int64_t)c * kTile * p.N;
-            if (group_full && (c + 1) * kTile <= p.L && fw_vec) {
+            IO* dxk = dxg + (int64_t)pc * kTile * p.g_sl;
+            IO* ddk = ddg + (int64_t)pc * kTile * p.g_sl;
+            float* fwk = fw_base + (int64_t)pc * kTile * p.N;
+            if (group_full && !(ragged_seq && pc == last_chunk) && fw_vec) {
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
-                    st_off(dxk, offg, from_float<IO>(dxv[j]), j * sg);
-                    st_off(ddk, offg, from_float<IO>(dv[j]), j * sg);
+                    st_off(dxk, offg, from_float<IO>(dxv[j]), jw(j) * sg);
+                    st_off(ddk, offg, from_float<IO>(dv[j]), jw(j) * sg);
                 }
                 if constexpr (kFw == 2)
                     st_off(reinterpret_cast<float2*>(fwk), fw_off, make_float2(fw[0], fw[1]));
                 else
                     st_off(reinterpret_cast<float4*>(fwk), fw_off, make_float4(fw[0], fw[1], fw[2], fw[3]));
             } else {
-                const int t0 = c * kTile + 4 * qo;
+                const int t0 = pc * kTile + 4 * (rev ? NQ - 1 - qo : qo);
                 for (int j = 0; j < 4; ++j)
-                    if (co_ok && t0 + j < p.L) {
-                        st_off(dxk, offg, from_float<IO>(dxv[j]), j * sg);
-                        st_off(ddk, offg, from_float<IO>(dv[j]), j * sg);
+                    if (co_ok && t0 + (int)jw(j) < p.L) {
+                        st_off(dxk, offg, from_float<IO>(dxv[j]), jw(j) * sg);
+                        st_off(ddk, offg, from_float<IO>(dv[j]), jw(j) * sg);
                     }
                 for (int i = 0; i < kFw; ++i)
-                    if (c * kTile + fw_tt < p.L && fw_n + i < p.N) st_off(fwk, fw_off + 4u * i, fw[i]);
+                    if (pc * kTile + (rev ? kTile - 1 - fw_tt : fw_tt) < p.L && fw_n + i < p.N)
+                        st_off(fwk, fw_off + 4u * i, fw[i]);
             }
         };
 
@@ -438,8 +458,8 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
                 s += sDD[q * kWave + lane];
                 sb += sDD[(4 + q) * kWave + lane];
             }
-            p.partD[(int64_t)b * p.ED + d0 + lane] = s;
-            if (p.softplus) p.partDb[(int64_t)b * p.ED + d0 + lane] = sb;
+            p.partD[(int64_t)bs * p.ED + d0 + lane] = s;
+            if (p.softplus) p.partDb[(int64_t)bs * p.ED + d0 + lane] = sb;
         }
         return;
     }
@@ -453,8 +473,11 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
         const int n = w * NS + i;
         const int64_t dn = (int64_t)min(d, p.ED - 1) * p.N + min(n, p.N - 1);
         const float av = p.A[dn];
-        A2[i] = (dvalid && n < p.N) ? av * kLog2e : 0.0f;
-        ag[i] = 0.0f;
+        const bool ok = dvalid && n < p.N;
+        A2[i] = ok ? av * kLog2e : 0.0f;
+        // a*g flowing in from the steps after this row's last one (zero at the sequence end)
+        const float ag_in = p.ag0 ? p.ag0[(int64_t)bs * p.ED * p.N + dn] : 0.0f;
+        ag[i] = ok ? ag_in : 0.0f;
         dAacc[i] = 0.0f;
     }
     // state at the start of chunk c: checkpoint written after chunk c-1, or h0 / zero
@@ -462,7 +485,7 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
     auto load_state = [&](int k, float (&hs)[NS]) {
         const int c = chunk_of(min(k, ntiles - 1));
         const uint32_t ck_lane = (uint32_t)min(d0 + lane_now(), p.ED - 1);
-        const float* ck_base = p.ckpt + ((int64_t)b * ntiles + max(c - 1, 0)) * p.N * p.ED;
+        const float* ck_base = p.ckpt + ((int64_t)b * p.nchunks + max(c - 1, 0)) * p.N * p.ED;
         const float* h0_base = p.h0 ? p.h0 + (int64_t)b * p.ED * p.N : ck_base;
         const bool first = c == 0;
 #pragma unroll
@@ -625,14 +648,17 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
         });
         // The partial sums go to single-buffered LDS tiles.  The service waves read tile k-1 at
         // the start of this interval and publish that in sConsumed; by the end of the sweep
-        // that has normally happened, so this wait falls through (bounded: a wave never spins
-        // forever).
+        // that has normally happened, so this wait falls through.  It is bounded (a wave never
+        // spins forever); if the bound is ever reached the tiles may be overwritten while they
+        // are still being read, so the launch is marked as failed: the finish kernel then
+        // returns NaN gradients instead of silently wrong ones.
         if (k >= 1) {
             int spins = 0;
             while (consumed < kSvc * k && ++spins < (1 << 20)) {
                 __builtin_amdgcn_s_sleep(1);
                 consumed = __hip_atomic_load(sConsumed, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP);
             }
+            if ((consumed < kSvc * k || p.expire_waits) && lane_now() == 0) *p.status = 1;
         }
 #pragma unroll
         for (int q = 0; q < NQ; ++q) {
@@ -657,7 +683,7 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
 #pragma unroll
         for (int i = 0; i < NS; ++i) {
             const int n = w * NS + i;
-            if (n < p.N) p.partA[((int64_t)b * p.ED + d) * p.N + n] = dAacc[i];
+            if (n < p.N) p.partA[((int64_t)bs * p.ED + d) * p.N + n] = dAacc[i];
         }
     }
     __syncthreads();  // final
@@ -665,7 +691,7 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
 
 template <typename IO, int NS, int NW, bool HAS_Z>
 static int launch_fast(const BwdParams& p, hipStream_t stream) {
-    dim3 grid((p.ED + kWave - 1) / kWave, p.batch);
+    dim3 grid((p.ED + kWave - 1) / kWave, p.batch * (p.nseg > 1 ? p.nseg : 1));
     dim3 block((NW + kSvc) * kWave);
     constexpr size_t lds = sizeof(float) * BwdFastLds<NS, NW>::floats;
     static_assert(lds <= 160 * 1024, "LDS budget");

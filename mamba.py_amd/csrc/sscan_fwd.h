@@ -1,0 +1,67 @@
+// Parameters and launchers of the forward kernel of the fused selective scan, shared with the
+// backward entry point (which runs the same kernel in a carry mode when it cuts the sequence).
+#pragma once
+
+#include "common.h"
+
+namespace mpa {
+
+struct FwdParams {
+    const void* x;
+    const void* delta;
+    const void* z;
+    const float* A;
+    const float* D;
+    const float* dbias;
+    const float* h0;
+    const float* bcpack;  // packed B/C, see pack_bc_kernel (only at 16 or more states per lane)
+    const void* Bm;
+    const void* C;
+    int64_t bc_sb, bc_sl;
+    void* y;
+    void* ypre;  // output before the gate (only with z), strides of y
+    float* ckpt;
+    float* hlast;
+    float* dsum;     // segmented mode, first pass: sums of delta per (row, step group, channel)
+    int nseg;        // > 1: every batch row is cut into nseg segments of seg_tiles tiles, one
+    int seg_tiles;   // workgroup row (blockIdx.y) per (batch row, segment)
+    int batch, L, ED, N, nchunks;
+    int softplus;
+    int reverse;     // the walk runs from the last physical step to the first
+    int in_tmajor;   // x / delta have unit stride along time
+    int out_tmajor;  // y has unit stride along time
+    int64_t u_sb, u_sl, u_sd;
+    int64_t z_sb, z_sl, z_sd;
+    int64_t d_sb, d_sl, d_sd;
+    int64_t y_sb, y_sl, y_sd;
+};
+
+// What one launch of the kernel computes.
+//   kScan    the selective scan: states, readout y, optional checkpoints and last state.
+//   kCarry   states only (no readout, no reducer waves): the end state of every segment from a
+//            zero state, and its sum of delta, for seg_carry_kernel.
+//   kGCarry  the carry of the BACKWARD recurrence, g[t] = dy[t]*C[t] + a[t+1]*g[t+1], in the
+//            form ag[t] = a[t]*(ag[t+1] + C[t]*dy[t]): the same kernel walking the other way
+//            with dy (times silu(z) when gated) in place of delta*x, C in place of B and the
+//            decay applied after the addition.
+enum FwdMode { kScan = 0, kCarry = 1, kGCarry = 2 };
+
+// A sequence cut into nseg segments of seg_tiles tiles (the last one may be shorter), and where
+// the per-segment buffers sit in the workspace (offsets in floats): end states from zero
+// [rows][dim][dstate], true initial states (same shape), sums of delta [rows][4][dim];
+// rows = batch * nseg.  nseg = 1: not cut, no buffers.
+struct SegPlan {
+    int nseg, seg_tiles;
+    size_t off_hend, off_h0, off_dsum, floats;
+};
+SegPlan seg_plan(const mpa_sscan_shape* s, int ns, int thin);
+
+// Launch sscan_fwd_kernel in `mode` (FwdMode) for the (ns, nw) decomposition; the carry modes
+// exist for ns <= 8.
+int launch_fwd_any(const FwdParams& p, int io_dtype, int ns, int nw, int mode, hipStream_t stream);
+// segh0[row] = state at the start of every segment, from the end states and delta sums of the
+// first pass; hlast (optional) = state after the last segment.
+int launch_seg_carry(const float* A, const float* h0, const float* hend, const float* dsum, float* segh0,
+                     float* hlast, int batch, int nseg, int ED, int N, hipStream_t st);
+
+}  // namespace mpa

@@ -22,57 +22,33 @@
 //    a small pre-pass packs them as float32 in the order each scan wave consumes them and the
 //    scan waves fetch them with scalar loads into SGPRs.
 //  * The only parallel axes are batch * dim/64 workgroups and the states inside them.  When a
-//    launch without checkpoints (inference) would cover a fraction of the chip, the sequence is
-//    cut into segments that run side by side: a first pass finds every segment's end state from
-//    zero and its sum of delta, seg_carry_kernel chains them, a second pass is the normal
-//    kernel from the true initial states (see seg_plan).
+//    launch would cover a fraction of the chip, the sequence is cut into segments that run side
+//    by side: a first pass (kernel mode kCarry: no readout) finds every segment's end state
+//    from zero and its sum of delta, seg_carry_kernel chains them, a second pass is the normal
+//    kernel from the true initial states (see seg_plan).  The backward uses the same first pass
+//    for its own carry (mode kGCarry, see sscan_bwd.hip).
+//  * Time is addressed through one mapping, walk position -> physical step, so that the scan
+//    can run from the last step to the first (MPA_SSCAN_REVERSE) without flipped copies: the
+//    service waves stage every tile in walk order and the scan waves never see the direction.
 //  * Both channel-contiguous and time-contiguous ((B,ED,L) memory) operands are read and
 //    written coalesced: a service thread owns 4 consecutive steps of one channel, and the
 //    thread -> (channel, step group) map follows the unit-stride axis.
-#include "common.h"
+#include "sscan_fwd.h"
 
 namespace mpa {
 
-struct FwdParams {
-    const void* x;
-    const void* delta;
-    const void* z;
-    const float* A;
-    const float* D;
-    const float* dbias;
-    const float* h0;
-    const float* bcpack;  // packed B/C, see pack_bc_kernel (only at 16 or more states per lane)
-    const void* Bm;
-    const void* C;
-    int64_t bc_sb, bc_sl;
-    void* y;
-    void* ypre;  // output before the gate (only with z), strides of y
-    float* ckpt;
-    float* hlast;
-    float* dsum;     // segmented mode, first pass: sums of delta per (row, step group, channel)
-    int nseg;        // > 1: every batch row is cut into nseg segments of seg_tiles tiles, one
-    int seg_tiles;   // workgroup row (blockIdx.y) per (batch row, segment)
-    int batch, L, ED, N, nchunks;
-    int softplus;
-    int in_tmajor;   // x / delta have unit stride along time
-    int out_tmajor;  // y has unit stride along time
-    int64_t u_sb, u_sl, u_sd;
-    int64_t z_sb, z_sl, z_sd;
-    int64_t d_sb, d_sl, d_sd;
-    int64_t y_sb, y_sl, y_sd;
-};
 
 // ---------------------------------------------------------------------------------------------
 // B/C pre-pass.  Output layout, float32:
 //     [batch][tile][wave][sub-tile][B | C][kSS steps][NS states]
 // i.e. the values one scan wave needs for one sub-tile of kSS steps are contiguous (the scan
-// waves fetch them one sub-tile ahead of use).  Steps beyond the sequence end and states
-// beyond d_state are written as zeros.
+// waves fetch them one sub-tile ahead of use); tiles and steps are in walk order.  Steps beyond
+// the sequence end and states beyond d_state are written as zeros.
 // ---------------------------------------------------------------------------------------------
 template <typename IO>
 __global__ void __launch_bounds__(256) pack_bc_kernel(const void* Bm, const void* C, float* out,
                                                       int L, int N, int NS, int NW, int kSS,
-                                                      int nchunks, int64_t bc_sb, int64_t bc_sl) {
+                                                      int nchunks, int reverse, int64_t bc_sb, int64_t bc_sl) {
     const int NP = NS * NW;
     const int64_t per_b = (int64_t)nchunks * 2 * kTile * NP;
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -88,7 +64,9 @@ __global__ void __launch_bounds__(256) pack_bc_kernel(const void* Bm, const void
     const int which = r / (kSS * NS);
     r %= kSS * NS;
     const int tt = sub * kSS + r / NS, s = r % NS;
-    const int t = c * kTile + tt, n = w * NS + s;
+    // (c, tt) count tiles and steps in walk order; a reverse walk starts at the physical end
+    const int t = reverse ? (nchunks - 1 - c) * kTile + (kTile - 1 - tt) : c * kTile + tt;
+    const int n = w * NS + s;
     float v = 0.0f;
     if (t < L && n < N)
         v = load_as_float<IO>(which ? C : Bm, b * bc_sb + (int64_t)t * bc_sl + n);
@@ -128,34 +106,43 @@ struct FwdLds {
     static constexpr size_t floats = tiles + (kBcastBC<NS> ? 2 * 2 * NS * NW * kTile : 0);
 };
 
+
 // One scan step / one group of four steps on the broadcast path: B and C of step TT come out of
 // lane TT of the registers vb[i] / vc[i] inside the FMA (fmac_bcast).
-template <int TT, int NS>
+template <int TT, int NS, int MODE>
 __device__ __forceinline__ float scan_step_bcast(float dlv, float uuv, const float (&A2)[NS], float (&h)[NS],
                                                  const float (&vb)[NS], const float (&vc)[NS]) {
-    float sum;
+    float sum = 0.0f;
 #pragma unroll
     for (int i = 0; i < NS; ++i) {
         const float a = fast_exp2(dlv * A2[i]);
-        h[i] = fmac_bcast<TT>(a * h[i], vb[i], uuv);
-        sum = i == 0 ? mul_bcast<TT>(vc[i], h[i]) : fmac_bcast<TT>(sum, vc[i], h[i]);
+        if constexpr (MODE == kGCarry) {
+            h[i] = a * fmac_bcast<TT>(h[i], vb[i], uuv);
+        } else {
+            h[i] = fmac_bcast<TT>(a * h[i], vb[i], uuv);
+        }
+        if constexpr (MODE == kScan) sum = i == 0 ? mul_bcast<TT>(vc[i], h[i]) : fmac_bcast<TT>(sum, vc[i], h[i]);
     }
     return sum;
 }
-template <int Q, int NS>
+template <int Q, int NS, int MODE>
 __device__ __forceinline__ float4 scan_group_bcast(const float (&dl)[kTile], const float (&uu)[kTile],
                                                    const float (&A2)[NS], float (&h)[NS],
                                                    const float (&vb)[NS], const float (&vc)[NS]) {
     float4 y;
-    y.x = scan_step_bcast<4 * Q + 0, NS>(dl[4 * Q + 0], uu[4 * Q + 0], A2, h, vb, vc);
-    y.y = scan_step_bcast<4 * Q + 1, NS>(dl[4 * Q + 1], uu[4 * Q + 1], A2, h, vb, vc);
-    y.z = scan_step_bcast<4 * Q + 2, NS>(dl[4 * Q + 2], uu[4 * Q + 2], A2, h, vb, vc);
-    y.w = scan_step_bcast<4 * Q + 3, NS>(dl[4 * Q + 3], uu[4 * Q + 3], A2, h, vb, vc);
+    y.x = scan_step_bcast<4 * Q + 0, NS, MODE>(dl[4 * Q + 0], uu[4 * Q + 0], A2, h, vb, vc);
+    y.y = scan_step_bcast<4 * Q + 1, NS, MODE>(dl[4 * Q + 1], uu[4 * Q + 1], A2, h, vb, vc);
+    y.z = scan_step_bcast<4 * Q + 2, NS, MODE>(dl[4 * Q + 2], uu[4 * Q + 2], A2, h, vb, vc);
+    y.w = scan_step_bcast<4 * Q + 3, NS, MODE>(dl[4 * Q + 3], uu[4 * Q + 3], A2, h, vb, vc);
     return y;
 }
 
-template <typename IO, int NS, int NW, bool HAS_Z>
-__global__ void __launch_bounds__((NW + kService) * kWave) sscan_fwd_kernel(const FwdParams p) {
+// waves of a workgroup: the carry modes store no output and run without reducer waves
+template <int NW, int MODE>
+constexpr int kFwdWaves = NW + (MODE == kScan ? kService : kLoaders);
+
+template <typename IO, int NS, int NW, bool HAS_Z, int MODE>
+__global__ void __launch_bounds__((kFwdWaves<NW, MODE>) * kWave) sscan_fwd_kernel(const FwdParams p) {
     constexpr int NQ = kTile / 4;  // step groups (of 4) per tile
     static_assert(kLoaders == NQ && kReducers == NQ, "a tile has 64 * NQ items of (channel, 4 steps)");
 
@@ -169,11 +156,13 @@ __global__ void __launch_bounds__((NW + kService) * kWave) sscan_fwd_kernel(cons
     float* const sBC = reinterpret_cast<float*>(sY + 2 * NW);  // [2][B|C][NP states][kTile steps]
     constexpr int NP = NS * NW;
     constexpr bool kBcast = kBcastBC<NS>;
+    static_assert(MODE == kScan || kBcast, "the carry modes exist on the broadcast path only");
 
     const int lane = threadIdx.x & (kWave - 1);
     const int w = wave_id();
     // Row of the launch: a batch row, or one segment of it (segmented mode).  h0 / h_last / dsum
-    // are indexed by the launch row, the caller's tensors by (batch row, first step of the row).
+    // are indexed by the launch row, the caller's tensors by (batch row, physical step).
+    // Tiles are counted in WALK order: walk tile kk is the kk-th tile the recurrence visits.
     const int bs = blockIdx.y;
     int b = bs, tile0 = 0, ntiles = p.nchunks;
     if (p.nseg > 1) {
@@ -181,8 +170,13 @@ __global__ void __launch_bounds__((NW + kService) * kWave) sscan_fwd_kernel(cons
         tile0 = (bs - b * p.nseg) * p.seg_tiles;
         ntiles = min(p.seg_tiles, p.nchunks - tile0);
     }
-    const int tbase = tile0 * kTile;               // first step of the row
-    const int Lrow = min(p.L - tbase, ntiles * kTile);  // steps of the row
+    // walk tile -> physical chunk of kTile steps; inside a tile walk step s is physical step
+    // s (forward) or kTile-1-s (reverse).  The ragged chunk is always the physical last one, so a
+    // reverse walk starts with its padded steps: delta = 0 and u = 0 there leave the state alone.
+    const bool rev = p.reverse != 0;
+    const int last_chunk = p.nchunks - 1;
+    auto phys_chunk = [&](int k) { return rev ? last_chunk - (tile0 + k) : tile0 + k; };
+    const bool ragged_seq = p.nchunks * kTile > p.L;
     const int d0 = blockIdx.x * kWave;
     constexpr bool has_z = HAS_Z;
 
@@ -206,43 +200,45 @@ __global__ void __launch_bounds__((NW + kService) * kWave) sscan_fwd_kernel(cons
         if (sw < kLoaders) {
             // ------------------------------- loaders -------------------------------
             const int ci = p.in_tmajor ? item / NQ : item % kWave;
-            const int qi = p.in_tmajor ? item % NQ : item / kWave;
+            const int qi = p.in_tmajor ? item % NQ : item / kWave;  // walk step group of the item
+            const int qp = rev ? NQ - 1 - qi : qi;                  // its physical step group
             const bool ci_ok = ci <= cmax;
             const int cic = min(ci, cmax);
             const float Dv = p.D[d0 + cic];
             const float bias = p.dbias ? p.dbias[d0 + cic] : 0.0f;
-            // wave-uniform tile origins (scalar registers) + per-thread 32-bit element
-            // offsets that do not change from tile to tile: one global_load per element and no
+            // wave-uniform chunk origins (scalar registers) + per-thread 32-bit element
+            // offsets that do not change from tile to tile: one load per element and no
             // address arithmetic in the loop
-            const IO* const xg = static_cast<const IO*>(p.x) + (b * p.u_sb + tbase * p.u_sl + (int64_t)d0 * p.u_sd);
-            const IO* const dg = static_cast<const IO*>(p.delta) + (b * p.d_sb + tbase * p.d_sl + (int64_t)d0 * p.d_sd);
-            const IO* const zg = static_cast<const IO*>(p.z) + (b * p.z_sb + tbase * p.z_sl + (int64_t)d0 * p.z_sd);
-            // byte offset of the item's first step (one vector register per tensor, see ld_off);
-            // its other three steps are one row stride further each, which goes into the scalar
-            // offset of the access
-            const uint32_t offx = ((uint32_t)(4 * qi) * (uint32_t)p.u_sl + (uint32_t)cic * (uint32_t)p.u_sd) * kES;
-            const uint32_t offd = ((uint32_t)(4 * qi) * (uint32_t)p.d_sl + (uint32_t)cic * (uint32_t)p.d_sd) * kES;
-            const uint32_t offz = ((uint32_t)(4 * qi) * (uint32_t)p.z_sl + (uint32_t)cic * (uint32_t)p.z_sd) * kES;
+            const IO* const xg = static_cast<const IO*>(p.x) + (b * p.u_sb + (int64_t)d0 * p.u_sd);
+            const IO* const dg = static_cast<const IO*>(p.delta) + (b * p.d_sb + (int64_t)d0 * p.d_sd);
+            const IO* const zg = static_cast<const IO*>(p.z) + (b * p.z_sb + (int64_t)d0 * p.z_sd);
+            // byte offset of the item's lowest physical step (one vector register per tensor, see
+            // ld_off); walk step j of the item is jw(j) row strides further, which goes into the
+            // scalar offset of the access
+            const uint32_t offx = ((uint32_t)(4 * qp) * (uint32_t)p.u_sl + (uint32_t)cic * (uint32_t)p.u_sd) * kES;
+            const uint32_t offd = ((uint32_t)(4 * qp) * (uint32_t)p.d_sl + (uint32_t)cic * (uint32_t)p.d_sd) * kES;
+            const uint32_t offz = ((uint32_t)(4 * qp) * (uint32_t)p.z_sl + (uint32_t)cic * (uint32_t)p.z_sd) * kES;
             const uint32_t sx = (uint32_t)p.u_sl * kES, sd = (uint32_t)p.d_sl * kES, sz = (uint32_t)p.z_sl * kES;
-            // Loads of a ragged tile run past the sequence end.  That is harmless (the values
+            auto jw = [&](int j) { return (uint32_t)(rev ? 3 - j : j); };
+            // Loads of the ragged chunk run past the sequence end.  That is harmless (the values
             // are masked at staging) as long as the address is inside the tensor: the ragged
-            // tile is read through windows that end with the tensor's last element, whatever
+            // chunk is read through windows that end with the tensor's last element, whatever
             // the strides (out-of-window loads return zero).
-            const bool ragged_end = ntiles * kTile > Lrow;
             const bool group_full = cmax == kWave - 1;
             // B/C of a tile: kTile * NP elements each, kBcPer per loader thread, step fastest
             constexpr int kBcPer = kBcast ? NP * kTile / (kLoaders * kWave) : 0;
             static_assert(!kBcast || NP * kTile % (kLoaders * kWave) == 0, "whole elements per thread");
-            const IO* const Bg = static_cast<const IO*>(p.Bm) + (b * p.bc_sb + tbase * p.bc_sl);
-            const IO* const Cg = static_cast<const IO*>(p.C) + (b * p.bc_sb + tbase * p.bc_sl);
+            const IO* const Bg = static_cast<const IO*>(p.Bm) + b * p.bc_sb;
+            const IO* const Cg = static_cast<const IO*>(p.C) + b * p.bc_sb;
             int bct[kBcPer > 0 ? kBcPer : 1], bcn[kBcPer > 0 ? kBcPer : 1];
             uint32_t offbc[kBcPer > 0 ? kBcPer : 1];
 #pragma unroll
             for (int r = 0; r < kBcPer; ++r) {
                 const int e = item + r * (kLoaders * kWave);
-                bct[r] = e % kTile;
+                bct[r] = e % kTile;  // walk step
                 bcn[r] = e / kTile;
-                offbc[r] = ((uint32_t)bct[r] * (uint32_t)p.bc_sl + (uint32_t)min(bcn[r], p.N - 1)) * kES;
+                offbc[r] = ((uint32_t)(rev ? kTile - 1 - bct[r] : bct[r]) * (uint32_t)p.bc_sl +
+                            (uint32_t)min(bcn[r], p.N - 1)) * kES;
             }
 
             // Raw values of three tiles in flight: HBM latency under load is longer than one
@@ -262,15 +258,16 @@ __global__ void __launch_bounds__((NW + kService) * kWave) sscan_fwd_kernel(cons
                 // tiles beyond the last one are clamped to it; the loads are unconditional (a
                 // branch around them would force a wait on their data)
                 const int k = min(kk, ntiles - 1);
-                const IO* xk = xg + (int64_t)k * kTile * p.u_sl;
-                const IO* dk = dg + (int64_t)k * kTile * p.d_sl;
-                const IO* zk = zg + (int64_t)k * kTile * p.z_sl;
-                const IO* Bk = Bg + (int64_t)k * kTile * p.bc_sl;
-                const IO* Ck = Cg + (int64_t)k * kTile * p.bc_sl;
+                const int pc = phys_chunk(k);
+                const IO* xk = xg + (int64_t)pc * kTile * p.u_sl;
+                const IO* dk = dg + (int64_t)pc * kTile * p.d_sl;
+                const IO* zk = zg + (int64_t)pc * kTile * p.z_sl;
+                const IO* Bk = Bg + (int64_t)pc * kTile * p.bc_sl;
+                const IO* Ck = Cg + (int64_t)pc * kTile * p.bc_sl;
                 uint32_t wx = 0xffffffffu, wd = wx, wz = wx, wbc = wx;
-                if (ragged_end && k == ntiles - 1) {
-                    // elements from this tile's origin to one past the tensor's last element
-                    const int64_t tb = (int64_t)k * kTile + tbase;
+                if (ragged_seq && pc == last_chunk) {
+                    // elements from this chunk's origin to one past the tensor's last element
+                    const int64_t tb = (int64_t)pc * kTile;
                     auto left = [&](int64_t sb_, int64_t sl_, int64_t sd_, int64_t width) {
                         const int64_t end = (p.batch - 1) * sb_ + (p.L - 1) * sl_ + (width - 1) * sd_ + 1;
                         return window_bytes(end, b * sb_ + tb * sl_ + (int64_t)d0 * sd_, kES);
@@ -282,14 +279,14 @@ __global__ void __launch_bounds__((NW + kService) * kWave) sscan_fwd_kernel(cons
                 }
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
-                    raw.x[j] = ld_off(xk, offx, j * sx, wx);
-                    raw.d[j] = ld_off(dk, offd, j * sd, wd);
-                    if (has_z) raw.z[j] = ld_off(zk, offz, j * sz, wz);
+                    raw.x[j] = ld_off(xk, offx, jw(j) * sx, wx);
+                    raw.d[j] = ld_off(dk, offd, jw(j) * sd, wd);
+                    if (has_z) raw.z[j] = ld_off(zk, offz, jw(j) * sz, wz);
                 }
 #pragma unroll
                 for (int r = 0; r < kBcPer; ++r) {
                     raw.b[r] = ld_off(Bk, offbc[r], 0, wbc);
-                    raw.c[r] = ld_off(Ck, offbc[r], 0, wbc);
+                    if constexpr (MODE == kScan) raw.c[r] = ld_off(Ck, offbc[r], 0, wbc);
                 }
                 if (!kBcast) raw.warm = warm[(int64_t)k * kPackVec];
             };
@@ -302,7 +299,7 @@ __global__ void __launch_bounds__((NW + kService) * kWave) sscan_fwd_kernel(cons
                     const bool ok = bcn[r] < p.N;
                     float* dst = sBC + (k & 1) * (2 * NP * kTile) + bcn[r] * kTile + bct[r];
                     dst[0] = ok ? to_float(raw.b[r]) : 0.0f;
-                    dst[NP * kTile] = ok ? to_float(raw.c[r]) : 0.0f;
+                    if constexpr (MODE == kScan) dst[NP * kTile] = ok ? to_float(raw.c[r]) : 0.0f;
                 }
                 float xv[4], dv[4], gg[4];
 #pragma unroll
@@ -314,12 +311,13 @@ __global__ void __launch_bounds__((NW + kService) * kWave) sscan_fwd_kernel(cons
 #pragma unroll
                     for (int j = 0; j < 4; ++j) dv[j] = softplus_f(dv[j] + bias);
                 }
-                if (!group_full || (k + 1) * kTile > Lrow) {
+                const int pc = phys_chunk(k);
+                if (!group_full || (ragged_seq && pc == last_chunk)) {
                     // ragged edge: delta = 0, u = 0 keeps the state of padded steps/channels
-                    const int t0 = k * kTile + 4 * qi;
+                    const int t0 = pc * kTile + 4 * qp;
 #pragma unroll
                     for (int j = 0; j < 4; ++j) {
-                        const bool ok = ci_ok && t0 + j < Lrow;
+                        const bool ok = ci_ok && t0 + (int)jw(j) < p.L;
                         xv[j] = ok ? xv[j] : 0.0f;
                         dv[j] = ok ? dv[j] : 0.0f;
                     }
@@ -327,17 +325,28 @@ __global__ void __launch_bounds__((NW + kService) * kWave) sscan_fwd_kernel(cons
                 dsum += (dv[0] + dv[1]) + (dv[2] + dv[3]);
                 const int q4 = 4 * qi;
                 *reinterpret_cast<float4*>(&sDl[k & 1][ci][q4]) = make_float4(dv[0], dv[1], dv[2], dv[3]);
-                *reinterpret_cast<float4*>(&sU[k & 1][ci][q4]) =
-                    make_float4(dv[0] * xv[0], dv[1] * xv[1], dv[2] * xv[2], dv[3] * xv[3]);
-                *reinterpret_cast<float4*>(&sDx[k & 3][ci][q4]) =
-                    make_float4(Dv * xv[0], Dv * xv[1], Dv * xv[2], Dv * xv[3]);
                 if (has_z) {
 #pragma unroll
                     for (int j = 0; j < 4; ++j) {
                         const float zv = to_float(raw.z[j]);
                         gg[j] = zv * sigmoid_f(zv);
                     }
-                    *reinterpret_cast<float4*>(&sG[k & 3][ci][q4]) = make_float4(gg[0], gg[1], gg[2], gg[3]);
+                }
+                if constexpr (MODE == kGCarry) {
+                    // `x` is the upstream gradient dy here; the recurrence sees dy * silu(z)
+                    if (has_z) {
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) xv[j] *= gg[j];
+                    }
+                    *reinterpret_cast<float4*>(&sU[k & 1][ci][q4]) = make_float4(xv[0], xv[1], xv[2], xv[3]);
+                } else {
+                    *reinterpret_cast<float4*>(&sU[k & 1][ci][q4]) =
+                        make_float4(dv[0] * xv[0], dv[1] * xv[1], dv[2] * xv[2], dv[3] * xv[3]);
+                }
+                if constexpr (MODE == kScan) {
+                    *reinterpret_cast<float4*>(&sDx[k & 3][ci][q4]) =
+                        make_float4(Dv * xv[0], Dv * xv[1], Dv * xv[2], Dv * xv[3]);
+                    if (has_z) *reinterpret_cast<float4*>(&sG[k & 3][ci][q4]) = make_float4(gg[0], gg[1], gg[2], gg[3]);
                 }
             };
             // tile j travels in register set j % 3; staging runs two tiles ahead of the scan
@@ -365,43 +374,46 @@ __global__ void __launch_bounds__((NW + kService) * kWave) sscan_fwd_kernel(cons
                 __syncthreads();
             }
             if (p.dsum && ci_ok) p.dsum[((int64_t)bs * NQ + qi) * p.ED + d0 + ci] = dsum;
-        } else {
+        } else if constexpr (MODE == kScan) {
             // ------------------------------- reducers -------------------------------
             const int co = p.out_tmajor ? item / NQ : item % kWave;
-            const int qo = p.out_tmajor ? item % NQ : item / kWave;
+            const int qo = p.out_tmajor ? item % NQ : item / kWave;  // walk step group
+            const int qpo = rev ? NQ - 1 - qo : qo;                  // physical step group
             const bool co_ok = co <= cmax;
             const int q4 = 4 * qo;
-            const uint32_t offy = ((uint32_t)q4 * (uint32_t)p.y_sl + (uint32_t)min(co, cmax) * (uint32_t)p.y_sd) * kES;
+            const uint32_t offy = ((uint32_t)(4 * qpo) * (uint32_t)p.y_sl + (uint32_t)min(co, cmax) * (uint32_t)p.y_sd) * kES;
             const uint32_t sy = (uint32_t)p.y_sl * kES;
-            IO* const yg = static_cast<IO*>(p.y) + (b * p.y_sb + tbase * p.y_sl + (int64_t)d0 * p.y_sd);
-            IO* const ypg = static_cast<IO*>(p.ypre) + (b * p.y_sb + tbase * p.y_sl + (int64_t)d0 * p.y_sd);
+            auto jw = [&](int j) { return (uint32_t)(rev ? 3 - j : j); };
+            IO* const yg = static_cast<IO*>(p.y) + (b * p.y_sb + (int64_t)d0 * p.y_sd);
+            IO* const ypg = static_cast<IO*>(p.ypre) + (b * p.y_sb + (int64_t)d0 * p.y_sd);
             auto reduce_store = [&](int k) {
-                if (!p.y) return;  // first pass of the segmented mode: only the end states count
-                IO* yk = yg + (int64_t)k * kTile * p.y_sl;
-                IO* ypk = ypg + (int64_t)k * kTile * p.y_sl;
+                const int pc = phys_chunk(k);
+                IO* yk = yg + (int64_t)pc * kTile * p.y_sl;
+                IO* ypk = ypg + (int64_t)pc * kTile * p.y_sl;
                 float4 s = *reinterpret_cast<const float4*>(&sDx[k & 3][co][q4]);
 #pragma unroll
                 for (int ww = 0; ww < NW; ++ww) {
                     const float4 v = *reinterpret_cast<const float4*>(&sY[(k & 1) * NW + ww][co][q4]);
                     s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
                 }
-                const int t0 = k * kTile + q4;
+                const int t0 = pc * kTile + 4 * qpo;  // lowest physical step of the item
+                const bool whole = !(ragged_seq && pc == last_chunk) || t0 + 3 < p.L;
                 if (has_z) {
                     if (p.ypre) {
                         const float pv[4] = {s.x, s.y, s.z, s.w};
                         for (int j = 0; j < 4; ++j)
-                            if (co_ok && t0 + j < Lrow) st_off(ypk, offy, from_float<IO>(pv[j]), j * sy);
+                            if (co_ok && t0 + (int)jw(j) < p.L) st_off(ypk, offy, from_float<IO>(pv[j]), jw(j) * sy);
                     }
                     const float4 g = *reinterpret_cast<const float4*>(&sG[k & 3][co][q4]);
                     s.x *= g.x; s.y *= g.y; s.z *= g.z; s.w *= g.w;
                 }
                 const float sv[4] = {s.x, s.y, s.z, s.w};
-                if (co_ok && t0 + 3 < Lrow) {
+                if (co_ok && whole) {
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) st_off(yk, offy, from_float<IO>(sv[j]), j * sy);
+                    for (int j = 0; j < 4; ++j) st_off(yk, offy, from_float<IO>(sv[j]), jw(j) * sy);
                 } else if (co_ok) {
                     for (int j = 0; j < 4; ++j)
-                        if (t0 + j < Lrow) st_off(yk, offy, from_float<IO>(sv[j]), j * sy);
+                        if (t0 + (int)jw(j) < p.L) st_off(yk, offy, from_float<IO>(sv[j]), jw(j) * sy);
                 }
             };
             // the reducers run one tile behind the scan waves
@@ -449,16 +461,18 @@ __global__ void __launch_bounds__((NW + kService) * kWave) sscan_fwd_kernel(cons
 #pragma unroll
             for (int i = 0; i < NS; ++i) {
                 r.vb[i] = bck[i * kTile];
-                r.vc[i] = bck[NP * kTile + i * kTile];
+                if constexpr (MODE == kScan) r.vc[i] = bck[NP * kTile + i * kTile];
             }
         }
     };
+    // state after walk tile tile0 + k of the batch row (the state after the very last tile is
+    // h_last, not a checkpoint)
     auto store_ckpt = [&](int k) {
-        if (p.ckpt && dvalid && k + 1 < ntiles) {  // never in segmented mode (b, ntiles: whole rows)
+        if (MODE == kScan && p.ckpt && dvalid && tile0 + k < last_chunk) {
 #pragma unroll
             for (int i = 0; i < NS; ++i) {
                 const int n = w * NS + i;
-                if (n < p.N) p.ckpt[(((int64_t)b * ntiles + k) * p.N + n) * p.ED + d] = h[i];
+                if (n < p.N) p.ckpt[(((int64_t)b * p.nchunks + tile0 + k) * p.N + n) * p.ED + d] = h[i];
             }
         }
     };
@@ -473,13 +487,19 @@ __global__ void __launch_bounds__((NW + kService) * kWave) sscan_fwd_kernel(cons
     if constexpr (kBcast) {
         auto tile_compute = [&](int k, const TileRegs& cur, TileRegs& next) {
             CTile& yt = sY[(k & 1) * NW + w];
-            *reinterpret_cast<float4*>(&yt[lane][0]) = scan_group_bcast<0, NS>(cur.dl, cur.uu, A2, h, cur.vb, cur.vc);
+            const float4 y0 = scan_group_bcast<0, NS, MODE>(cur.dl, cur.uu, A2, h, cur.vb, cur.vc);
+            if constexpr (MODE == kScan) *reinterpret_cast<float4*>(&yt[lane][0]) = y0;
             __builtin_amdgcn_sched_barrier(0);
             read_tile(k + 1, next);
             __builtin_amdgcn_sched_barrier(0);
-            *reinterpret_cast<float4*>(&yt[lane][4]) = scan_group_bcast<1, NS>(cur.dl, cur.uu, A2, h, cur.vb, cur.vc);
-            *reinterpret_cast<float4*>(&yt[lane][8]) = scan_group_bcast<2, NS>(cur.dl, cur.uu, A2, h, cur.vb, cur.vc);
-            *reinterpret_cast<float4*>(&yt[lane][12]) = scan_group_bcast<3, NS>(cur.dl, cur.uu, A2, h, cur.vb, cur.vc);
+            const float4 y1 = scan_group_bcast<1, NS, MODE>(cur.dl, cur.uu, A2, h, cur.vb, cur.vc);
+            const float4 y2 = scan_group_bcast<2, NS, MODE>(cur.dl, cur.uu, A2, h, cur.vb, cur.vc);
+            const float4 y3 = scan_group_bcast<3, NS, MODE>(cur.dl, cur.uu, A2, h, cur.vb, cur.vc);
+            if constexpr (MODE == kScan) {
+                *reinterpret_cast<float4*>(&yt[lane][4]) = y1;
+                *reinterpret_cast<float4*>(&yt[lane][8]) = y2;
+                *reinterpret_cast<float4*>(&yt[lane][12]) = y3;
+            }
             store_ckpt(k);
         };
         __syncthreads();
@@ -595,25 +615,21 @@ __global__ void __launch_bounds__(256) seg_carry_kernel(const float* __restrict_
 }
 
 // Segments per batch row.  The scan is serial in time, so a launch has only batch * dim/64
-// workgroups; when those cover a fraction of the chip's 256 CUs and no checkpoints are wanted
-// (inference prefill), the sequence is cut into segments that run side by side: twice the
-// arithmetic, nseg times the parallelism.
-struct SegPlan {
-    int nseg, seg_tiles;
-    size_t off_hend, off_h0, off_dsum, floats;
-};
-static SegPlan seg_plan(const mpa_sscan_shape* s, int ns) {
+// workgroups; when those cover a fraction of the chip's 256 CUs the sequence is cut into
+// segments that run side by side: up to twice the arithmetic, nseg times the parallelism.
+// `thin` is the coverage below which the cut pays: a third of the CUs for the forward (its first
+// pass costs 0.8 of the second), half of them for the backward (its first pass costs a quarter).
+SegPlan seg_plan(const mpa_sscan_shape* s, int ns, int thin) {
     SegPlan sp{1, 0, 0, 0, 0, 0};
     if (ns > 8) return sp;
     const int64_t ntiles = (s->seqlen + kTile - 1) / kTile;
     const int64_t groups = s->batch * ((s->dim + kWave - 1) / kWave);
     int64_t want = 1;
-    const char* v = getenv("MPA_FWD_NSEG");
-    if (v) {
-        want = atoi(v);
-    } else if (groups * 3 <= 256 && ntiles >= 64) {
+    if (s->plan_segments > 0) {
+        want = s->plan_segments;
+    } else if (groups * thin <= 256 && ntiles >= 32) {
         want = 256 / groups;
-        if (want > ntiles / 16) want = ntiles / 16;  // segments of 256 steps or more
+        if (want > ntiles / 8) want = ntiles / 8;  // segments of 128 steps or more
         if (want > 64) want = 64;
     }
     if (want > ntiles) want = ntiles;
@@ -629,31 +645,55 @@ static SegPlan seg_plan(const mpa_sscan_shape* s, int ns) {
     return sp;
 }
 
-template <typename IO, int NS, int NW, bool HAS_Z>
+template <typename IO, int NS, int NW, bool HAS_Z, int MODE>
 static int launch_fwd(const FwdParams& p, hipStream_t stream) {
     dim3 grid((p.ED + kWave - 1) / kWave, p.batch * (p.nseg > 1 ? p.nseg : 1));
-    dim3 block((NW + kService) * kWave);
+    dim3 block(kFwdWaves<NW, MODE> * kWave);
     constexpr size_t lds = sizeof(float) * FwdLds<NS, NW>::floats;
     static LdsLimitOnce lds_limit;
-    const int attr_rc = lds_limit.ensure(sscan_fwd_kernel<IO, NS, NW, HAS_Z>, lds);
+    const int attr_rc = lds_limit.ensure(sscan_fwd_kernel<IO, NS, NW, HAS_Z, MODE>, lds);
     if (attr_rc != MPA_OK) return attr_rc;
-    hipLaunchKernelGGL((sscan_fwd_kernel<IO, NS, NW, HAS_Z>), grid, block, lds, stream, p);
+    hipLaunchKernelGGL((sscan_fwd_kernel<IO, NS, NW, HAS_Z, MODE>), grid, block, lds, stream, p);
     return check_launch();
 }
 
 template <typename IO>
-static int dispatch_fwd(const FwdParams& p, int ns, int nw, hipStream_t stream) {
+static int dispatch_fwd(const FwdParams& p, int ns, int nw, int mode, hipStream_t stream) {
 #define MPA_CASE(NS_, NW_)                                                        \
-    if (ns == NS_ && nw == NW_)                                                   \
-        return p.z ? launch_fwd<IO, NS_, NW_, true>(p, stream)                    \
-                   : launch_fwd<IO, NS_, NW_, false>(p, stream);
+    if (ns == NS_ && nw == NW_ && mode == kScan)                                  \
+        return p.z ? launch_fwd<IO, NS_, NW_, true, kScan>(p, stream)             \
+                   : launch_fwd<IO, NS_, NW_, false, kScan>(p, stream);
     MPA_CASE(2, 8) MPA_CASE(4, 4) MPA_CASE(8, 2) MPA_CASE(16, 1)
     MPA_CASE(4, 8) MPA_CASE(8, 4) MPA_CASE(16, 2) MPA_CASE(32, 1)
     MPA_CASE(8, 8) MPA_CASE(16, 4) MPA_CASE(32, 2)
     MPA_CASE(16, 8) MPA_CASE(32, 4)
     MPA_CASE(32, 8)
 #undef MPA_CASE
+    // carry passes: the gate only matters to the backward's carry (dy * silu(z))
+#define MPA_CASE(NS_, NW_)                                                        \
+    if (ns == NS_ && nw == NW_ && mode == kCarry)                                 \
+        return launch_fwd<IO, NS_, NW_, false, kCarry>(p, stream);                \
+    if (ns == NS_ && nw == NW_ && mode == kGCarry)                                \
+        return p.z ? launch_fwd<IO, NS_, NW_, true, kGCarry>(p, stream)           \
+                   : launch_fwd<IO, NS_, NW_, false, kGCarry>(p, stream);
+    MPA_CASE(2, 8) MPA_CASE(4, 4) MPA_CASE(8, 2)
+    MPA_CASE(4, 8) MPA_CASE(8, 4)
+    MPA_CASE(8, 8)
+#undef MPA_CASE
     return MPA_ERR_BAD_SHAPE;
+}
+
+int launch_fwd_any(const FwdParams& p, int io_dtype, int ns, int nw, int mode, hipStream_t stream) {
+    return io_dtype == MPA_F32 ? dispatch_fwd<float>(p, ns, nw, mode, stream)
+                               : dispatch_fwd<bf16_t>(p, ns, nw, mode, stream);
+}
+
+int launch_seg_carry(const float* A, const float* h0, const float* hend, const float* dsum, float* segh0,
+                     float* hlast, int batch, int nseg, int ED, int N, hipStream_t st) {
+    const int64_t total = (int64_t)batch * ED * N;
+    hipLaunchKernelGGL(seg_carry_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, A, h0, hend, dsum,
+                       segh0, hlast, batch, nseg, ED, N);
+    return check_launch();
 }
 
 int validate_shape(const mpa_sscan_shape* s) {
@@ -662,6 +702,7 @@ int validate_shape(const mpa_sscan_shape* s) {
     if (s->dstate > MPA_MAX_DSTATE || s->batch > 65535) return MPA_ERR_BAD_SHAPE;
     if (s->seqlen > (int64_t)1 << 30 || s->dim > (int64_t)1 << 30) return MPA_ERR_BAD_SHAPE;
     if (s->io_dtype != MPA_F32 && s->io_dtype != MPA_BF16) return MPA_ERR_BAD_DTYPE;
+    if (s->plan_states_per_lane < 0 || s->plan_segments < 0 || s->reserved != 0) return MPA_ERR_BAD_SHAPE;
     const int64_t st[] = {s->z_sb, s->z_sl, s->z_sd, s->u_sb, s->u_sl, s->u_sd, s->d_sb, s->d_sl, s->d_sd, s->y_sb, s->y_sl,
                           s->y_sd, s->g_sb, s->g_sl, s->g_sd, s->bc_sb, s->bc_sl, s->dbc_sb, s->dbc_sl};
     for (int64_t v : st)
@@ -687,19 +728,14 @@ int padded_states(int64_t n) {
 // States per lane (NS) for a launch.  The only parallel axes are batch*dim/64 workgroups and
 // d_state/NS scan waves inside each; a workgroup holds at most 8 scan waves.  Fewer states per
 // lane mean more waves (better latency hiding) but more LDS traffic per state; ask for about
-// two scan waves per SIMD over the chip's 1024 SIMDs when the problem offers them.
-int pick_states_per_lane(int64_t batch, int64_t dim, int64_t dstate, int ns_cap, const char* env) {
+// two scan waves per SIMD over the chip's 1024 SIMDs when the problem offers them.  `pinned`
+// (the caller's plan_states_per_lane) wins when it is a value the kernels exist for.
+int pick_states_per_lane(int64_t batch, int64_t dim, int64_t dstate, int ns_cap, int pinned) {
     const int np = padded_states(dstate);
     const int ns_min = np / 8 > 2 ? np / 8 : 2;
     const int ns_max = ns_cap < np ? ns_cap : np;
     if (ns_max < ns_min) return -1;
-    if (env) {
-        const char* v = getenv(env);
-        if (v) {
-            const int ns = atoi(v);
-            if (ns >= ns_min && ns <= ns_max && (ns & (ns - 1)) == 0) return ns;
-        }
-    }
+    if (pinned >= ns_min && pinned <= ns_max && (pinned & (pinned - 1)) == 0) return pinned;
     const int64_t groups = batch * ((dim + kWave - 1) / kWave);
     int ns = ns_max;
     while (ns > ns_min && groups * (np / ns) < 2048) ns /= 2;
@@ -716,13 +752,14 @@ int launch_pack_bc(const mpa_sscan_shape* s, const void* B, const void* C, float
     const int np = padded_states(s->dstate);
     const int nchunks = (int)((s->seqlen + kTile - 1) / kTile);
     const int64_t per_b = (int64_t)nchunks * 2 * kTile * np;
+    const int reverse = (s->flags & MPA_SSCAN_REVERSE) ? 1 : 0;
     dim3 grid((unsigned)((per_b + 255) / 256), (unsigned)s->batch);
     if (s->io_dtype == MPA_F32)
         hipLaunchKernelGGL(pack_bc_kernel<float>, grid, dim3(256), 0, st, B, C, out, (int)s->seqlen,
-                           (int)s->dstate, ns, np / ns, kss, nchunks, s->bc_sb, s->bc_sl);
+                           (int)s->dstate, ns, np / ns, kss, nchunks, reverse, s->bc_sb, s->bc_sl);
     else
         hipLaunchKernelGGL(pack_bc_kernel<bf16_t>, grid, dim3(256), 0, st, B, C, out, (int)s->seqlen,
-                           (int)s->dstate, ns, np / ns, kss, nchunks, s->bc_sb, s->bc_sl);
+                           (int)s->dstate, ns, np / ns, kss, nchunks, reverse, s->bc_sb, s->bc_sl);
     return check_launch();
 }
 
@@ -736,11 +773,15 @@ extern "C" int64_t mpa_sscan_ckpt_elems(const mpa_sscan_shape* s) {
     return s->batch * nchunks * s->dstate * s->dim;
 }
 
-extern "C" size_t mpa_sscan_fwd_workspace_bytes(const mpa_sscan_shape* s) {
+// forward cut: a third of the CUs or fewer covered (see seg_plan)
+static constexpr int kFwdThin = 3;
+
+extern "C" size_t mpa_sscan_fwd_workspace_bytes(const mpa_sscan_shape* s, int with_ckpt) {
+    (void)with_ckpt;  // both kinds of call are cut by the same rule
     if (validate_shape(s) != MPA_OK) return 0;
     // the packed B/C exist only on the scalar-load path (more than 8 states per lane)
-    const int ns = pick_states_per_lane(s->batch, s->dim, s->dstate, 32, "MPA_FWD_NS");
-    if (ns <= 8) return (seg_plan(s, ns).floats * sizeof(float) + 255) / 256 * 256 + 256;
+    const int ns = pick_states_per_lane(s->batch, s->dim, s->dstate, 32, s->plan_states_per_lane);
+    if (ns <= 8) return (seg_plan(s, ns, kFwdThin).floats * sizeof(float) + 255) / 256 * 256 + 256;
     return (bcpack_floats(s) * sizeof(float) + 255) / 256 * 256;
 }
 
@@ -759,10 +800,10 @@ extern "C" int mpa_sscan_fwd(const mpa_sscan_shape* s, const void* x, const void
         !aligned_to(y, es) || (z && !aligned_to(z, es)) || (y_pregate && !aligned_to(y_pregate, es)) || !aligned_to(A, 4) || !aligned_to(D, 4) ||
         !aligned_to(workspace, 256))
         return MPA_ERR_MISALIGNED;
-    if (workspace_bytes < mpa_sscan_fwd_workspace_bytes(s)) return MPA_ERR_WORKSPACE;
+    if (workspace_bytes < mpa_sscan_fwd_workspace_bytes(s, h_ckpt != nullptr)) return MPA_ERR_WORKSPACE;
 
     const int np = padded_states(s->dstate);
-    const int ns = pick_states_per_lane(s->batch, s->dim, s->dstate, 32, "MPA_FWD_NS");
+    const int ns = pick_states_per_lane(s->batch, s->dim, s->dstate, 32, s->plan_states_per_lane);
     if (ns < 0) return MPA_ERR_BAD_SHAPE;
     const int nw = np / ns;
     hipStream_t st = static_cast<hipStream_t>(stream);
@@ -779,33 +820,29 @@ extern "C" int mpa_sscan_fwd(const mpa_sscan_shape* s, const void* x, const void
     p.batch = (int)s->batch; p.L = (int)s->seqlen; p.ED = (int)s->dim; p.N = (int)s->dstate;
     p.nchunks = (p.L + kTile - 1) / kTile;
     p.softplus = softplus ? 1 : 0;
+    p.reverse = (s->flags & MPA_SSCAN_REVERSE) ? 1 : 0;
     p.u_sb = s->u_sb; p.u_sl = s->u_sl; p.u_sd = s->u_sd;
     p.z_sb = s->z_sb; p.z_sl = s->z_sl; p.z_sd = s->z_sd;
     p.d_sb = s->d_sb; p.d_sl = s->d_sl; p.d_sd = s->d_sd;
     p.y_sb = s->y_sb; p.y_sl = s->y_sl; p.y_sd = s->y_sd;
     p.in_tmajor = (s->u_sd != 1 && s->u_sl == 1) ? 1 : 0;
     p.out_tmajor = (s->y_sd != 1 && s->y_sl == 1) ? 1 : 0;
-    auto run = [&](const FwdParams& q) {
-        return s->io_dtype == MPA_F32 ? dispatch_fwd<float>(q, ns, nw, st) : dispatch_fwd<bf16_t>(q, ns, nw, st);
-    };
-    const SegPlan sp = h_ckpt ? SegPlan{1, 0, 0, 0, 0, 0} : seg_plan(s, ns);
-    if (sp.nseg <= 1) return run(p);
+    const SegPlan sp = seg_plan(s, ns, kFwdThin);
+    if (sp.nseg <= 1) return launch_fwd_any(p, s->io_dtype, ns, nw, kScan, st);
 
     // segmented mode: end states of every segment from zero, carry, then the real pass
     float* wsf = static_cast<float*>(workspace);
     FwdParams p1 = p;
     p1.nseg = sp.nseg; p1.seg_tiles = sp.seg_tiles;
-    p1.z = nullptr; p1.y = nullptr; p1.ypre = nullptr; p1.h0 = nullptr;
+    p1.z = nullptr; p1.y = nullptr; p1.ypre = nullptr; p1.h0 = nullptr; p1.ckpt = nullptr;
     p1.hlast = wsf + sp.off_hend; p1.dsum = wsf + sp.off_dsum;
-    rc = run(p1);
+    rc = launch_fwd_any(p1, s->io_dtype, ns, nw, kCarry, st);
     if (rc != MPA_OK) return rc;
-    const int64_t total = (int64_t)p.batch * p.ED * p.N;
-    hipLaunchKernelGGL(seg_carry_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, A, h0,
-                       wsf + sp.off_hend, wsf + sp.off_dsum, wsf + sp.off_h0, h_last, p.batch, sp.nseg, p.ED, p.N);
-    rc = check_launch();
+    rc = launch_seg_carry(A, h0, wsf + sp.off_hend, wsf + sp.off_dsum, wsf + sp.off_h0, h_last, p.batch, sp.nseg,
+                          p.ED, p.N, st);
     if (rc != MPA_OK) return rc;
     FwdParams p2 = p;
     p2.nseg = sp.nseg; p2.seg_tiles = sp.seg_tiles;
     p2.h0 = wsf + sp.off_h0; p2.hlast = nullptr;
-    return run(p2);
+    return launch_fwd_any(p2, s->io_dtype, ns, nw, kScan, st);
 }

@@ -52,9 +52,11 @@ class LM(nn.Module):
         return self.lm_head(self.norm_f(x))
 
     @torch.no_grad()
-    def prefill(self, tokens):
-        """Run the prompt once; returns (logits of the last position (B, vocab), caches)."""
-        x, caches = self.mamba(self.embedding(tokens), return_caches=True)
+    def prefill(self, tokens, caches=None):
+        """Run the prompt once; returns (logits of the last position (B, vocab), caches).  With
+        `caches` (from an earlier prefill or step) the prompt continues that sequence, so a long
+        prompt can be fed in pieces."""
+        x, caches = self.mamba(self.embedding(tokens), caches=caches, return_caches=True)
         return self.lm_head(self.norm_f(x[:, -1])), caches
 
     @torch.no_grad()
@@ -63,17 +65,35 @@ class LM(nn.Module):
         x, caches = self.mamba.step(self.embedding(token), caches)
         return self.lm_head(self.norm_f(x)), caches
 
-    @torch.no_grad()
-    def generate(self, prompt, num_tokens: int, sample: bool = False, temperature: float = 1.0):
-        """Greedy (or sampled) continuation of `prompt` (B, L): one prefill, then O(1) steps."""
-        logits, caches = self.prefill(prompt)
-        out = [prompt]
-        for _ in range(num_tokens):
-            if sample:
-                probs = torch.softmax(logits.float() / temperature, dim=-1)
-                nxt = torch.multinomial(probs, 1).squeeze(1)
-            else:
-                nxt = logits.argmax(-1)
-            out.append(nxt.unsqueeze(1))
-            logits, caches = self.step(nxt, caches)
-        return torch.cat(out, dim=1)
+    def generate(self, prompt, num_tokens: int, sample: bool = True, top_k: int = None, temperature: float = 1.0):
+        """The reference's call (mambapy/lm.py:119-155), same arguments, defaults and result:
+        prompt (B, L) -> the num_tokens generated tokens (B, num_tokens) on the prompt's device;
+        sampling (optionally restricted to the top_k most likely tokens) unless sample=False; the
+        module is put in eval mode for the call and back in train mode afterwards, as there.
+        Where the reference runs the whole sequence through forward again for every token, this
+        runs the prompt once and then one state-update step per token."""
+        if num_tokens <= 0:
+            return prompt[:, :0]
+        if top_k is not None:
+            top_k = min(top_k, self.vocab_size)
+        input_device = prompt.device
+        prompt = prompt.to(self.embedding.weight.device)
+        self.eval()
+        out = []
+        with torch.no_grad():
+            logits, caches = self.prefill(prompt)
+            for i in range(num_tokens):
+                if sample:
+                    probs = torch.softmax(logits.float() / temperature, dim=-1)
+                    if top_k is not None:
+                        values, _ = torch.topk(probs, k=top_k)
+                        probs[probs < values[:, -1, None]] = 0
+                        probs = probs / probs.sum(dim=1, keepdim=True)
+                    nxt = torch.multinomial(probs, num_samples=1).squeeze(1)
+                else:
+                    nxt = logits.argmax(dim=-1)
+                out.append(nxt.unsqueeze(1))
+                if i + 1 < num_tokens:          # the state after the last token is not needed
+                    logits, caches = self.step(nxt, caches)
+        self.train()
+        return torch.cat(out, dim=1).to(input_device)

@@ -187,40 +187,47 @@ class MambaBlock(nn.Module):
     def forward(self, x, cache: Optional[Tuple] = None, return_cache: bool = False):
         """x : (B, L, D) -> (B, L, D).  With return_cache=True also returns the decode cache
         (h (B,ED,N) float32, inputs (B,ED,d_conv-1)) after the last position, so that
-        generation can continue with step() instead of re-running the sequence."""
+        generation can continue with step() instead of re-running the sequence.  `cache` (the
+        same pair, from an earlier call or from step(); h may be None) is what the sequence
+        continues from: the state before position 0 and the inputs before it.  No gradient
+        flows into the cache."""
         L = x.shape[1]
         xz = self.in_proj(x)
         xin, z = xz.chunk(2, dim=-1)
         K = self.config.d_conv
+        h_in, win_in = cache if cache is not None else (None, None)
         window = None
         if 2 <= K <= 4:
             # causal depthwise convolution + bias + silu in one kernel, reading the x half of
             # the projection in place (no transposes) and returning the decode window
             cw, cb = self._conv_wb()
             if return_cache:
-                xs, window = causal_conv1d_fn(xin, cw, cb, return_window=True)
+                xs, window = causal_conv1d_fn(xin, cw, cb, window=win_in, return_window=True)
             else:
-                xs = causal_conv1d_fn(xin, cw, cb)
+                xs = causal_conv1d_fn(xin, cw, cb, window=win_in)
         else:
-            xc = self.conv1d(xin.transpose(1, 2))[:, :, :L]
+            pre = xin.transpose(1, 2)                        # (B, ED, L)
+            if win_in is not None:
+                full = torch.cat([win_in.detach().to(pre.dtype), pre], dim=2)
+                xc = F.conv1d(full, self.conv1d.weight, self.conv1d.bias, groups=self.config.d_inner)
+            else:
+                full = F.pad(pre, (K - 1, 0))
+                xc = self.conv1d(pre)[:, :, :L]
             xs = F.silu(xc).transpose(1, 2)                  # (B, L, ED), unit stride along L
+            if return_cache:
+                window = full[:, :, full.shape[2] - (K - 1):].detach().contiguous()
+        h0 = None if h_in is None else h_in.detach()
         # the gate y * silu(z) is applied inside the scan kernel (z is read in place)
         if return_cache:
-            y, h_last = self.ssm(xs, z, return_last_state=True)
+            y, h_last = self.ssm(xs, z, return_last_state=True, h0=h0)
         else:
-            y = self.ssm(xs, z)
+            y = self.ssm(xs, z, h0=h0)
         out = self.out_proj(y)
         if not return_cache:
             return out
-        if window is None:
-            pre = xin.transpose(1, 2)
-            if L >= K - 1:
-                window = pre[:, :, L - (K - 1):].contiguous()
-            else:
-                window = F.pad(pre, (K - 1 - L, 0)).contiguous()
         return out, (h_last, window)
 
-    def ssm(self, x, z=None, return_last_state: bool = False):
+    def ssm(self, x, z=None, return_last_state: bool = False, h0=None):
         """(B, L, ED) -> (B, L, ED): projections to (delta, B, C), then the fused scan
         (mambapy/mamba.py:236-272); with z the result is already gated, y * silu(z), as on the
         reference's fused path (mamba.py:259-260, 225-227)."""
@@ -231,9 +238,9 @@ class MambaBlock(nn.Module):
         delta = F.linear(dlow, self.dt_proj.weight)
         if self.config.fused_softplus:
             return selective_scan_fn(x, delta, A, Bm, C, D, z=z, delta_bias=self._dt_bias(),
-                                     delta_softplus=True, return_last_state=return_last_state)
+                                     delta_softplus=True, h0=h0, return_last_state=return_last_state)
         delta = F.softplus(delta + self.dt_proj.bias)
-        return selective_scan_fn(x, delta, A, Bm, C, D, z=z, return_last_state=return_last_state)
+        return selective_scan_fn(x, delta, A, Bm, C, D, z=z, h0=h0, return_last_state=return_last_state)
 
     def selective_scan(self, x, delta, A, B, C, D):
         """Same call as MambaBlock.selective_scan (mambapy/mamba.py:274-295)."""
@@ -301,11 +308,11 @@ class ResidualBlock(nn.Module):
         self.mixer = MambaBlock(config)
         self.norm = RMSNorm(config.d_model, config.rms_norm_eps, config.mup)
 
-    def forward(self, x, return_cache: bool = False):
+    def forward(self, x, cache: Optional[Tuple] = None, return_cache: bool = False):
         if return_cache:
-            y, cache = self.mixer(self.norm(x), return_cache=True)
+            y, cache = self.mixer(self.norm(x), cache=cache, return_cache=True)
             return y + x, cache
-        return self.mixer(self.norm(x)) + x
+        return self.mixer(self.norm(x), cache=cache) + x
 
     def step(self, x, cache):
         y, cache = self.mixer.step(self.norm(x), cache)
@@ -323,21 +330,25 @@ class Mamba(nn.Module):
         self.config = config
         self.layers = nn.ModuleList([ResidualBlock(config) for _ in range(config.n_layers)])
 
-    def forward(self, x, return_caches: bool = False):
+    def forward(self, x, caches=None, return_caches: bool = False):
+        """x : (B, L, D) -> (B, L, D) [, caches].  `caches` (one (h, inputs) pair per layer, as
+        returned by an earlier call with return_caches=True, by step() or by empty_caches()) makes
+        the call continue that sequence."""
         # Same arithmetic as x = layer(x) for every layer, in another order of kernels: the add
         # that ends layer i is done by the norm kernel that starts layer i+1 (pre-norm
         # residual stream: `hidden` is the last mixer output, `residual` the running sum).
         hidden, residual = x, None
-        caches = []
-        for layer in self.layers:
+        new_caches = []
+        for i, layer in enumerate(self.layers):
             normed, residual = layer.norm.add_norm(hidden, residual)
+            cache = None if caches is None else caches[i]
             if return_caches:
-                hidden, c = layer.mixer(normed, return_cache=True)
-                caches.append(c)
+                hidden, c = layer.mixer(normed, cache=cache, return_cache=True)
+                new_caches.append(c)
             else:
-                hidden = layer.mixer(normed)
+                hidden = layer.mixer(normed, cache=cache)
         x = hidden + residual if self.layers else x
-        return (x, caches) if return_caches else x
+        return (x, new_caches) if return_caches else x
 
     def step(self, x, caches):
         hidden, residual = x, None

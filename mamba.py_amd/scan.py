@@ -9,7 +9,9 @@ Mirrors, by name and argument meaning:
 PyTorch supplies device memory, streams and the autograd graph; all arithmetic runs in
 libmambapy_amd.so.  Tensors must live on a ROCm device: there is no CPU path.
 """
+import contextlib
 import ctypes
+import os
 
 import torch
 
@@ -50,7 +52,55 @@ def _rows_unit_stride(t):
     return t if t.stride(-1) == 1 else t.contiguous()
 
 
-def _sscan_shape(x, delta, Bm, y_like, g_like, dbc_like, N, flags, z=None):
+class LaunchPlan:
+    """Overrides of the decomposition the library would choose from the shape (None / False =
+    let it choose).  The library itself reads no environment: the MPA_* variables below are
+    read here, once, when the module is imported, and travel to the kernels inside the shape
+    struct of every call.
+
+        MPA_FWD_NS / MPA_BWD_NS       states of d_state per lane (a power of two)
+        MPA_FWD_NSEG / MPA_BWD_NSEG   segments a sequence is cut into (1 = never cut)
+        MPA_BWD_GENERAL=1             general backward kernel even where the fast one applies
+    """
+    _FIELDS = ("fwd_states_per_lane", "bwd_states_per_lane", "fwd_segments", "bwd_segments",
+               "bwd_general", "expire_waits")
+
+    def __init__(self):
+        env = lambda k: int(os.environ[k]) if os.environ.get(k, "").strip() else None
+        self.fwd_states_per_lane = env("MPA_FWD_NS")
+        self.bwd_states_per_lane = env("MPA_BWD_NS")
+        self.fwd_segments = env("MPA_FWD_NSEG")
+        self.bwd_segments = env("MPA_BWD_NSEG")
+        self.bwd_general = os.environ.get("MPA_BWD_GENERAL", "") == "1"
+        self.expire_waits = False  # test hook (MPA_PLAN_EXPIRE_WAITS)
+
+    def fill(self, shape, backward):
+        shape.plan_states_per_lane = (self.bwd_states_per_lane if backward else self.fwd_states_per_lane) or 0
+        shape.plan_segments = (self.bwd_segments if backward else self.fwd_segments) or 0
+        shape.plan_flags = (_lib.MPA_PLAN_BWD_GENERAL if self.bwd_general else 0) | \
+                           (_lib.MPA_PLAN_EXPIRE_WAITS if self.expire_waits else 0)
+
+
+plan = LaunchPlan()
+
+
+@contextlib.contextmanager
+def plan_override(**kw):
+    """with plan_override(fwd_segments=4, bwd_states_per_lane=2): ...  (tuning and tests)"""
+    for k in kw:
+        if k not in LaunchPlan._FIELDS:
+            raise TypeError(f"unknown plan field {k!r}")
+    old = {k: getattr(plan, k) for k in kw}
+    for k, v in kw.items():
+        setattr(plan, k, v)
+    try:
+        yield plan
+    finally:
+        for k, v in old.items():
+            setattr(plan, k, v)
+
+
+def _sscan_shape(x, delta, Bm, y_like, g_like, dbc_like, N, flags, z=None, backward=False):
     s = _lib.SscanShape()
     s.batch, s.seqlen, s.dim = x.shape
     s.dstate = N
@@ -64,6 +114,7 @@ def _sscan_shape(x, delta, Bm, y_like, g_like, dbc_like, N, flags, z=None):
     s.g_sb, s.g_sl, s.g_sd = g_like.stride()
     s.bc_sb, s.bc_sl = Bm.stride(0), Bm.stride(1)
     s.dbc_sb, s.dbc_sl = dbc_like.stride(0), dbc_like.stride(1)
+    plan.fill(s, backward)
     return s
 
 
@@ -72,7 +123,7 @@ class SelectiveScanFn(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, x, delta, A, B, C, D, z, delta_bias, delta_softplus, h0, return_last_state,
-                need_grad=True):
+                need_grad=True, reverse=False):
         _require_gpu(x, delta, A, B, C, D, z, delta_bias, h0)
         lib = _lib.load()
         dt = x.dtype
@@ -88,6 +139,8 @@ class SelectiveScanFn(torch.autograd.Function):
             raise RuntimeError("z must have the shape of x")
         if delta_bias is not None and not delta_softplus:
             raise RuntimeError("delta_bias needs delta_softplus=True")
+        if h0 is not None and h0.requires_grad and need_grad:
+            raise RuntimeError("selective_scan_fn: no gradient is computed for h0; pass h0.detach()")
         x_ = x.detach()
         delta_ = delta.detach().to(dt)
         B_ = _rows_unit_stride(B.detach().to(dt))
@@ -99,7 +152,8 @@ class SelectiveScanFn(torch.autograd.Function):
         y = torch.empty((Bsz, L, ED), dtype=dt, device=x.device)
         # need_grad: checkpoints (and the pre-gate output) are written only for a backward pass;
         # without them the library is also free to cut a long sequence into parallel segments
-        flags = _lib.MPA_SSCAN_DELTA_SOFTPLUS if delta_softplus else 0
+        flags = (_lib.MPA_SSCAN_DELTA_SOFTPLUS if delta_softplus else 0) | \
+                (_lib.MPA_SSCAN_REVERSE if reverse else 0)
         shape = _sscan_shape(x_, delta_, B_, y, y, B_, N, flags, z_)
         ckpt = y_pre = None
         if need_grad:
@@ -109,7 +163,7 @@ class SelectiveScanFn(torch.autograd.Function):
                 y_pre = torch.empty_like(y)  # output before the gate, read again by the backward
         h_last = torch.empty((Bsz, ED, N), dtype=torch.float32, device=x.device) \
             if return_last_state else None
-        nbytes = lib.mpa_sscan_fwd_workspace_bytes(ctypes.byref(shape))
+        nbytes = lib.mpa_sscan_fwd_workspace_bytes(ctypes.byref(shape), 1 if need_grad else 0)
         ws = torch.empty(nbytes, dtype=torch.uint8, device=x.device)
         with torch.cuda.device(x.device):
             rc = lib.mpa_sscan_fwd(ctypes.byref(shape), _ptr(x_), _ptr(delta_), _ptr(A_), _ptr(B_),
@@ -147,7 +201,7 @@ class SelectiveScanFn(torch.autograd.Function):
         dB = torch.empty((Bsz, L, N), dtype=dt, device=x.device)
         dC = torch.empty_like(dB)
         dbias = torch.empty((ED,), dtype=torch.float32, device=x.device) if bias is not None else None
-        shape = _sscan_shape(x, delta, B, dy, dx, dB, N, ctx.flags, z)
+        shape = _sscan_shape(x, delta, B, dy, dx, dB, N, ctx.flags, z, backward=True)
         nbytes = lib.mpa_sscan_bwd_workspace_bytes(ctypes.byref(shape))
         ws = torch.empty(nbytes, dtype=torch.uint8, device=x.device)
         with torch.cuda.device(x.device):
@@ -160,24 +214,28 @@ class SelectiveScanFn(torch.autograd.Function):
         tx, td, tA, tB, tC, tD, tz, tb = ctx.in_dtypes
         return (dx.to(tx), ddelta.to(td), dA.to(tA), dB.to(tB), dC.to(tC), dD.to(tD),
                 None if dz is None else dz.to(tz), None if dbias is None else dbias.to(tb),
-                None, None, None, None)
+                None, None, None, None, None)
 
 
 def selective_scan_fn(x, delta, A, B, C, D, z=None, delta_bias=None, delta_softplus=False,
-                      h0=None, return_last_state=False):
+                      h0=None, return_last_state=False, reverse=False):
     """y = selective scan of (x, delta, A, B, C, D), optionally with softplus(delta + bias)
     and the gate y*silu(z) folded in (the fused form the reference reaches through
     `use_cuda`, mambapy/mamba.py:252-261), in this package's (B, L, ED) layout.
 
     x, delta, z : (B, L, ED);  A : (ED, N);  B, C : (B, L, N);  D, delta_bias : (ED);
     h0 : optional (B, ED, N) initial state.  Returns y (B, L, ED) [, last state (B, ED, N)].
+    reverse=True runs the recurrence from the last step to the first: the same result as
+    flipping x, delta, z, B, C along time, scanning and flipping y back (the backward direction
+    of the reference's bidirectional block, mambapy/vim.py:228-261), without the copies; h0 is
+    then the state before step L-1 and the last state the one after step 0.
     """
     # grad mode is off inside Function.forward and parameters keep requires_grad under no_grad,
     # so whether a backward can follow is decided here
     need_grad = torch.is_grad_enabled() and any(
         t is not None and t.requires_grad for t in (x, delta, A, B, C, D, z, delta_bias))
     return SelectiveScanFn.apply(x, delta, A, B, C, D, z, delta_bias, bool(delta_softplus), h0,
-                                 bool(return_last_state), need_grad)
+                                 bool(return_last_state), need_grad, bool(reverse))
 
 
 def selective_scan(x, delta, A, B, C, D):
@@ -206,7 +264,7 @@ class PScan(torch.autograd.Function):
     and never modifies its inputs (mambapy/pscan.py:151-224).  Any L: no padding."""
 
     @staticmethod
-    def forward(ctx, A_in, X_in):
+    def forward(ctx, A_in, X_in, reverse=False):
         _require_gpu(A_in, X_in)
         if A_in.shape != X_in.shape or X_in.dim() != 4:
             raise RuntimeError(f"pscan expects two (B, L, D, N) tensors, got {tuple(A_in.shape)} "
@@ -218,12 +276,13 @@ class PScan(torch.autograd.Function):
         A = A_in.detach().to(dt)
         X = X_in.detach().to(dt)
         H = torch.empty(X.shape, dtype=dt, device=X.device)
-        shape = _pscan_shape(A, X, H)
+        shape = _pscan_shape(A, X, H, reverse=reverse)
         with torch.cuda.device(X.device):
             rc = lib.mpa_pscan_fwd(ctypes.byref(shape), _ptr(A), _ptr(X), _ptr(H), _stream(X.device))
         _lib.check(rc, "mpa_pscan_fwd")
         ctx.save_for_backward(A, H)
         ctx.in_dtypes = (A_in.dtype, X_in.dtype)
+        ctx.reverse = bool(reverse)
         return H
 
     @staticmethod
@@ -233,15 +292,21 @@ class PScan(torch.autograd.Function):
         G = grad_output_in.to(H.dtype)
         gA = torch.empty_like(H)
         gX = torch.empty_like(H)
-        shape = _pscan_shape(A, G, H, gA, gX)
+        shape = _pscan_shape(A, G, H, gA, gX, reverse=ctx.reverse)
         with torch.cuda.device(H.device):
             rc = lib.mpa_pscan_bwd(ctypes.byref(shape), _ptr(A), _ptr(H), _ptr(G), _ptr(gA), _ptr(gX),
                                    _stream(H.device))
         _lib.check(rc, "mpa_pscan_bwd")
-        return gA.to(ctx.in_dtypes[0]), gX.to(ctx.in_dtypes[1])
+        return gA.to(ctx.in_dtypes[0]), gX.to(ctx.in_dtypes[1]), None
 
 
 pscan = PScan.apply
+
+
+def pscan_rev(A, X):
+    """H[t] = A[t]*H[t+1] + X[t], H[L] = 0: the scan of mambapy/pscan.py:94-149
+    (PScan.pscan_rev, `flip . pscan . flip`) as a differentiable call of its own."""
+    return PScan.apply(A, X, True)
 
 
 # ------------------------------------------------------------------------------------------

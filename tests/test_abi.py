@@ -29,7 +29,7 @@ def test_library_exports_every_declared_symbol(pkg):
         assert hasattr(lib, n), f"{n} is declared in the header but not exported"
     assert set(pkg._lib.EXPORTS) == set(_declared_functions())
     assert lib.mpa_arch() == b"gfx950"
-    assert lib.mpa_version() == 100
+    assert lib.mpa_version() == 200
 
 
 def test_status_codes_without_launch(pkg):
@@ -47,6 +47,10 @@ def test_status_codes_without_launch(pkg):
     assert lib.mpa_sscan_fwd(ctypes.byref(s), *([None] * 14), 0, None) == 1  # null data pointers
     assert lib.mpa_sscan_ckpt_elems(ctypes.byref(s)) == 1 * 1 * 16 * 8
     assert lib.mpa_sscan_bwd_workspace_bytes(ctypes.byref(s)) > 0
+    assert lib.mpa_sscan_fwd_workspace_bytes(ctypes.byref(s), 0) > 0
+    s.reserved = 1
+    assert lib.mpa_sscan_fwd(ctypes.byref(s), *([None] * 14), 0, None) == 2  # reserved field must be 0
+    s.reserved = 0
     assert lib.mpa_status_string(6) == b"workspace too small"
     p = L.PscanShape()
     assert lib.mpa_pscan_fwd(ctypes.byref(p), None, None, None, None) == 2
@@ -68,3 +72,43 @@ def test_cpu_tensors_are_rejected(pkg):
                            torch.zeros(8))
     with pytest.raises(RuntimeError, match="ROCm device"):
         pkg.pscan(torch.zeros(1, 4, 8, 16), torch.zeros(1, 4, 8, 16))
+
+
+def test_workspace_queries_follow_the_plan_fields_not_the_environment(pkg, monkeypatch):
+    # the library keeps no global state and reads no environment: the segment count a caller
+    # pins in the shape struct decides the workspace, a variable of the same name does not
+    L = pkg._lib
+    lib = L.load()
+    s = L.SscanShape()
+    s.batch, s.seqlen, s.dim, s.dstate = 1, 4096, 64, 16
+    base = lib.mpa_sscan_fwd_workspace_bytes(ctypes.byref(s), 1)
+    monkeypatch.setenv("MPA_FWD_NSEG", "1")
+    monkeypatch.setenv("MPA_FWD_NS", "16")
+    assert lib.mpa_sscan_fwd_workspace_bytes(ctypes.byref(s), 1) == base
+    s.plan_segments = 1
+    never_cut = lib.mpa_sscan_fwd_workspace_bytes(ctypes.byref(s), 1)
+    s.plan_segments = 8
+    cut8 = lib.mpa_sscan_fwd_workspace_bytes(ctypes.byref(s), 1)
+    assert never_cut < cut8
+    assert cut8 >= 2 * 8 * 64 * 16 * 4          # start and end states of 8 segments
+    b0 = lib.mpa_sscan_bwd_workspace_bytes(ctypes.byref(s))
+    s.plan_segments = 1
+    assert lib.mpa_sscan_bwd_workspace_bytes(ctypes.byref(s)) < b0
+
+
+def test_launch_plan_reads_the_environment_once_in_python(pkg, monkeypatch):
+    scan = pkg.scan
+    monkeypatch.setenv("MPA_BWD_NSEG", "5")
+    monkeypatch.setenv("MPA_BWD_GENERAL", "1")
+    p = scan.LaunchPlan()
+    s = pkg._lib.SscanShape()
+    p.fill(s, backward=True)
+    assert s.plan_segments == 5 and s.plan_flags == pkg._lib.MPA_PLAN_BWD_GENERAL
+    p.fill(s, backward=False)
+    assert s.plan_segments == 0
+    with pkg.plan_override(fwd_segments=3):
+        assert pkg.plan.fwd_segments == 3
+    assert pkg.plan.fwd_segments is None
+    with pytest.raises(TypeError):
+        with pkg.plan_override(nonsense=1):
+            pass

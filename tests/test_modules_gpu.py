@@ -105,12 +105,20 @@ def test_lm_forward_generate_and_bf16(pkg, dev):
         assert logits.shape == (2, 37, 101) and torch.isfinite(logits).all()
         last, caches = lm.prefill(tok)
         assert rel_err(last, logits[:, -1]) <= 1e-4
-        out = lm.generate(tok[:, :5], 6)
-        assert out.shape == (2, 11)
+        # the reference's contract (lm.py:119-155): only the new tokens come back, on the prompt's
+        # device, and the module is left in train mode
+        new = lm.generate(tok[:, :5], 6, sample=False)
+        assert new.shape == (2, 6) and lm.training
         # greedy continuation must agree with re-running the full forward (the reference's
-        # O(L^2) generate, lm.py:119-155)
+        # O(L^2) generate)
+        out = torch.cat([tok[:, :5], new], 1)
         again = lm(out[:, :-1]).argmax(-1)
         assert torch.equal(again[:, 4:], out[:, 5:])
+        torch.manual_seed(11)
+        sampled = lm.generate(tok[:, :5].cpu(), 4, top_k=3)   # default: sampling; prompt on the CPU
+        assert sampled.shape == (2, 4) and sampled.device.type == "cpu"
+        top3 = lm(tok[:, :5])[:, -1].topk(3).indices.cpu()
+        assert all(sampled[b, 0] in top3[b] for b in range(2))
         lm16 = lm.to(torch.bfloat16)
         l16 = lm16(tok)
         assert l16.dtype == torch.bfloat16 and rel_err(l16, logits) <= 5e-2
@@ -187,3 +195,103 @@ def test_graphed_decoder_replays_match_eager_steps(pkg, dev):
         for t in range(5):
             want, caches = model.step(x[t], caches)
             assert rel_err(decoder(x[t]), want) <= 1e-5, t
+
+
+def test_forward_continues_from_a_cache(pkg, dev):
+    # a sequence fed in pieces (each piece started from the cache the piece before returned)
+    # gives what one pass gives, at block, stack and LM level; a cache must never be ignored
+    torch.manual_seed(21)
+    cfg = pkg.MambaConfig(d_model=32, n_layers=3)
+    model = pkg.Mamba(cfg).to(dev)
+    x = torch.randn(2, 50, 32, device=dev)
+    with torch.no_grad():
+        y_full, c_full = model(x, return_caches=True)
+        y1, c1 = model(x[:, :17], return_caches=True)
+        y2, c2 = model(x[:, 17:18], caches=c1, return_caches=True)      # a piece shorter than the window
+        y3, c3 = model(x[:, 18:], caches=c2, return_caches=True)
+        assert rel_err(torch.cat([y1, y2, y3], 1), y_full) <= 1e-5
+        for (h, w), (hf, wf) in zip(c3, c_full):
+            assert rel_err(h, hf) <= 1e-5 and torch.equal(w, wf)
+        # from the caches of step(): empty caches, two steps, then the rest in one call
+        caches = model.empty_caches(2)
+        ys = []
+        for t in range(2):
+            y, caches = model.step(x[:, t], caches)
+            ys.append(y)
+        rest = model(x[:, 2:], caches=caches)
+        assert rel_err(torch.cat([torch.stack(ys, 1), rest], 1), y_full) <= 1e-5
+        blk = model.layers[0].mixer
+        a = blk(x)
+        b1, c = blk(x[:, :30], return_cache=True)
+        b2 = blk(x[:, 30:], cache=c)
+        assert rel_err(torch.cat([b1, b2], 1), a) <= 1e-5
+        assert rel_err(blk(x[:, 30:]), a[:, 30:]) > 1e-3     # the cache matters
+    lm = pkg.LM(cfg, 77).to(dev)
+    tok = torch.randint(0, 77, (2, 40), device=dev)
+    l_all, _ = lm.prefill(tok)
+    _, c = lm.prefill(tok[:, :25])
+    l_cont, _ = lm.prefill(tok[:, 25:], caches=c)
+    assert rel_err(l_cont, l_all) <= 1e-5
+
+
+def test_training_through_a_continued_forward(pkg, dev):
+    # truncated backpropagation: the second piece is trained from the detached state of the first
+    torch.manual_seed(23)
+    cfg = pkg.MambaConfig(d_model=32, n_layers=1)
+    blk = pkg.MambaBlock(cfg).to(dev)
+    x = torch.randn(2, 40, 32, device=dev)
+    with torch.no_grad():
+        _, cache = blk(x[:, :20], return_cache=True)
+    xr = x[:, 20:].clone().requires_grad_()
+    y = blk(xr, cache=cache)
+    y.square().mean().backward()
+    assert torch.isfinite(xr.grad).all() and xr.grad.abs().max() > 0
+
+
+def test_block_with_inner_layernorms_matches_float64_layer(pkg, dev):
+    # inner_layernorms=True (mambapy/mamba.py:196-203, 246): RMSNorm over the dt_rank, d_state and
+    # d_state slices of the x_proj output, i.e. rows that are strided slices of one projection
+    torch.manual_seed(31)
+    cfg = pkg.MambaConfig(d_model=64, n_layers=1, inner_layernorms=True)
+    blk = pkg.MambaBlock(cfg).to(dev)
+    with torch.no_grad():
+        for n in (blk.dt_layernorm, blk.B_layernorm, blk.C_layernorm):
+            n.weight.uniform_(0.5, 1.5)
+    x = torch.randn(2, 45, 64)
+    g = torch.randn(2, 45, 64)
+
+    p = {k: v.detach().double().cpu().requires_grad_() for k, v in blk.named_parameters()}
+
+    def ref_forward(xx):
+        L = xx.shape[1]
+        xz = F.linear(xx, p["in_proj.weight"])
+        xin, z = xz.chunk(2, dim=-1)
+        xc = F.conv1d(xin.transpose(1, 2), p["conv1d.weight"], p["conv1d.bias"], padding=cfg.d_conv - 1,
+                      groups=cfg.d_inner)[:, :, :L].transpose(1, 2)
+        xs = F.silu(xc)
+        dlow, Bm, C = torch.split(F.linear(xs, p["x_proj.weight"]), [cfg.dt_rank, cfg.d_state, cfg.d_state], dim=-1)
+        dlow = so.rmsnorm_ref(dlow, p["dt_layernorm.weight"], cfg.rms_norm_eps)
+        Bm = so.rmsnorm_ref(Bm, p["B_layernorm.weight"], cfg.rms_norm_eps)
+        C = so.rmsnorm_ref(C, p["C_layernorm.weight"], cfg.rms_norm_eps)
+        delta = so.softplus_ref(F.linear(dlow, p["dt_proj.weight"], p["dt_proj.bias"]))
+        y = so.selective_scan_ref(xs, delta, -torch.exp(p["A_log"]), Bm, C, p["D"])
+        return F.linear(y * F.silu(z), p["out_proj.weight"])
+
+    xr = x.double().requires_grad_()
+    yr = ref_forward(xr)
+    yr.backward(g.double())
+    xg = x.to(dev).requires_grad_()
+    y = blk(xg)
+    y.backward(g.to(dev))
+    assert rel_err(y, yr) <= 1e-4
+    assert rel_err(xg.grad, xr.grad) <= 2e-4
+    for k, v in blk.named_parameters():
+        assert rel_err(v.grad, p[k].grad) <= 5e-4, k
+    # decode: steps from empty caches reproduce the parallel forward with the norms in place
+    with torch.no_grad():
+        cache = (None, torch.zeros(2, cfg.d_inner, cfg.d_conv - 1, device=dev))
+        ys = []
+        for t in range(12):
+            yt, cache = blk.step(x[:, t].to(dev), cache)
+            ys.append(yt)
+        assert rel_err(torch.stack(ys, 1), yr[:, :12]) <= 1e-4

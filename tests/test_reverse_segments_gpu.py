@@ -1,0 +1,270 @@
+"""GPU parity of the launch variants of the fused scan and of the generic scan:
+  * reverse direction (MPA_SSCAN_REVERSE; mpa_pscan_* with reverse = 1) against
+    flip . oracle . flip, which is how the reference obtains its backward direction
+    (mambapy/vim.py:228-261 for the block, mambapy/pscan.py:99-101 for the scan);
+  * sequences cut into segments, in the training form (checkpoints + backward), against the
+    float64 oracle and against the launch that is not cut;
+  * forward at d_state above 64;
+  * the bounded wait of the backward kernel failing loudly.
+All calls go through the C ABI."""
+import pytest
+import torch
+
+from oracle import c_oracle, scan_oracle as so
+from util import GRAD_KEYS, TOL, rel_err, run_gpu_fwd_bwd
+
+pytestmark = pytest.mark.gpu
+
+NAMES = ("x", "delta", "A", "B", "C", "D")
+TIME_KEYS = ("y", "dx", "ddelta", "dB", "dC")
+
+
+def _flip_time(inp):
+    return {k: (v.flip(1) if v.dim() == 3 else v) for k, v in inp.items()}
+
+
+def _reverse_oracle(inp):
+    """Gradients and output of the scan that runs from the last step to the first."""
+    ref = c_oracle.sscan_fwd_bwd(**_flip_time(inp))
+    return {k: (v.flip(1) if k in TIME_KEYS else v) for k, v in ref.items()}
+
+
+def _check(got, ref, tol, what):
+    for k in ("y",) + GRAD_KEYS:
+        e = rel_err(got[k], ref[k])
+        assert e <= tol, f"{what}: {k} rel err {e:.3e} > {tol}"
+
+
+# ---------------------------------------------------------------------------------------------
+# reverse direction of the fused scan
+# ---------------------------------------------------------------------------------------------
+
+@pytest.mark.parametrize("Bs,L,ED,N", [
+    (2, 64, 64, 16), (1, 1, 3, 16), (2, 37, 70, 16), (3, 129, 200, 12), (1, 250, 64, 4),
+    (2, 48, 64, 32), (1, 40, 65, 64),
+])
+def test_reverse_scan_equals_flip_scan_flip_fp32(pkg, dev, Bs, L, ED, N):
+    inp = so.make_inputs(Bs, L, ED, N, seed=900 + L + N)
+    ref = _reverse_oracle(inp)
+    got = run_gpu_fwd_bwd(pkg, inp, dev, reverse=True)
+    _check(got, ref, TOL[torch.float32], f"reverse B{Bs} L{L} ED{ED} N{N}")
+
+
+def test_reverse_scan_bf16_time_contiguous_and_sliced_BC(pkg, dev):
+    # the layouts MambaBlock.forward produces: (B, ED, L) memory viewed as (B, L, ED), and B, C
+    # as slices of one projection
+    Bs, L, ED, N, R = 2, 77, 100, 16, 7
+    inp = so.make_inputs(Bs, L, ED, N, seed=931, dtype=torch.bfloat16)
+    ref = _reverse_oracle(inp)
+    tm = lambda t: t.to(dev).transpose(1, 2).contiguous().transpose(1, 2).requires_grad_()
+    x, delta = tm(inp["x"]), tm(inp["delta"])
+    proj = torch.zeros(Bs, L, R + 2 * N, device=dev, dtype=torch.bfloat16)
+    proj[..., R:R + N] = inp["B"].to(dev)
+    proj[..., R + N:] = inp["C"].to(dev)
+    proj.requires_grad_()
+    _, Bm, C = torch.split(proj, [R, N, N], dim=-1)
+    A, D = inp["A"].to(dev).requires_grad_(), inp["D"].to(dev).requires_grad_()
+    y = pkg.selective_scan_fn(x, delta, A, Bm, C, D, reverse=True)
+    y.backward(inp["dy"].to(dev))
+    got = dict(y=y, dx=x.grad, ddelta=delta.grad, dA=A.grad, dD=D.grad,
+               dB=proj.grad[..., R:R + N], dC=proj.grad[..., R + N:])
+    _check(got, ref, TOL[torch.bfloat16], "reverse strided bf16")
+
+
+@pytest.mark.parametrize("general", [False, True])
+def test_reverse_gate_softplus_bias_h0_last_state(pkg, dev, general):
+    # every fused extra at once, both backward kernels; float64 autograd through the oracle's
+    # sequential scan on time-flipped inputs is the reference
+    Bs, L, ED, N = 2, 90, 80, 16
+    inp = so.make_inputs(Bs, L, ED, N, seed=951)
+    g = torch.Generator().manual_seed(952)
+    z = torch.randn(Bs, L, ED, generator=g)
+    raw = torch.randn(Bs, L, ED, generator=g) * 0.5 - 4.0
+    bias = torch.randn(ED, generator=g) * 0.3
+    h0 = torch.randn(Bs, ED, N, generator=g)
+    f64 = lambda t: t.double().requires_grad_()
+    x, r, A, Bm, C, D, zz, bb = map(f64, (inp["x"], raw, inp["A"], inp["B"], inp["C"], inp["D"], z, bias))
+    fl = lambda t: t.flip(1)
+    delta = so.softplus_ref(fl(r) + bb)
+    yr, hl = so.selective_scan_ref(fl(x), delta, A, fl(Bm), fl(C), D, h0=h0.double(), return_last_state=True)
+    yr = fl(yr) * (zz * torch.sigmoid(zz))
+    yr.backward(inp["dy"].double())
+    ref = dict(y=yr, dx=x.grad, ddelta=r.grad, dA=A.grad, dB=Bm.grad, dC=C.grad, dD=D.grad,
+               dz=zz.grad, dbias=bb.grad, hl=hl)
+    t = lambda v: v.to(dev).requires_grad_()
+    gx, gr, gA, gB, gC, gD, gz, gb = map(t, (inp["x"], raw, inp["A"], inp["B"], inp["C"], inp["D"], z, bias))
+    with pkg.plan_override(bwd_general=general):
+        y, h_last = pkg.selective_scan_fn(gx, gr, gA, gB, gC, gD, z=gz, delta_bias=gb, delta_softplus=True,
+                                          h0=h0.to(dev), return_last_state=True, reverse=True)
+        y.backward(inp["dy"].to(dev))
+    got = dict(y=y, dx=gx.grad, ddelta=gr.grad, dA=gA.grad, dB=gB.grad, dC=gC.grad, dD=gD.grad,
+               dz=gz.grad, dbias=gb.grad, hl=h_last)
+    for k in ref:
+        e = rel_err(got[k], ref[k])
+        assert e <= TOL[torch.float32], f"{k}: {e:.3e}"
+
+
+def test_bidirectional_pair_shares_inputs_without_copies(pkg, dev):
+    # what a bidirectional block computes (mambapy/vim.py:228-261): one scan per direction over
+    # the same tensors, the outputs added; checked against the two oracles
+    inp = so.make_inputs(2, 150, 96, 16, seed=971)
+    names = NAMES
+    ref_f = c_oracle.sscan_fwd_bwd(**inp)
+    ref_b = _reverse_oracle(inp)
+    args = [inp[k].to(dev).requires_grad_() for k in names]
+    y = pkg.selective_scan_fn(*args) + pkg.selective_scan_fn(*args, reverse=True)
+    y.backward(inp["dy"].to(dev))
+    got = dict(y=y, **{k: a.grad for k, a in zip(GRAD_KEYS, args)})
+    for k in ("y",) + GRAD_KEYS:
+        assert rel_err(got[k], ref_f[k] + ref_b[k]) <= TOL[torch.float32], k
+
+
+def test_reverse_wide_state_forward(pkg, dev):
+    # d_state 128: B and C reach the scan waves through the packed scalar-load path
+    inp = so.make_inputs(2, 70, 64, 128, seed=981)
+    fl = _flip_time(inp)
+    ref = c_oracle.sscan_fwd(*[fl[k] for k in NAMES]).flip(1)
+    with torch.no_grad():
+        y = pkg.selective_scan_fn(*[inp[k].to(dev) for k in NAMES], reverse=True)
+    assert rel_err(y, ref) <= TOL[torch.float32]
+
+
+# ---------------------------------------------------------------------------------------------
+# reverse direction of the generic scan (mambapy/pscan.py:94-149)
+# ---------------------------------------------------------------------------------------------
+
+@pytest.mark.parametrize("shape", [(2, 64, 8, 16), (1, 37, 5, 3), (2, 13, 16, 16), (1, 1, 4, 4)])
+def test_pscan_rev_forward_backward(pkg, dev, shape):
+    g = torch.Generator().manual_seed(sum(shape))
+    A = torch.rand(*shape, generator=g) * 0.9 + 0.05
+    X = torch.randn(*shape, generator=g)
+    G = torch.randn(*shape, generator=g)
+    Ar, Xr = A.double().requires_grad_(), X.double().requires_grad_()
+    Hr = so.linear_recurrence(Ar.flip(1), Xr.flip(1)).flip(1)   # pscan.py:99-101
+    Hr.backward(G.double())
+    Ag, Xg = A.to(dev).requires_grad_(), X.to(dev).requires_grad_()
+    H = pkg.pscan_rev(Ag, Xg)
+    H.backward(G.to(dev))
+    assert rel_err(H, Hr) <= 1e-5
+    assert rel_err(Xg.grad, Xr.grad) <= 1e-5
+    assert rel_err(Ag.grad, Ar.grad) <= 1e-5
+    # the last step has no successor: its A receives no gradient
+    assert torch.count_nonzero(Ag.grad[:, -1]) == 0
+
+
+def test_pscan_rev_on_transposed_views_bf16(pkg, dev):
+    # (B, D, L, N) memory viewed as (B, L, D, N), as the reference's transposed views are
+    shape = (2, 45, 24, 16)
+    g = torch.Generator().manual_seed(7)
+    A = (torch.rand(*shape, generator=g) * 0.9 + 0.05).to(torch.bfloat16)
+    X = torch.randn(*shape, generator=g).to(torch.bfloat16)
+    Hr = so.linear_recurrence(A.double().flip(1), X.double().flip(1)).flip(1)
+    tv = lambda t: t.to(dev).transpose(1, 2).contiguous().transpose(1, 2)
+    H = pkg.pscan_rev(tv(A), tv(X))
+    assert rel_err(H, Hr) <= TOL[torch.bfloat16]
+
+
+# ---------------------------------------------------------------------------------------------
+# sequences cut into segments, training form
+# ---------------------------------------------------------------------------------------------
+
+@pytest.mark.parametrize("Bs,L,ED,N,nseg,reverse", [
+    (1, 160, 64, 16, 2, False), (2, 100, 70, 16, 3, False), (1, 1000, 96, 16, 7, False),
+    (1, 333, 130, 8, 3, True), (2, 517, 64, 16, 7, True), (1, 48, 64, 16, 2, False),
+    (1, 16, 64, 16, 5, False),
+])
+def test_segmented_training_matches_oracle(pkg, dev, Bs, L, ED, N, nseg, reverse):
+    inp = so.make_inputs(Bs, L, ED, N, seed=400 + L + nseg)
+    ref = _reverse_oracle(inp) if reverse else c_oracle.sscan_fwd_bwd(**inp)
+    with pkg.plan_override(fwd_segments=nseg, bwd_segments=nseg):
+        got = run_gpu_fwd_bwd(pkg, inp, dev, reverse=reverse)
+        again = run_gpu_fwd_bwd(pkg, inp, dev, reverse=reverse)
+    _check(got, ref, TOL[torch.float32], f"nseg={nseg}")
+    for k in got:
+        assert torch.equal(got[k], again[k]), f"{k} not bitwise reproducible"
+    with pkg.plan_override(fwd_segments=1, bwd_segments=1):
+        one = run_gpu_fwd_bwd(pkg, inp, dev, reverse=reverse)
+    for k in got:
+        assert rel_err(got[k], one[k].double()) <= 2e-5, k
+
+
+@pytest.mark.parametrize("fwd_seg,bwd_seg", [(1, 4), (5, 1), (3, 7)])
+def test_forward_and_backward_may_be_cut_differently(pkg, dev, fwd_seg, bwd_seg):
+    # the backward needs the checkpoints only, which are indexed by tile whatever the cut
+    inp = so.make_inputs(1, 700, 128, 16, seed=455, dtype=torch.bfloat16)
+    ref = c_oracle.sscan_fwd_bwd(**inp)
+    with pkg.plan_override(fwd_segments=fwd_seg, bwd_segments=bwd_seg):
+        got = run_gpu_fwd_bwd(pkg, inp, dev)
+    _check(got, ref, TOL[torch.bfloat16], f"cuts {fwd_seg}/{bwd_seg}")
+
+
+def test_segmented_training_gated_softplus(pkg, dev):
+    Bs, L, ED, N = 1, 300, 80, 16
+    inp = so.make_inputs(Bs, L, ED, N, seed=461)
+    g = torch.Generator().manual_seed(462)
+    z = torch.randn(Bs, L, ED, generator=g)
+    raw = torch.randn(Bs, L, ED, generator=g) * 0.5 - 4.0
+    bias = torch.randn(ED, generator=g) * 0.3
+    h0 = torch.randn(Bs, ED, N, generator=g)
+    f64 = lambda t: t.double().requires_grad_()
+    x, r, A, Bm, C, D, zz, bb = map(f64, (inp["x"], raw, inp["A"], inp["B"], inp["C"], inp["D"], z, bias))
+    delta = so.softplus_ref(r + bb)
+    yr, hl = so.selective_scan_ref(x, delta, A, Bm, C, D, h0=h0.double(), return_last_state=True)
+    yr = yr * (zz * torch.sigmoid(zz))
+    yr.backward(inp["dy"].double())
+    ref = dict(y=yr, dx=x.grad, ddelta=r.grad, dA=A.grad, dB=Bm.grad, dC=C.grad, dD=D.grad,
+               dz=zz.grad, dbias=bb.grad, hl=hl)
+    t = lambda v: v.to(dev).requires_grad_()
+    gx, gr, gA, gB, gC, gD, gz, gb = map(t, (inp["x"], raw, inp["A"], inp["B"], inp["C"], inp["D"], z, bias))
+    with pkg.plan_override(fwd_segments=4, bwd_segments=3):
+        y, h_last = pkg.selective_scan_fn(gx, gr, gA, gB, gC, gD, z=gz, delta_bias=gb, delta_softplus=True,
+                                          h0=h0.to(dev), return_last_state=True)
+        y.backward(inp["dy"].to(dev))
+    got = dict(y=y, dx=gx.grad, ddelta=gr.grad, dA=gA.grad, dB=gB.grad, dC=gC.grad, dD=gD.grad,
+               dz=gz.grad, dbias=gb.grad, hl=h_last)
+    for k in ref:
+        e = rel_err(got[k], ref[k])
+        assert e <= TOL[torch.float32], f"{k}: {e:.3e}"
+
+
+def test_batch_one_training_is_cut_by_the_library(pkg, dev):
+    # the reference's published regime: batch 1, d_model 1024 (ED 2048), here 2048 steps in bf16.
+    # 32 workgroups would cover an eighth of the chip: both directions are cut without being asked
+    inp = so.make_inputs(1, 2048, 2048, 16, seed=471, dtype=torch.bfloat16)
+    ref = c_oracle.sscan_fwd_bwd(**inp)
+    got = run_gpu_fwd_bwd(pkg, inp, dev)
+    _check(got, ref, TOL[torch.bfloat16], "B=1 ED=2048")
+
+
+# ---------------------------------------------------------------------------------------------
+# forward at wide d_state
+# ---------------------------------------------------------------------------------------------
+
+@pytest.mark.parametrize("N,ED,L", [(96, 70, 50), (128, 64, 130), (256, 64, 40), (100, 130, 33)])
+def test_forward_wide_state(pkg, dev, N, ED, L):
+    # 64 < d_state <= 256: 16 or 32 states per lane, B and C packed for scalar loads
+    inp = so.make_inputs(2, L, ED, N, seed=500 + N)
+    g = torch.Generator().manual_seed(501 + N)
+    h0 = torch.randn(2, ED, N, generator=g)
+    ref, hl = c_oracle.sscan_fwd(*[inp[k] for k in NAMES], h0=h0.double(), return_last_state=True)
+    with torch.no_grad():
+        y, h_last = pkg.selective_scan_fn(*[inp[k].to(dev) for k in NAMES], h0=h0.to(dev),
+                                          return_last_state=True)
+    assert rel_err(y, ref) <= TOL[torch.float32]
+    assert rel_err(h_last, hl) <= TOL[torch.float32]
+
+
+# ---------------------------------------------------------------------------------------------
+# failure is loud
+# ---------------------------------------------------------------------------------------------
+
+def test_expired_wait_poisons_the_parameter_gradients(pkg, dev):
+    # The backward kernel waits, with a bound, for a counter in shared memory.  The test hook makes
+    # the kernel behave as if the bound had been reached (every wave still runs to its end): the
+    # call must not return clean-looking numbers.
+    inp = so.make_inputs(2, 100, 64, 16, seed=601)
+    with pkg.plan_override(expire_waits=True):
+        got = run_gpu_fwd_bwd(pkg, inp, dev)
+    assert torch.isnan(got["dA"]).all() and torch.isnan(got["dD"]).all()
+    clean = run_gpu_fwd_bwd(pkg, inp, dev)           # the flag is cleared by the next call
+    assert torch.isfinite(clean["dA"]).all() and torch.isfinite(clean["dD"]).all()

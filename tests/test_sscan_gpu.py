@@ -35,22 +35,20 @@ def test_ragged_shapes_fp32(pkg, dev, Bs, L, ED, N):
 
 
 @pytest.mark.parametrize("ns", [1, 2, 4])
-def test_every_state_split_agrees(pkg, dev, ns, monkeypatch):
+def test_every_state_split_agrees(pkg, dev, ns):
     # the wave decomposition (states per lane) is a tuning choice; every choice must agree
-    monkeypatch.setenv("MPA_FWD_NS", str(ns))
-    monkeypatch.setenv("MPA_BWD_NS", str(ns))
     inp = so.make_inputs(2, 200, 160, 16, seed=5)
     ref = c_oracle.sscan_fwd_bwd(**inp)
-    got = run_gpu_fwd_bwd(pkg, inp, dev)
+    with pkg.plan_override(fwd_states_per_lane=ns, bwd_states_per_lane=ns):
+        got = run_gpu_fwd_bwd(pkg, inp, dev)
     _check(got, ref, TOL[torch.float32], f"ns={ns}")
 
 
 @pytest.mark.parametrize("ns", [8, 16])
-def test_forward_wide_lanes(pkg, dev, ns, monkeypatch):
-    monkeypatch.setenv("MPA_FWD_NS", str(ns))
+def test_forward_wide_lanes(pkg, dev, ns):
     inp = so.make_inputs(2, 200, 160, 16, seed=6)
     ref = c_oracle.sscan_fwd(*[inp[k] for k in ("x", "delta", "A", "B", "C", "D")])
-    with torch.no_grad():
+    with torch.no_grad(), pkg.plan_override(fwd_states_per_lane=ns):
         y = pkg.selective_scan(*[inp[k].to(dev) for k in ("x", "delta", "A", "B", "C", "D")])
     assert rel_err(y, ref) <= TOL[torch.float32]
 
@@ -199,11 +197,11 @@ def test_gated_backward_bf16_and_time_contiguous(pkg, dev):
         assert e <= TOL[torch.bfloat16], f"{k}: {e:.3e}"
 
 
-def test_gated_backward_fast_equals_general_kernel(pkg, dev, monkeypatch):
+def test_gated_backward_fast_equals_general_kernel(pkg, dev):
     # the two backward kernels (saved pre-gate output vs recomputed one) must agree
     a, _ = _gated_case(pkg, dev, 2, 80, 128, 16, torch.float32, 321)
-    monkeypatch.setenv("MPA_BWD_GENERAL", "1")
-    b, _ = _gated_case(pkg, dev, 2, 80, 128, 16, torch.float32, 321)
+    with pkg.plan_override(bwd_general=True):
+        b, _ = _gated_case(pkg, dev, 2, 80, 128, 16, torch.float32, 321)
     for k in a:
         assert rel_err(a[k], b[k]) <= 2e-6, k
 
@@ -267,20 +265,19 @@ def _inference_case(pkg, dev, Bs, L, ED, N, dtype, seed, gated):
     (1, 160, 64, 16, 3, False), (2, 100, 70, 16, 4, True), (1, 37, 130, 8, 2, False),
     (1, 1000, 96, 16, 7, True), (3, 64, 64, 4, 4, False), (1, 16, 64, 16, 5, False), (1, 33, 5, 16, 64, True),
 ])
-def test_segmented_forward_matches_oracle_and_single_pass(pkg, dev, Bs, L, ED, N, nseg, gated, monkeypatch):
+def test_segmented_forward_matches_oracle_and_single_pass(pkg, dev, Bs, L, ED, N, nseg, gated):
     # inference form (no checkpoints) with the sequence cut into segments that run side by side
-    monkeypatch.setenv("MPA_FWD_NSEG", str(nseg))
-    y, hg, yr, hl = _inference_case(pkg, dev, Bs, L, ED, N, torch.float32, 300 + L, gated)
+    with pkg.plan_override(fwd_segments=nseg):
+        y, hg, yr, hl = _inference_case(pkg, dev, Bs, L, ED, N, torch.float32, 300 + L, gated)
     assert rel_err(y, yr) <= TOL[torch.float32]
     assert rel_err(hg, hl) <= TOL[torch.float32]
-    monkeypatch.setenv("MPA_FWD_NSEG", "1")
-    y1, h1, _, _ = _inference_case(pkg, dev, Bs, L, ED, N, torch.float32, 300 + L, gated)
+    with pkg.plan_override(fwd_segments=1):
+        y1, h1, _, _ = _inference_case(pkg, dev, Bs, L, ED, N, torch.float32, 300 + L, gated)
     assert rel_err(y, y1.double()) <= 1e-5 and rel_err(hg, h1.double()) <= 1e-5
 
 
-def test_segmented_forward_is_picked_for_a_single_long_sequence(pkg, dev, monkeypatch):
+def test_segmented_forward_is_picked_for_a_single_long_sequence(pkg, dev):
     # batch 1, 24 channel groups, 4096 steps in bf16: the library cuts the sequence by itself
-    monkeypatch.delenv("MPA_FWD_NSEG", raising=False)
     y, hg, yr, hl = _inference_case(pkg, dev, 1, 4096, 1536, 16, torch.bfloat16, 77, True)
     assert rel_err(y, yr) <= TOL[torch.bfloat16]
     assert rel_err(hg, hl) <= TOL[torch.float32]
@@ -288,7 +285,7 @@ def test_segmented_forward_is_picked_for_a_single_long_sequence(pkg, dev, monkey
     bc = torch.empty(1, 4096, 16, dtype=torch.bfloat16, device=dev)
     shape = pkg.scan._sscan_shape(big, big, bc, big, big, bc, 16, 0)
     import ctypes
-    need = pkg._lib.load().mpa_sscan_fwd_workspace_bytes(ctypes.byref(shape))
+    need = pkg._lib.load().mpa_sscan_fwd_workspace_bytes(ctypes.byref(shape), 0)
     assert need > 2 * 10 * 1536 * 16 * 4  # room for the states of 10 segments
 
 
@@ -316,12 +313,11 @@ def test_chunk_split_consistency_with_carried_state(pkg, dev):
     assert rel_err(h2, h_full) <= 1e-6
 
 
-def test_long_sequence_fp32_and_segmented_inference(pkg, dev, monkeypatch):
+def test_long_sequence_fp32_and_segmented_inference(pkg, dev):
     # 50 000 steps, far beyond the benchmark shapes (the reference materialises (B, L, ED, N)
     # tensors and pads L to a power of two, pscan.py:165-174): forward + backward
     # against the float64 C oracle, then the same forward without gradients, which the library
     # cuts into parallel segments by itself (one batch row, two channel groups)
-    monkeypatch.delenv("MPA_FWD_NSEG", raising=False)
     inp = so.make_inputs(1, 50000, 96, 16, seed=4242)
     ref = c_oracle.sscan_fwd_bwd(**inp)
     got = run_gpu_fwd_bwd(pkg, inp, dev)
