@@ -135,6 +135,24 @@ int64_t mpa_sscan_ckpt_elems(const mpa_sscan_shape* s);
  * h_ckpt, 0 for one that does not (the two are cut differently). */
 size_t mpa_sscan_fwd_workspace_bytes(const mpa_sscan_shape* s, int with_ckpt);
 
+/* ---- fused selective scan, forward, for callers that cannot allocate ------------------------
+ * No counterpart in the reference.  It is for callers that cannot provide a workspace because they
+ * cannot call hipMalloc: code under HIP graph capture, tight serving loops, harnesses that forbid
+ * allocation.  Same arguments and results as mpa_sscan_fwd (bit for bit) without `workspace`: the
+ * scratch is a static device array of MPA_NOALLOC_SCRATCH_BYTES that the library owns, one copy on
+ * every GPU it runs on, held until the process ends.  The call allocates and frees nothing.
+ * A shape whose mpa_sscan_fwd_workspace_bytes() exceeds MPA_NOALLOC_SCRATCH_BYTES is refused with
+ * MPA_ERR_WORKSPACE before anything is launched (sequences cut into segments need
+ * 2 * batch * segments * dim * dstate floats and a little more; d_state above 64 needs the packed
+ * B/C of the whole sequence).  All calls on one GPU share that GPU's array: calls that overlap
+ * on one GPU (different streams or threads) race; calls on one stream are ordered.
+ */
+#define MPA_NOALLOC_SCRATCH_BYTES (16u << 20)
+int mpa_sscan_fwd_noalloc(const mpa_sscan_shape* s, const void* x, const void* delta, const float* A,
+                          const void* B, const void* C, const float* D, const void* z,
+                          const float* delta_bias, const float* h0, void* y, void* y_pregate,
+                          float* h_ckpt, float* h_last, void* stream);
+
 /* ---- fused selective scan, backward -----------------------------------------------------
  * Replaces what autograd records for mamba.py:284-293 plus PScan.backward
  * (mambapy/pscan.py:188-224): given dy it writes dx, ddelta (io_dtype), dB, dC (io_dtype),

@@ -18,7 +18,9 @@ MPA_CONV_SILU = 1
 MPA_CKPT_STEPS = 16
 MPA_MAX_DSTATE = 256
 
-EXPORTS = ("mpa_version", "mpa_arch", "mpa_status_string", "mpa_sscan_fwd",
+MPA_NOALLOC_SCRATCH_BYTES = 16 << 20
+
+EXPORTS = ("mpa_version", "mpa_arch", "mpa_status_string", "mpa_sscan_fwd", "mpa_sscan_fwd_noalloc",
            "mpa_sscan_ckpt_elems", "mpa_sscan_fwd_workspace_bytes", "mpa_sscan_bwd", "mpa_sscan_bwd_workspace_bytes",
            "mpa_pscan_fwd", "mpa_pscan_bwd", "mpa_ssm_step",
            "mpa_conv1d_fwd", "mpa_conv1d_bwd", "mpa_conv1d_bwd_workspace_bytes",
@@ -70,6 +72,7 @@ def load():
     lib.mpa_status_string.argtypes = [ctypes.c_int]
     sp = ctypes.POINTER(SscanShape)
     lib.mpa_sscan_fwd.argtypes = [sp] + [vp] * 14 + [sz, vp]
+    lib.mpa_sscan_fwd_noalloc.argtypes = [sp] + [vp] * 13 + [vp]
     lib.mpa_sscan_fwd_workspace_bytes.argtypes = [sp, ctypes.c_int]
     lib.mpa_sscan_fwd_workspace_bytes.restype = sz
     lib.mpa_sscan_ckpt_elems.argtypes = [sp]

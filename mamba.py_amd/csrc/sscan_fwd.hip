@@ -785,11 +785,11 @@ extern "C" size_t mpa_sscan_fwd_workspace_bytes(const mpa_sscan_shape* s, int wi
     return (bcpack_floats(s) * sizeof(float) + 255) / 256 * 256;
 }
 
-extern "C" int mpa_sscan_fwd(const mpa_sscan_shape* s, const void* x, const void* delta,
-                             const float* A, const void* B, const void* C, const float* D,
-                             const void* z, const float* delta_bias, const float* h0, void* y,
-                             void* y_pregate, float* h_ckpt, float* h_last, void* workspace,
-                             size_t workspace_bytes, void* stream) {
+static int sscan_fwd_impl(const mpa_sscan_shape* s, const void* x, const void* delta,
+                          const float* A, const void* B, const void* C, const float* D,
+                          const void* z, const float* delta_bias, const float* h0, void* y,
+                          void* y_pregate, float* h_ckpt, float* h_last, void* workspace,
+                          size_t workspace_bytes, void* stream) {
     int rc = validate_shape(s);
     if (rc != MPA_OK) return rc;
     if (!x || !delta || !A || !B || !C || !D || !y || !workspace) return MPA_ERR_NULL_POINTER;
@@ -845,4 +845,56 @@ extern "C" int mpa_sscan_fwd(const mpa_sscan_shape* s, const void* x, const void
     p2.nseg = sp.nseg; p2.seg_tiles = sp.seg_tiles;
     p2.h0 = wsf + sp.off_h0; p2.hlast = nullptr;
     return launch_fwd_any(p2, s->io_dtype, ns, nw, kScan, st);
+}
+
+extern "C" int mpa_sscan_fwd(const mpa_sscan_shape* s, const void* x, const void* delta,
+                             const float* A, const void* B, const void* C, const float* D,
+                             const void* z, const float* delta_bias, const float* h0, void* y,
+                             void* y_pregate, float* h_ckpt, float* h_last, void* workspace,
+                             size_t workspace_bytes, void* stream) {
+    return sscan_fwd_impl(s, x, delta, A, B, C, D, z, delta_bias, h0, y, y_pregate, h_ckpt, h_last, workspace,
+                          workspace_bytes, stream);
+}
+
+// ---- the entry point that allocates nothing -------------------------------------------------
+// Scratch of mpa_sscan_fwd_noalloc: device memory that belongs to the library's code object, one
+// copy per GPU the library is loaded on, held until the process ends.  In host code the name
+// below is only a handle for hipGetSymbolAddress; the device address it yields (different on
+// every GPU) is what goes to the kernels.
+static __device__ __align__(256) unsigned char scratch[MPA_NOALLOC_SCRATCH_BYTES];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::atomic<void*> g_scratch_ptr[kMaxDevices];
+
+// device address of `scratch` on the current device, resolved once per device
+int scratch_address(void** out) {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return MPA_ERR_LAUNCH;
+    void* ptr = g_scratch_ptr[dev].load(std::memory_order_acquire);
+    if (!ptr) {
+        if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess || !ptr) return MPA_ERR_LAUNCH;
+        g_scratch_ptr[dev].store(ptr, std::memory_order_release);
+    }
+    *out = ptr;
+    return MPA_OK;
+}
+}  // namespace
+
+extern "C" int mpa_sscan_fwd_noalloc(const mpa_sscan_shape* s, const void* x, const void* delta,
+                                     const float* A, const void* B, const void* C, const float* D,
+                                     const void* z, const float* delta_bias, const float* h0, void* y,
+                                     void* y_pregate, float* h_ckpt, float* h_last, void* stream) {
+    const int rc = validate_shape(s);
+    if (rc != MPA_OK) return rc;
+    // the scratch the call needs is a function of the shape alone: too large a call is refused
+    // before anything touches the device
+    if (mpa_sscan_fwd_workspace_bytes(s, h_ckpt != nullptr) > MPA_NOALLOC_SCRATCH_BYTES) return MPA_ERR_WORKSPACE;
+    void* ptr = nullptr;
+    const int arc = scratch_address(&ptr);
+    if (arc != MPA_OK) return arc;
+    // Nothing in the scratch has to start at zero: every word the kernels read (segment end
+    // states, sums of delta, packed B/C) is written earlier in the same call.
+    return sscan_fwd_impl(s, x, delta, A, B, C, D, z, delta_bias, h0, y, y_pregate, h_ckpt, h_last, ptr,
+                          MPA_NOALLOC_SCRATCH_BYTES, stream);
 }
