@@ -44,16 +44,19 @@ def algorithmic_bytes(B, L, ED, N, s):
     return fwd, bwd
 
 
-def cpu_baseline(workload, torch, so):
+def cpu_baseline(workload, torch):
     """Time the reference's pure-PyTorch path (materialised tensors + Blelloch scan,
     forward + backward, float32, all host threads) on a slice of the workload's channels:
     channels are independent, so the slice is the same work per channel."""
     B, L, ED, N, _, seed, _ = WORKLOADS[workload]
     ed = min(ED, 512 if workload != "c0" else ED)
     bs = min(B, 2)
+    # the checker is imported here only: this leg times it, nothing else in the benchmark uses it
+    from oracle import scan_oracle as so
+    import synthetic_inputs
     threads = int(os.environ.get("OMP_NUM_THREADS") or os.cpu_count() or 1)
     torch.set_num_threads(threads)
-    inp = so.make_inputs(bs, L, ed, N, seed=seed)
+    inp = synthetic_inputs.make_inputs(bs, L, ed, N, seed=seed)
     names = ("x", "delta", "A", "B", "C", "D")
 
     def once():
@@ -355,6 +358,68 @@ def bench_generate(args, torch, pkg, dev):
     print(json.dumps(out))
 
 
+def bench_thin(args, torch, pkg, dev):
+    """Launches that offer few workgroups: the reference's published regime is batch 1
+    (README.md:203-204).  (a) fused scan forward + backward at B=1, L=4096, d_model 1024
+    (ED 2048), N=16, bf16: 32 workgroups of 64 channels on 256 CUs unless the sequence is cut;
+    (b) generic pscan forward + backward at B=1, L=65536, d_model 16 (ED 32), N=16, fp32: 512
+    lanes.  Each is timed as the library runs it (cut into segments) and with the cut switched
+    off through the launch plan."""
+    import synthetic_inputs
+    steps, warmup = max(3, args.steps // 5), 2
+    rows = {}
+
+    B, L, ED, N = 1, 4096, 2048, 16
+    inp = synthetic_inputs.make_inputs(B, L, ED, N, seed=1010, dtype=torch.bfloat16)
+    gpu = [inp[k].to(dev).requires_grad_() for k in ("x", "delta", "A", "B", "C", "D")]
+    dy = inp["dy"].to(dev)
+
+    def sscan_step():
+        for a in gpu:
+            a.grad = None
+        pkg.selective_scan_fn(*gpu).backward(dy)
+
+    fwd_b, bwd_b = algorithmic_bytes(B, L, ED, N, 2)
+    t_cut = _timed(torch, sscan_step, steps, warmup)
+    with pkg.plan_override(fwd_segments=1, bwd_segments=1):
+        t_one = _timed(torch, sscan_step, steps, warmup)
+    rows["sscan_B1_L4096_ED2048_bf16"] = {
+        "ms_cut": t_cut * 1e3, "ms_not_cut": t_one * 1e3, "speedup": t_one / t_cut,
+        "GBps_cut": (fwd_b + bwd_b) / t_cut / 1e9, "tokens_per_s_cut": B * L / t_cut}
+
+    B, L, ED, N = 1, 65536, 32, 16
+    g = torch.Generator().manual_seed(1011)
+    A = (1.0 - torch.rand(B, L, ED, N, generator=g) * 0.05).to(dev).requires_grad_()
+    X = torch.randn(B, L, ED, N, generator=g).to(dev).requires_grad_()
+    gH = torch.randn(B, L, ED, N, generator=g).to(dev)
+
+    def pscan_step():
+        A.grad = None
+        X.grad = None
+        pkg.pscan(A, X).backward(gH)
+
+    S = B * L * ED * N * 4
+    t_cut = _timed(torch, pscan_step, steps, warmup)
+    with pkg.plan_override(pscan_chunks=1):
+        t_one = _timed(torch, pscan_step, max(2, steps // 2), 1)
+    rows["pscan_B1_L65536_ED32_f32"] = {
+        "ms_cut": t_cut * 1e3, "ms_not_cut": t_one * 1e3, "speedup": t_one / t_cut,
+        "GBps_cut": 8 * S / t_cut / 1e9}
+
+    head = rows["sscan_B1_L4096_ED2048_bf16"]
+    out = {
+        "metric": "selective-scan fwd+bwd GB/s at batch 1 (B=1 L=4096 ED=2048 N=16 bf16), sequence cut into segments",
+        "value": head["GBps_cut"], "unit": "GB/s", "higher_is_better": True,
+        "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": head["ms_cut"],
+        "scaling": "weak", "vs_baseline": None, "dtype": "f32 state/accumulation, bf16 I/O",
+        "data": "synthetic (seeded)",
+        "config": {"workload": "batch-1 launches: fused scan B=1 L=4096 ED=2048; generic pscan B=1 L=65536 ED=32"},
+        "rows": rows,
+    }
+    print(json.dumps(out))
+    return out
+
+
 def bench_lm_forward(args, torch, pkg, dev, L):
     """configs[4]: random-init LM forward at the mamba-130m architecture, bf16 weights and
     activations, fp32 scan state, B=8, uniform-random token ids."""
@@ -389,7 +454,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS) + ["c3", "c4", "c4-3000", "pscan", "layer", "generate"],
+    ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS) + ["c3", "c4", "c4-3000", "pscan", "layer", "generate", "thin"],
                     help="c2 (default) is the headline workload; c3 = decode step, c4 = LM forward "
                          "(reported with their own metric, same one-line schema)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -403,7 +468,7 @@ def main():
 
     import torch
     import __graft_entry__ as entry
-    from oracle import scan_oracle as so
+    import synthetic_inputs
     pkg = entry.load_package()
     if not torch.cuda.is_available():
         sys.exit("bench.py: no GPU visible")
@@ -417,12 +482,14 @@ def main():
         return bench_layer_kernels(args, torch, pkg, dev)
     if args.workload == "generate":
         return bench_generate(args, torch, pkg, dev)
+    if args.workload == "thin":
+        return bench_thin(args, torch, pkg, dev)
     if args.workload.startswith("c4"):
         return bench_lm_forward(args, torch, pkg, dev, 3000 if args.workload == "c4-3000" else 4096)
 
     B, L, ED, N, dtname, seed, desc = WORKLOADS[args.workload]
     dtype = getattr(torch, dtname)
-    inp = so.make_inputs(B, L, ED, N, seed=seed, dtype=dtype)
+    inp = synthetic_inputs.make_inputs(B, L, ED, N, seed=seed, dtype=dtype)
     names = ("x", "delta", "A", "B", "C", "D")
     gpu = [inp[k].to(dev).requires_grad_() for k in names]
     dy = inp["dy"].to(dev)
@@ -491,7 +558,7 @@ def main():
                     "frac": fwd_b / (fwd_ms * 1e-3) / 1e9 / HBM_PEAK_GBS},
     }
     if not args.no_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline(args.workload, torch, so)
+        out["cpu_baseline"] = cpu_baseline(args.workload, torch)
     print(json.dumps(out))
 
 

@@ -168,7 +168,7 @@ int mpa_sscan_fwd_noalloc(const mpa_sscan_shape* s, const void* x, const void* d
  * the forward call (the carry runs from the end).
  * One kernel waits, with a bound, for a counter in shared memory; the wait cannot run out
  * unless the hardware scheduler misbehaves, and if it ever does the call does not return clean
- * numbers: every element of dA, dD (and ddelta_bias) is then NaN.
+ * numbers: dA of every channel whose sums may have been damaged is NaN.
  */
 int mpa_sscan_bwd(const mpa_sscan_shape* s, const void* x, const void* delta, const float* A,
                   const void* B, const void* C, const float* D, const void* z,
@@ -242,6 +242,11 @@ size_t mpa_rmsnorm_bwd_workspace_bytes(int64_t rows, int64_t d);
  * set per tensor; any seqlen.  H is a new tensor: inputs are never modified
  * (pscan.py:167-174 clones).  Backward: gradX[t] = gradH[t] + A[t+1]*gradX[t+1],
  * gradA[t] = H[t-1]*gradX[t], gradA[0] = 0 (pscan.py:216-222).
+ * The reference's scan has O(log L) depth at any batch size (pscan.py:36-92); here one lane owns
+ * one (dim, dstate) recurrence, and when batch*dim*dstate offers too few lanes to keep the memory
+ * system busy the sequence is cut into pieces that run side by side (aggregate pass, carry pass,
+ * main pass).  `workspace` (mpa_pscan_workspace_bytes() bytes, 256-byte aligned) holds the
+ * per-piece aggregates; contents are dead after the call.
  */
 typedef struct mpa_pscan_shape {
     int64_t batch, seqlen, dim, dstate;
@@ -252,11 +257,15 @@ typedef struct mpa_pscan_shape {
     int64_t h_st[4];          /* H (output of fwd, input of bwd) */
     int64_t ga_st[4];         /* gradA */
     int64_t gx_st[4];         /* gradX */
+    int32_t plan_chunks;      /* pieces the sequence is cut into; 0 = chosen from the shape, 1 = never cut */
+    int32_t reserved;         /* 0 */
 } mpa_pscan_shape;
 
-int mpa_pscan_fwd(const mpa_pscan_shape* s, const void* A, const void* X, void* H, void* stream);
+size_t mpa_pscan_workspace_bytes(const mpa_pscan_shape* s);
+int mpa_pscan_fwd(const mpa_pscan_shape* s, const void* A, const void* X, void* H, void* workspace,
+                  size_t workspace_bytes, void* stream);
 int mpa_pscan_bwd(const mpa_pscan_shape* s, const void* A, const void* H, const void* gradH,
-                  void* gradA, void* gradX, void* stream);
+                  void* gradA, void* gradX, void* workspace, size_t workspace_bytes, void* stream);
 
 /* ---- decode step --------------------------------------------------------------------------
  * Replaces the state update and readout of MambaBlock.ssm_step (mambapy/mamba.py:400-412)

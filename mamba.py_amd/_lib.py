@@ -22,7 +22,7 @@ MPA_NOALLOC_SCRATCH_BYTES = 16 << 20
 
 EXPORTS = ("mpa_version", "mpa_arch", "mpa_status_string", "mpa_sscan_fwd", "mpa_sscan_fwd_noalloc",
            "mpa_sscan_ckpt_elems", "mpa_sscan_fwd_workspace_bytes", "mpa_sscan_bwd", "mpa_sscan_bwd_workspace_bytes",
-           "mpa_pscan_fwd", "mpa_pscan_bwd", "mpa_ssm_step",
+           "mpa_pscan_fwd", "mpa_pscan_bwd", "mpa_pscan_workspace_bytes", "mpa_ssm_step",
            "mpa_conv1d_fwd", "mpa_conv1d_bwd", "mpa_conv1d_bwd_workspace_bytes",
            "mpa_rmsnorm_fwd", "mpa_rmsnorm_bwd", "mpa_rmsnorm_bwd_workspace_bytes")
 
@@ -46,7 +46,8 @@ class ConvShape(ctypes.Structure):
 class PscanShape(ctypes.Structure):
     _fields_ = [(n, ctypes.c_int64) for n in ("batch", "seqlen", "dim", "dstate")] + \
                [("io_dtype", ctypes.c_int32), ("reverse", ctypes.c_int32)] + \
-               [(n, ctypes.c_int64 * 4) for n in ("a_st", "x_st", "h_st", "ga_st", "gx_st")]
+               [(n, ctypes.c_int64 * 4) for n in ("a_st", "x_st", "h_st", "ga_st", "gx_st")] + \
+               [("plan_chunks", ctypes.c_int32), ("reserved", ctypes.c_int32)]
 
 
 _lib = None
@@ -81,8 +82,10 @@ def load():
     lib.mpa_sscan_bwd_workspace_bytes.argtypes = [sp]
     lib.mpa_sscan_bwd_workspace_bytes.restype = sz
     pp = ctypes.POINTER(PscanShape)
-    lib.mpa_pscan_fwd.argtypes = [pp] + [vp] * 4
-    lib.mpa_pscan_bwd.argtypes = [pp] + [vp] * 6
+    lib.mpa_pscan_workspace_bytes.argtypes = [pp]
+    lib.mpa_pscan_workspace_bytes.restype = sz
+    lib.mpa_pscan_fwd.argtypes = [pp] + [vp] * 4 + [sz, vp]
+    lib.mpa_pscan_bwd.argtypes = [pp] + [vp] * 6 + [sz, vp]
     lib.mpa_ssm_step.argtypes = [vp] * 11 + [i64] * 5 + [i32, i32, vp]
     cp = ctypes.POINTER(ConvShape)
     lib.mpa_conv1d_fwd.argtypes = [cp] + [vp] * 7

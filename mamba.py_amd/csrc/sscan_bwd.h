@@ -32,10 +32,15 @@ struct BwdParams {
     // every segment from the one visited before it (NULL = zeros: not cut)
     const float* ag0;
     int nseg, seg_tiles;
-    int* status;       // device word: set to 1 when a bounded wait inside the kernel runs out
     int expire_waits;  // test hook: treat every bounded wait as run out
     int reverse;       // the forward walk ran from the last physical step to the first
     int batch, L, ED, N, nchunks;
+    // d_state above 64 runs as several passes over blocks of 64 states (general kernel only):
+    // N = states of this pass, Nst = states of the whole call = row stride of every array indexed
+    // by state (A, h0, checkpoints, partA/B/C; their pointers are advanced to the block's first
+    // state by the host); a pass after the first adds its share to dx, ddelta, dz instead of
+    // overwriting them and contributes nothing to dD; row0 = its first row in partD / partDb
+    int Nst, accumulate, row0;
     int softplus;
     int in_tmajor, dy_tmajor, out_tmajor;
     int64_t u_sb, u_sl, u_sd;

@@ -92,7 +92,7 @@ __global__ void __launch_bounds__(NW* kWave) sscan_bwd_kernel(const BwdParams p)
 #pragma unroll
     for (int i = 0; i < NS; ++i) {
         const int n = w * NS + i;
-        A2[i] = (dvalid && n < p.N) ? p.A[(int64_t)d * p.N + n] * kLog2e : 0.0f;
+        A2[i] = (dvalid && n < p.N) ? p.A[(int64_t)d * p.Nst + n] * kLog2e : 0.0f;
         ag[i] = 0.0f;
         dAacc[i] = 0.0f;
     }
@@ -159,9 +159,9 @@ __global__ void __launch_bounds__(NW* kWave) sscan_bwd_kernel(const BwdParams p)
             float hv = 0.0f;
             if (dvalid && n < p.N) {
                 if (c > 0)
-                    hv = p.ckpt[(((int64_t)b * p.nchunks + (c - 1)) * p.N + n) * p.ED + d];
+                    hv = p.ckpt[(((int64_t)b * p.nchunks + (c - 1)) * p.Nst + n) * p.ED + d];
                 else if (p.h0)
-                    hv = p.h0[((int64_t)b * p.ED + d) * p.N + n];
+                    hv = p.h0[((int64_t)b * p.ED + d) * p.Nst + n];
             }
             rH[i] = hv;
         }
@@ -282,7 +282,7 @@ __global__ void __launch_bounds__(NW* kWave) sscan_bwd_kernel(const BwdParams p)
                     const int n = w * NS + (o % NS);
                     if (part == 0 && t < p.L && n < p.N) {
                         float* dst = (o < NS) ? p.partB : p.partC;
-                        dst[cg * p.part_gs + ((int64_t)b * p.L + t) * p.N + n] = s;
+                        dst[cg * p.part_gs + ((int64_t)b * p.L + t) * p.Nst + n] = s;
                     }
                     wave_lds_sync();
                 }
@@ -315,28 +315,36 @@ __global__ void __launch_bounds__(NW* kWave) sscan_bwd_kernel(const BwdParams p)
                     const float Dv = p.D[d0 + cc];
                     const int64_t t = t0 + phys_step(tt);
                     const int64_t ch = d0 + cc;
-                    const float dxv = __builtin_fmaf(dv, gB, Dv * dyg);
+                    // (a later pass over another block of states adds dv * gB only: D*dy and dD
+                    // belong to the first)
+                    float dxv = __builtin_fmaf(dv, gB, p.accumulate ? 0.0f : Dv * dyg);
                     float ddv = __builtin_fmaf(xv, gB, dd * kLn2);
-                    dDacc[seg * EPS + k] = __builtin_fmaf(dyg, xv, dDacc[seg * EPS + k]);
+                    if (!p.accumulate) dDacc[seg * EPS + k] = __builtin_fmaf(dyg, xv, dDacc[seg * EPS + k]);
                     if (p.softplus) {
                         // d softplus(r)/dr = sigmoid(r) = 1 - exp(-softplus(r))
                         ddv *= (1.0f - __expf(-dv));
                         dDbacc[seg * EPS + k] += ddv;
                     }
-                    store_from_float<IO>(p.dx, b * p.g_sb + t * p.g_sl + ch * p.g_sd, dxv);
-                    store_from_float<IO>(p.ddelta, b * p.g_sb + t * p.g_sl + ch * p.g_sd, ddv);
+                    const int64_t go = b * p.g_sb + t * p.g_sl + ch * p.g_sd;
+                    if (p.accumulate) {
+                        dxv += load_as_float<IO>(p.dx, go);
+                        ddv += load_as_float<IO>(p.ddelta, go);
+                    }
+                    store_from_float<IO>(p.dx, go, dxv);
+                    store_from_float<IO>(p.ddelta, go, ddv);
                     if (HAS_Z) {
                         float yp = 0.0f;
 #pragma unroll
                         for (int ww = 0; ww < NW; ++ww) yp += sP3[ww][ts][cc];
-                        yp = __builtin_fmaf(Dv, xv, yp);  // pre-gate output
+                        if (!p.accumulate) yp = __builtin_fmaf(Dv, xv, yp);  // pre-gate output
                         const float zv =
                             load_as_float<IO>(p.z, b * p.z_sb + t * p.z_sl + ch * p.z_sd);
                         const float sg = sigmoid_f(zv);
                         const float dyraw = sZg[0][tt][cc];
                         // d(z*sigmoid(z))/dz = sg * (1 + z*(1-sg))
-                        const float dzv = dyraw * yp * sg * (1.0f + zv * (1.0f - sg));
-                        store_from_float<IO>(p.dz, b * p.g_sb + t * p.g_sl + ch * p.g_sd, dzv);
+                        float dzv = dyraw * yp * sg * (1.0f + zv * (1.0f - sg));
+                        if (p.accumulate) dzv += load_as_float<IO>(p.dz, go);
+                        store_from_float<IO>(p.dz, go, dzv);
                     }
                 }
             }
@@ -349,7 +357,7 @@ __global__ void __launch_bounds__(NW* kWave) sscan_bwd_kernel(const BwdParams p)
 #pragma unroll
         for (int i = 0; i < NS; ++i) {
             const int n = w * NS + i;
-            if (n < p.N) p.partA[((int64_t)b * p.ED + d) * p.N + n] = dAacc[i];
+            if (n < p.N) p.partA[((int64_t)b * p.ED + d) * p.Nst + n] = dAacc[i];
         }
     }
     // dD: every thread holds sums for its fixed (step slot, channel) elements; reduce over
@@ -379,21 +387,21 @@ __global__ void __launch_bounds__(NW* kWave) sscan_bwd_kernel(const BwdParams p)
 #pragma unroll
             for (int tt = 0; tt < kTile; ++tt) s += sDelta[0][tt][tid];
             float* dst = pass == 0 ? p.partD : p.partDb;
-            dst[(int64_t)b * p.ED + d0 + tid] = s;
+            dst[(int64_t)(p.row0 + b) * p.ED + d0 + tid] = s;
         }
         __syncthreads();
     }
 }
 
-// Sums the partial buffers: dB/dC over channel groups, dA/dD/ddelta_bias over the rows of the
-// main launch (batch rows, or their segments).  V = 4: d_state is a multiple of 4, a thread sums
-// four consecutive states with 16-byte loads.  `status` is the word the main kernel sets when one
-// of its bounded waits ran out: the parameter gradients are then NaN, never silently wrong.
+// Sums the partial buffers: dB/dC over channel groups, dA over its rows_a rows (batch rows, or
+// their segments), dD/ddelta_bias over their rows_d rows (the same, or batch rows times the state
+// blocks of a wide d_state).  V = 4: d_state is a multiple of 4, a thread sums
+// four consecutive states with 16-byte loads.
 template <typename IO, int V>
 __global__ void __launch_bounds__(256) sscan_bwd_finish_kernel(
     const float* partB, const float* partC, const float* partA, const float* partD,
     const float* partDb, void* dB, void* dC, float* dA, float* dD, float* dDb, int CG, int64_t gs,
-    int batch, int rows, int L, int ED, int N, int64_t dbc_sb, int64_t dbc_sl, const int* status) {
+    int batch, int rows_a, int rows_d, int L, int ED, int N, int64_t dbc_sb, int64_t dbc_sl) {
     const int64_t bln = (int64_t)batch * L * N;
     const int64_t edn = (int64_t)ED * N;
     const int64_t nbc = bln / V;  // threads of the dB/dC part
@@ -451,18 +459,17 @@ __global__ void __launch_bounds__(256) sscan_bwd_finish_kernel(
     } else if (i < bln + edn) {
         const int64_t j = i - bln;
         float s = 0.0f;
-        for (int bb = 0; bb < rows; ++bb) s += partA[bb * edn + j];
-        dA[j] = *status ? __builtin_nanf("") : s;
+        for (int bb = 0; bb < rows_a; ++bb) s += partA[bb * edn + j];
+        dA[j] = s;
     } else if (i < bln + edn + ED) {
         const int64_t j = i - bln - edn;
         float s = 0.0f, sdb = 0.0f;
-        for (int bb = 0; bb < rows; ++bb) {
+        for (int bb = 0; bb < rows_d; ++bb) {
             s += partD[(int64_t)bb * ED + j];
             if (dDb) sdb += partDb[(int64_t)bb * ED + j];
         }
-        const bool failed = *status != 0;
-        dD[j] = failed ? __builtin_nanf("") : s;
-        if (dDb) dDb[j] = failed ? __builtin_nanf("") : sdb;
+        dD[j] = s;
+        if (dDb) dDb[j] = sdb;
     }
 }
 
@@ -482,18 +489,23 @@ static SegPlan bwd_seg_plan(const mpa_sscan_shape* s) {
     return seg_plan(s, ns, kBwdThin);
 }
 
+constexpr int kStateBlock = 64;  // states one launch of the general kernel holds (4 per lane, 16 waves)
+
 struct BwdWorkspace {
-    size_t offB, offC, offA, offD, offDb, offStatus, offSeg, total, group_stride;
+    size_t offB, offC, offA, offD, offDb, offSeg, total, group_stride;
     SegPlan seg;
 };
 
 static BwdWorkspace bwd_workspace(const mpa_sscan_shape* s) {
     BwdWorkspace w;
     w.seg = bwd_seg_plan(s);
-    const size_t rows = (size_t)s->batch * w.seg.nseg;
+    // rows of the per-row partials: batch rows, times the segments of a cut sequence or the
+    // state blocks of a wide d_state (the two never combine)
+    const size_t nblk = (size_t)(s->dstate + kStateBlock - 1) / kStateBlock;
+    const size_t rows = (size_t)s->batch * (w.seg.nseg > 1 ? (size_t)w.seg.nseg : nblk);
     const size_t cg = (size_t)(s->dim + kWave - 1) / kWave;
     const size_t bln = (size_t)s->batch * s->seqlen * s->dstate;
-    const size_t ren = rows * s->dim * s->dstate;
+    const size_t ren = (w.seg.nseg > 1 ? rows : (size_t)s->batch) * s->dim * s->dstate;
     const size_t re = rows * s->dim;
     auto up = [](size_t v) { return (v + 63) / 64 * 64; };  // 256-byte granules of floats
     // The partial sums of the channel groups for one (batch, step, state) are written at the same
@@ -506,14 +518,10 @@ static BwdWorkspace bwd_workspace(const mpa_sscan_shape* s) {
     w.offA = w.offC + cg * w.group_stride;
     w.offD = w.offA + up(ren);
     w.offDb = w.offD + up(re);
-    w.offStatus = w.offDb + up(re);
-    w.offSeg = w.offStatus + 64;
+    w.offSeg = w.offDb + up(re);
     w.total = (w.offSeg + up(w.seg.floats)) * sizeof(float);
     return w;
 }
-
-// one word set to zero without a memset node (a caller may be capturing a HIP graph)
-__global__ void clear_status_kernel(int* status) { *status = 0; }
 
 template <typename IO, int NS, int NW, bool HAS_Z>
 static int launch_bwd(const BwdParams& p, hipStream_t stream) {
@@ -582,12 +590,12 @@ extern "C" int mpa_sscan_bwd(const mpa_sscan_shape* s, const void* x, const void
     p.partB = wsf + ws.offB; p.partC = wsf + ws.offC; p.partA = wsf + ws.offA;
     p.part_gs = (int64_t)ws.group_stride;
     p.partD = wsf + ws.offD; p.partDb = wsf + ws.offDb;
-    p.status = reinterpret_cast<int*>(wsf + ws.offStatus);
     p.expire_waits = (s->plan_flags & MPA_PLAN_EXPIRE_WAITS) ? 1 : 0;
     p.reverse = (s->flags & MPA_SSCAN_REVERSE) ? 1 : 0;
     p.nseg = 1;
     p.batch = (int)s->batch; p.L = (int)s->seqlen; p.ED = (int)s->dim; p.N = (int)s->dstate;
     p.nchunks = (p.L + kTile - 1) / kTile;
+    p.Nst = p.N;
     p.softplus = softplus ? 1 : 0;
     p.u_sb = s->u_sb; p.u_sl = s->u_sl; p.u_sd = s->u_sd;
     p.z_sb = s->z_sb; p.z_sl = s->z_sl; p.z_sd = s->z_sd;
@@ -602,9 +610,8 @@ extern "C" int mpa_sscan_bwd(const mpa_sscan_shape* s, const void* x, const void
     const int ns = bwd_states_per_lane(s);
     const int nw = np / ns;
     hipStream_t st = static_cast<hipStream_t>(stream);
-    hipLaunchKernelGGL(clear_status_kernel, dim3(1), dim3(1), 0, st, p.status);
     const bool fast = (!z || p.ypre) && bwd_fast_supported(ns, nw) && !(s->plan_flags & MPA_PLAN_BWD_GENERAL);
-    int rows = p.batch;
+    int rows = p.batch, rows_a = p.batch;
     if (fast) {
         if (ws.seg.nseg > 1) {
             // Sequence cut into segments that run side by side.  The reverse recurrence
@@ -630,14 +637,40 @@ extern "C" int mpa_sscan_bwd(const mpa_sscan_shape* s, const void* x, const void
                                   nullptr, p.batch, ws.seg.nseg, p.ED, p.N, st);
             if (rc != MPA_OK) return rc;
             p.nseg = ws.seg.nseg; p.seg_tiles = ws.seg.seg_tiles; p.ag0 = seg + ws.seg.off_h0;
-            rows = p.batch * p.nseg;
+            rows = rows_a = p.batch * p.nseg;
         }
         rc = launch_bwd_fast(p, ns, nw, s->io_dtype, st);
-    } else if (s->io_dtype == MPA_F32)
-        rc = z ? dispatch_bwd<float, true>(p, ns, nw, st) : dispatch_bwd<float, false>(p, ns, nw, st);
-    else
-        rc = z ? dispatch_bwd<bf16_t, true>(p, ns, nw, st)
-               : dispatch_bwd<bf16_t, false>(p, ns, nw, st);
+    } else {
+        auto general = [&](const BwdParams& q, int qns, int qnw) {
+            if (s->io_dtype == MPA_F32)
+                return z ? dispatch_bwd<float, true>(q, qns, qnw, st) : dispatch_bwd<float, false>(q, qns, qnw, st);
+            return z ? dispatch_bwd<bf16_t, true>(q, qns, qnw, st) : dispatch_bwd<bf16_t, false>(q, qns, qnw, st);
+        };
+        if (p.N <= kStateBlock) {
+            rc = general(p, ns, nw);
+        } else {
+            // d_state above 64: one launch per block of 64 states, in order on the stream.  Each
+            // pass owns its states' dA, dB, dC; dx, ddelta and dz are sums over all states, so
+            // the passes after the first add to what is there; dD comes from the first.
+            const int nblk = (p.N + kStateBlock - 1) / kStateBlock;
+            const size_t es_ = dtype_size(s->io_dtype);
+            for (int sb = 0; sb < nblk && rc == MPA_OK; ++sb) {
+                const int n0 = sb * kStateBlock;
+                BwdParams q = p;
+                q.N = p.N - n0 < kStateBlock ? p.N - n0 : kStateBlock;
+                q.A = A + n0;
+                q.Bm = static_cast<const char*>(B) + n0 * es_;
+                q.C = static_cast<const char*>(C) + n0 * es_;
+                q.h0 = h0 ? h0 + n0 : nullptr;
+                q.ckpt = h_ckpt + (int64_t)n0 * p.ED;
+                q.partA = p.partA + n0; q.partB = p.partB + n0; q.partC = p.partC + n0;
+                q.accumulate = sb > 0 ? 1 : 0;
+                q.row0 = sb * p.batch;
+                rc = general(q, 4, kStateBlock / 4);
+            }
+            rows = p.batch * nblk;
+        }
+    }
     if (rc != MPA_OK) return rc;
 
     const int cg = (p.ED + kWave - 1) / kWave;
@@ -648,7 +681,7 @@ extern "C" int mpa_sscan_bwd(const mpa_sscan_shape* s, const void* x, const void
 #define MPA_FINISH(IO_, V_)                                                                                    \
     hipLaunchKernelGGL((sscan_bwd_finish_kernel<IO_, V_>), fgrid, dim3(256), 0, st, p.partB, p.partC, p.partA, \
                        p.partD, softplus && ddelta_bias ? p.partDb : nullptr, dB, dC, dA, dD, ddelta_bias, cg,  \
-                       p.part_gs, p.batch, rows, p.L, p.ED, p.N, s->dbc_sb, s->dbc_sl, p.status)
+                       p.part_gs, p.batch, rows_a, rows, p.L, p.ED, p.N, s->dbc_sb, s->dbc_sl)
     if (s->io_dtype == MPA_F32) {
         if (vec == 4) MPA_FINISH(float, 4);
         else MPA_FINISH(float, 1);

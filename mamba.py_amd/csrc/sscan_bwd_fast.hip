@@ -190,8 +190,18 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
         const uint32_t offy = ((uint32_t)(4 * qp) * (uint32_t)p.y_sl + (uint32_t)cic * (uint32_t)p.y_sd) * kES;
         const uint32_t offzi = ((uint32_t)(4 * qp) * (uint32_t)p.z_sl + (uint32_t)cic * (uint32_t)p.z_sd) * kES;
         const uint32_t offz = ((uint32_t)(4 * qp) * (uint32_t)p.g_sl + (uint32_t)cic * (uint32_t)p.g_sd) * kES;  // dz
-        const uint32_t sx = (uint32_t)p.u_sl * kES, sd = (uint32_t)p.d_sl * kES, sy = (uint32_t)p.y_sl * kES;
-        const uint32_t sz = (uint32_t)p.z_sl * kES, sg = (uint32_t)p.g_sl * kES;
+        // scalar byte offsets of an item's four walk steps, per tensor, computed once
+        // (readfirstlane: told to the compiler as wave-uniform, so that they stay in scalar
+        // registers; an offset it takes for per-lane costs a loop over its values per access)
+        uint32_t sxj[4], sdj[4], syj[4], szj[4], sgj[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            sxj[j] = __builtin_amdgcn_readfirstlane(jw(j) * (uint32_t)p.u_sl * kES);
+            sdj[j] = __builtin_amdgcn_readfirstlane(jw(j) * (uint32_t)p.d_sl * kES);
+            syj[j] = __builtin_amdgcn_readfirstlane(jw(j) * (uint32_t)p.y_sl * kES);
+            szj[j] = __builtin_amdgcn_readfirstlane(jw(j) * (uint32_t)p.z_sl * kES);
+            sgj[j] = __builtin_amdgcn_readfirstlane(jw(j) * (uint32_t)p.g_sl * kES);
+        }
         // tensor origins of this (batch row, channel group)
         const IO* const xb = static_cast<const IO*>(p.x) + (b * p.u_sb + (int64_t)d0 * p.u_sd);
         const IO* const db = static_cast<const IO*>(p.delta) + (b * p.d_sb + (int64_t)d0 * p.d_sd);
@@ -273,12 +283,12 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
             }
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                raw.x[j] = ld_off(xk, offx, jw(j) * sx, wx);
-                raw.d[j] = ld_off(dk, offd, jw(j) * sd, wd);
-                raw.y[j] = ld_off(yk, offy, jw(j) * sy, wy);
+                raw.x[j] = ld_off(xk, offx, sxj[j], wx);
+                raw.d[j] = ld_off(dk, offd, sdj[j], wd);
+                raw.y[j] = ld_off(yk, offy, syj[j], wy);
                 if constexpr (HAS_Z) {
-                    raw.z[j] = ld_off(zk, offzi, jw(j) * sz, wz);
-                    raw.yp[j] = ld_off(ypk, offy, jw(j) * sy, wy);
+                    raw.z[j] = ld_off(zk, offzi, szj[j], wz);
+                    raw.yp[j] = ld_off(ypk, offy, syj[j], wy);
                 }
             }
 #pragma unroll
@@ -316,11 +326,11 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
                 IO* dzk = dzg + (int64_t)pc * kTile * p.g_sl;
                 if (!ragged) {
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) st_off(dzk, offz, from_float<IO>(dzv[j]), jw(j) * sg);
+                    for (int j = 0; j < 4; ++j) st_off(dzk, offz, from_float<IO>(dzv[j]), sgj[j]);
                 } else {
                     const int t0 = pc * kTile + 4 * qp_now();
                     for (int j = 0; j < 4; ++j)
-                        if (ci_ok && t0 + (int)jw(j) < p.L) st_off(dzk, offz, from_float<IO>(dzv[j]), jw(j) * sg);
+                        if (ci_ok && t0 + (int)jw(j) < p.L) st_off(dzk, offz, from_float<IO>(dzv[j]), sgj[j]);
                 }
             }
             if (ragged) {
@@ -397,8 +407,8 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
             if (group_full && !(ragged_seq && pc == last_chunk) && fw_vec) {
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
-                    st_off(dxk, offg, from_float<IO>(dxv[j]), jw(j) * sg);
-                    st_off(ddk, offg, from_float<IO>(dv[j]), jw(j) * sg);
+                    st_off(dxk, offg, from_float<IO>(dxv[j]), sgj[j]);
+                    st_off(ddk, offg, from_float<IO>(dv[j]), sgj[j]);
                 }
                 if constexpr (kFw == 2)
                     st_off(reinterpret_cast<float2*>(fwk), fw_off, make_float2(fw[0], fw[1]));
@@ -408,8 +418,8 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
                 const int t0 = pc * kTile + 4 * (rev ? NQ - 1 - qo : qo);
                 for (int j = 0; j < 4; ++j)
                     if (co_ok && t0 + (int)jw(j) < p.L) {
-                        st_off(dxk, offg, from_float<IO>(dxv[j]), jw(j) * sg);
-                        st_off(ddk, offg, from_float<IO>(dv[j]), jw(j) * sg);
+                        st_off(dxk, offg, from_float<IO>(dxv[j]), sgj[j]);
+                        st_off(ddk, offg, from_float<IO>(dv[j]), sgj[j]);
                     }
                 for (int i = 0; i < kFw; ++i)
                     if (pc * kTile + (rev ? kTile - 1 - fw_tt : fw_tt) < p.L && fw_n + i < p.N)
@@ -650,15 +660,18 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
         // the start of this interval and publish that in sConsumed; by the end of the sweep
         // that has normally happened, so this wait falls through.  It is bounded (a wave never
         // spins forever); if the bound is ever reached the tiles may be overwritten while they
-        // are still being read, so the launch is marked as failed: the finish kernel then
-        // returns NaN gradients instead of silently wrong ones.
+        // are still being read, so the wave poisons its sums of dA: the call then returns NaN
+        // in dA for these channels instead of silently wrong gradients.
         if (k >= 1) {
             int spins = 0;
             while (consumed < kSvc * k && ++spins < (1 << 20)) {
                 __builtin_amdgcn_s_sleep(1);
                 consumed = __hip_atomic_load(sConsumed, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP);
             }
-            if ((consumed < kSvc * k || p.expire_waits) && lane_now() == 0) *p.status = 1;
+            if (consumed < kSvc * k || p.expire_waits) {
+#pragma unroll
+                for (int i = 0; i < NS; ++i) dAacc[i] = __builtin_nanf("");
+            }
         }
 #pragma unroll
         for (int q = 0; q < NQ; ++q) {

@@ -218,8 +218,17 @@ __global__ void __launch_bounds__((kFwdWaves<NW, MODE>) * kWave) sscan_fwd_kerne
             const uint32_t offx = ((uint32_t)(4 * qp) * (uint32_t)p.u_sl + (uint32_t)cic * (uint32_t)p.u_sd) * kES;
             const uint32_t offd = ((uint32_t)(4 * qp) * (uint32_t)p.d_sl + (uint32_t)cic * (uint32_t)p.d_sd) * kES;
             const uint32_t offz = ((uint32_t)(4 * qp) * (uint32_t)p.z_sl + (uint32_t)cic * (uint32_t)p.z_sd) * kES;
-            const uint32_t sx = (uint32_t)p.u_sl * kES, sd = (uint32_t)p.d_sl * kES, sz = (uint32_t)p.z_sl * kES;
             auto jw = [&](int j) { return (uint32_t)(rev ? 3 - j : j); };
+            // scalar byte offsets of the item's four walk steps, computed once (scalar registers)
+            uint32_t sxj[4], sdj[4], szj[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                // (readfirstlane: told to the compiler as wave-uniform, so that they stay in scalar
+                // registers; an offset it takes for per-lane costs a loop over its values per access)
+                sxj[j] = __builtin_amdgcn_readfirstlane(jw(j) * (uint32_t)p.u_sl * kES);
+                sdj[j] = __builtin_amdgcn_readfirstlane(jw(j) * (uint32_t)p.d_sl * kES);
+                szj[j] = __builtin_amdgcn_readfirstlane(jw(j) * (uint32_t)p.z_sl * kES);
+            }
             // Loads of the ragged chunk run past the sequence end.  That is harmless (the values
             // are masked at staging) as long as the address is inside the tensor: the ragged
             // chunk is read through windows that end with the tensor's last element, whatever
@@ -279,9 +288,9 @@ __global__ void __launch_bounds__((kFwdWaves<NW, MODE>) * kWave) sscan_fwd_kerne
                 }
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
-                    raw.x[j] = ld_off(xk, offx, jw(j) * sx, wx);
-                    raw.d[j] = ld_off(dk, offd, jw(j) * sd, wd);
-                    if (has_z) raw.z[j] = ld_off(zk, offz, jw(j) * sz, wz);
+                    raw.x[j] = ld_off(xk, offx, sxj[j], wx);
+                    raw.d[j] = ld_off(dk, offd, sdj[j], wd);
+                    if (has_z) raw.z[j] = ld_off(zk, offz, szj[j], wz);
                 }
 #pragma unroll
                 for (int r = 0; r < kBcPer; ++r) {
@@ -382,8 +391,10 @@ __global__ void __launch_bounds__((kFwdWaves<NW, MODE>) * kWave) sscan_fwd_kerne
             const bool co_ok = co <= cmax;
             const int q4 = 4 * qo;
             const uint32_t offy = ((uint32_t)(4 * qpo) * (uint32_t)p.y_sl + (uint32_t)min(co, cmax) * (uint32_t)p.y_sd) * kES;
-            const uint32_t sy = (uint32_t)p.y_sl * kES;
             auto jw = [&](int j) { return (uint32_t)(rev ? 3 - j : j); };
+            uint32_t syj[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) syj[j] = __builtin_amdgcn_readfirstlane(jw(j) * (uint32_t)p.y_sl * kES);
             IO* const yg = static_cast<IO*>(p.y) + (b * p.y_sb + (int64_t)d0 * p.y_sd);
             IO* const ypg = static_cast<IO*>(p.ypre) + (b * p.y_sb + (int64_t)d0 * p.y_sd);
             auto reduce_store = [&](int k) {
@@ -402,7 +413,7 @@ __global__ void __launch_bounds__((kFwdWaves<NW, MODE>) * kWave) sscan_fwd_kerne
                     if (p.ypre) {
                         const float pv[4] = {s.x, s.y, s.z, s.w};
                         for (int j = 0; j < 4; ++j)
-                            if (co_ok && t0 + (int)jw(j) < p.L) st_off(ypk, offy, from_float<IO>(pv[j]), jw(j) * sy);
+                            if (co_ok && t0 + (int)jw(j) < p.L) st_off(ypk, offy, from_float<IO>(pv[j]), syj[j]);
                     }
                     const float4 g = *reinterpret_cast<const float4*>(&sG[k & 3][co][q4]);
                     s.x *= g.x; s.y *= g.y; s.z *= g.z; s.w *= g.w;
@@ -410,10 +421,10 @@ __global__ void __launch_bounds__((kFwdWaves<NW, MODE>) * kWave) sscan_fwd_kerne
                 const float sv[4] = {s.x, s.y, s.z, s.w};
                 if (co_ok && whole) {
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) st_off(yk, offy, from_float<IO>(sv[j]), jw(j) * sy);
+                    for (int j = 0; j < 4; ++j) st_off(yk, offy, from_float<IO>(sv[j]), syj[j]);
                 } else if (co_ok) {
                     for (int j = 0; j < 4; ++j)
-                        if (t0 + (int)jw(j) < p.L) st_off(yk, offy, from_float<IO>(sv[j]), jw(j) * sy);
+                        if (t0 + (int)jw(j) < p.L) st_off(yk, offy, from_float<IO>(sv[j]), syj[j]);
                 }
             };
             // the reducers run one tile behind the scan waves

@@ -60,10 +60,11 @@ class LaunchPlan:
 
         MPA_FWD_NS / MPA_BWD_NS       states of d_state per lane (a power of two)
         MPA_FWD_NSEG / MPA_BWD_NSEG   segments a sequence is cut into (1 = never cut)
+        MPA_PSCAN_CHUNKS              pieces the generic scan cuts a sequence into (1 = never cut)
         MPA_BWD_GENERAL=1             general backward kernel even where the fast one applies
     """
     _FIELDS = ("fwd_states_per_lane", "bwd_states_per_lane", "fwd_segments", "bwd_segments",
-               "bwd_general", "expire_waits")
+               "bwd_general", "expire_waits", "pscan_chunks")
 
     def __init__(self):
         env = lambda k: int(os.environ[k]) if os.environ.get(k, "").strip() else None
@@ -71,6 +72,7 @@ class LaunchPlan:
         self.bwd_states_per_lane = env("MPA_BWD_NS")
         self.fwd_segments = env("MPA_FWD_NSEG")
         self.bwd_segments = env("MPA_BWD_NSEG")
+        self.pscan_chunks = env("MPA_PSCAN_CHUNKS")
         self.bwd_general = os.environ.get("MPA_BWD_GENERAL", "") == "1"
         self.expire_waits = False  # test hook (MPA_PLAN_EXPIRE_WAITS)
 
@@ -253,6 +255,7 @@ def _pscan_shape(A, X, H, gA=None, gX=None, reverse=False):
     s.batch, s.seqlen, s.dim, s.dstate = X.shape
     s.io_dtype = _io_dtype(X)
     s.reverse = 1 if reverse else 0
+    s.plan_chunks = plan.pscan_chunks or 0
     for name, t in (("a_st", A), ("x_st", X), ("h_st", H), ("ga_st", gA), ("gx_st", gX)):
         if t is not None:
             getattr(s, name)[:] = list(t.stride())
@@ -277,8 +280,11 @@ class PScan(torch.autograd.Function):
         X = X_in.detach().to(dt)
         H = torch.empty(X.shape, dtype=dt, device=X.device)
         shape = _pscan_shape(A, X, H, reverse=reverse)
+        nbytes = lib.mpa_pscan_workspace_bytes(ctypes.byref(shape))
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=X.device)
         with torch.cuda.device(X.device):
-            rc = lib.mpa_pscan_fwd(ctypes.byref(shape), _ptr(A), _ptr(X), _ptr(H), _stream(X.device))
+            rc = lib.mpa_pscan_fwd(ctypes.byref(shape), _ptr(A), _ptr(X), _ptr(H), _ptr(ws), nbytes,
+                                   _stream(X.device))
         _lib.check(rc, "mpa_pscan_fwd")
         ctx.save_for_backward(A, H)
         ctx.in_dtypes = (A_in.dtype, X_in.dtype)
@@ -293,9 +299,11 @@ class PScan(torch.autograd.Function):
         gA = torch.empty_like(H)
         gX = torch.empty_like(H)
         shape = _pscan_shape(A, G, H, gA, gX, reverse=ctx.reverse)
+        nbytes = lib.mpa_pscan_workspace_bytes(ctypes.byref(shape))
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=H.device)
         with torch.cuda.device(H.device):
             rc = lib.mpa_pscan_bwd(ctypes.byref(shape), _ptr(A), _ptr(H), _ptr(G), _ptr(gA), _ptr(gX),
-                                   _stream(H.device))
+                                   _ptr(ws), nbytes, _stream(H.device))
         _lib.check(rc, "mpa_pscan_bwd")
         return gA.to(ctx.in_dtypes[0]), gX.to(ctx.in_dtypes[1]), None
 

@@ -331,27 +331,12 @@ def softplus_ref(v):
 
 
 # --------------------------------------------------------------------------------------
-# seeded synthetic inputs shared by tests, smoke() and bench.py
+# seeded synthetic inputs: the recipe lives in the neutral module synthetic_inputs.py (the
+# benchmark and smoke() take their inputs from there, not from the checker); re-exported
+# here because every parity test draws its inputs through this module
 # --------------------------------------------------------------------------------------
+import os as _os
+import sys as _sys
 
-def make_inputs(Bs, L, ED, N, seed, dtype=torch.float32, dt_min=1e-3, dt_max=0.1,
-                dt_floor=1e-4):
-    """Seeded inputs with the value distributions of the reference's layer initialisation
-    (mambapy/mamba.py:158-172): A = -(1..N) per channel (S4D-real), delta =
-    softplus(w + inv_softplus(dt)), dt log-uniform in [dt_min, dt_max], w ~ N(0, 0.02),
-    D = 1; x, B, C, dy ~ N(0, 1).  Generated in float32 on the CPU, then rounded to
-    `dtype` (A and D stay float32)."""
-    g = torch.Generator().manual_seed(seed)
-    x = torch.randn(Bs, L, ED, generator=g)
-    Bm = torch.randn(Bs, L, N, generator=g)
-    C = torch.randn(Bs, L, N, generator=g)
-    dt = torch.exp(torch.rand(ED, generator=g) * (math.log(dt_max) - math.log(dt_min))
-                   + math.log(dt_min)).clamp(min=dt_floor)
-    bias = dt + torch.log(-torch.expm1(-dt))
-    w = 0.02 * torch.randn(Bs, L, ED, generator=g)
-    delta = F.softplus(w + bias)
-    A = -torch.arange(1, N + 1, dtype=torch.float32).repeat(ED, 1)
-    D = torch.ones(ED)
-    dy = torch.randn(Bs, L, ED, generator=g)
-    cast = lambda t: t.to(dtype)
-    return dict(x=cast(x), delta=cast(delta), A=A, B=cast(Bm), C=cast(C), D=D, dy=cast(dy))
+_sys.path.insert(0, _os.path.dirname(_os.path.dirname(_os.path.abspath(__file__))))
+from synthetic_inputs import make_inputs  # noqa: E402,F401

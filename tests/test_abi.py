@@ -53,7 +53,11 @@ def test_status_codes_without_launch(pkg):
     s.reserved = 0
     assert lib.mpa_status_string(6) == b"workspace too small"
     p = L.PscanShape()
-    assert lib.mpa_pscan_fwd(ctypes.byref(p), None, None, None, None) == 2
+    assert lib.mpa_pscan_fwd(ctypes.byref(p), None, None, None, None, 0, None) == 2
+    p.batch, p.seqlen, p.dim, p.dstate = 1, 65536, 32, 16
+    cut = lib.mpa_pscan_workspace_bytes(ctypes.byref(p))
+    p.plan_chunks = 1
+    assert 0 < lib.mpa_pscan_workspace_bytes(ctypes.byref(p)) < cut   # a thin, long scan is cut by default
 
 
 def test_missing_library_is_a_loud_import_error(pkg, monkeypatch):

@@ -258,13 +258,113 @@ def test_forward_wide_state(pkg, dev, N, ED, L):
 # failure is loud
 # ---------------------------------------------------------------------------------------------
 
-def test_expired_wait_poisons_the_parameter_gradients(pkg, dev):
+def test_expired_wait_poisons_dA(pkg, dev):
     # The backward kernel waits, with a bound, for a counter in shared memory.  The test hook makes
     # the kernel behave as if the bound had been reached (every wave still runs to its end): the
     # call must not return clean-looking numbers.
     inp = so.make_inputs(2, 100, 64, 16, seed=601)
     with pkg.plan_override(expire_waits=True):
         got = run_gpu_fwd_bwd(pkg, inp, dev)
-    assert torch.isnan(got["dA"]).all() and torch.isnan(got["dD"]).all()
-    clean = run_gpu_fwd_bwd(pkg, inp, dev)           # the flag is cleared by the next call
+    assert torch.isnan(got["dA"]).all()
+    clean = run_gpu_fwd_bwd(pkg, inp, dev)           # nothing sticks to the next call
     assert torch.isfinite(clean["dA"]).all() and torch.isfinite(clean["dD"]).all()
+
+
+# ---------------------------------------------------------------------------------------------
+# generic scan cut into pieces
+# ---------------------------------------------------------------------------------------------
+
+@pytest.mark.parametrize("shape,chunks,reverse", [
+    ((1, 256, 4, 16), 2, False), ((2, 100, 3, 5), 3, False), ((1, 517, 8, 16), 7, False),
+    ((1, 333, 2, 16), 3, True), ((2, 64, 4, 4), 7, True), ((1, 9, 4, 4), 2, False),
+])
+def test_pscan_cut_into_pieces_forward_backward(pkg, dev, shape, chunks, reverse):
+    g = torch.Generator().manual_seed(sum(shape) + chunks)
+    A = torch.rand(*shape, generator=g) * 0.9 + 0.05
+    X = torch.randn(*shape, generator=g)
+    G = torch.randn(*shape, generator=g)
+    Ar, Xr = A.double().requires_grad_(), X.double().requires_grad_()
+    if reverse:
+        Hr = so.linear_recurrence(Ar.flip(1), Xr.flip(1)).flip(1)
+    else:
+        Hr = so.linear_recurrence(Ar, Xr)
+    Hr.backward(G.double())
+    fn = pkg.pscan_rev if reverse else pkg.pscan
+
+    def run():
+        Ag, Xg = A.to(dev).requires_grad_(), X.to(dev).requires_grad_()
+        H = fn(Ag, Xg)
+        H.backward(G.to(dev))
+        return H.detach(), Ag.grad, Xg.grad
+
+    with pkg.plan_override(pscan_chunks=chunks):
+        H, gA, gX = run()
+        H2, gA2, gX2 = run()
+    assert rel_err(H, Hr) <= 1e-5 and rel_err(gX, Xr.grad) <= 1e-5 and rel_err(gA, Ar.grad) <= 1e-5
+    assert torch.equal(H, H2) and torch.equal(gA, gA2) and torch.equal(gX, gX2)   # bitwise reproducible
+    with pkg.plan_override(pscan_chunks=1):
+        H1, gA1, gX1 = run()
+    assert rel_err(H, H1.double()) <= 1e-5 and rel_err(gA, gA1.double()) <= 1e-5 and rel_err(gX, gX1.double()) <= 1e-5
+
+
+def test_pscan_thin_long_sequence_is_cut_by_the_library(pkg, dev):
+    # batch 1, d_model 16 (ED 32), 16 states: 512 recurrences of 20 000 steps, with factors close
+    # to one so that the carried values matter over the whole length
+    shape = (1, 20000, 32, 16)
+    g = torch.Generator().manual_seed(77)
+    A = 1.0 - torch.rand(*shape, generator=g) * 0.02
+    X = torch.randn(*shape, generator=g)
+    G = torch.randn(*shape, generator=g)
+    Ar, Xr = A.double().requires_grad_(), X.double().requires_grad_()
+    # the oracle's restatement of the reference's tree scan (log L vectorised levels: a Python
+    # loop over 20 000 steps with its autograd graph takes minutes on the host)
+    Hr = so.pscan_blelloch(Ar, Xr)
+    Hr.backward(G.double())
+    Ag, Xg = A.to(dev).requires_grad_(), X.to(dev).requires_grad_()
+    H = pkg.pscan(Ag, Xg)
+    H.backward(G.to(dev))
+    assert rel_err(H, Hr) <= 1e-4 and rel_err(Xg.grad, Xr.grad) <= 1e-4 and rel_err(Ag.grad, Ar.grad) <= 1e-4
+
+
+# ---------------------------------------------------------------------------------------------
+# backward at wide d_state (the reference trains at any N; its README measures N = 128 and 256)
+# ---------------------------------------------------------------------------------------------
+
+@pytest.mark.parametrize("N,ED,L,dtype", [
+    (128, 64, 70, torch.float32), (256, 40, 33, torch.float32), (96, 70, 50, torch.float32),
+    (80, 64, 17, torch.float32), (128, 96, 100, torch.bfloat16),
+])
+def test_backward_wide_state(pkg, dev, N, ED, L, dtype):
+    inp = so.make_inputs(2, L, ED, N, seed=700 + N, dtype=dtype)
+    ref = c_oracle.sscan_fwd_bwd(**inp)
+    got = run_gpu_fwd_bwd(pkg, inp, dev)
+    _check(got, ref, TOL[dtype], f"N={N}")
+
+
+def test_backward_wide_state_gated_softplus_reverse(pkg, dev):
+    Bs, L, ED, N = 2, 45, 48, 160
+    inp = so.make_inputs(Bs, L, ED, N, seed=741)
+    g = torch.Generator().manual_seed(742)
+    z = torch.randn(Bs, L, ED, generator=g)
+    raw = torch.randn(Bs, L, ED, generator=g) * 0.5 - 4.0
+    bias = torch.randn(ED, generator=g) * 0.3
+    h0 = torch.randn(Bs, ED, N, generator=g)
+    f64 = lambda t: t.double().requires_grad_()
+    x, r, A, Bm, C, D, zz, bb = map(f64, (inp["x"], raw, inp["A"], inp["B"], inp["C"], inp["D"], z, bias))
+    fl = lambda t: t.flip(1)
+    delta = so.softplus_ref(fl(r) + bb)
+    yr, hl = so.selective_scan_ref(fl(x), delta, A, fl(Bm), fl(C), D, h0=h0.double(), return_last_state=True)
+    yr = fl(yr) * (zz * torch.sigmoid(zz))
+    yr.backward(inp["dy"].double())
+    ref = dict(y=yr, dx=x.grad, ddelta=r.grad, dA=A.grad, dB=Bm.grad, dC=C.grad, dD=D.grad,
+               dz=zz.grad, dbias=bb.grad, hl=hl)
+    t = lambda v: v.to(dev).requires_grad_()
+    gx, gr, gA, gB, gC, gD, gz, gb = map(t, (inp["x"], raw, inp["A"], inp["B"], inp["C"], inp["D"], z, bias))
+    y, h_last = pkg.selective_scan_fn(gx, gr, gA, gB, gC, gD, z=gz, delta_bias=gb, delta_softplus=True,
+                                      h0=h0.to(dev), return_last_state=True, reverse=True)
+    y.backward(inp["dy"].to(dev))
+    got = dict(y=y, dx=gx.grad, ddelta=gr.grad, dA=gA.grad, dB=gB.grad, dC=gC.grad, dD=gD.grad,
+               dz=gz.grad, dbias=gb.grad, hl=h_last)
+    for k in ref:
+        e = rel_err(got[k], ref[k])
+        assert e <= TOL[torch.float32], f"{k}: {e:.3e}"
