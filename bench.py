@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the selective-scan hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c1|c0]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c1|c0|c3|c4|c4-3000|pscan|thin|layer|generate]
 
 One step = one forward + one backward of the fused selective scan over one batch of
 seeded synthetic input that is already resident in HBM.  Prints ONE JSON line.
@@ -9,6 +9,9 @@ seeded synthetic input that is already resident in HBM.  Prints ONE JSON line.
   roofline   the backward entry point (its two kernels), HIP-event time on the launch stream
   cpu_baseline  the CPU restatement of the reference's Blelloch-scan path (oracle "port"),
              timed on this host on a bounded sample of the same workload
+  other      (default workload only) one timed record for each of the other benchmark
+             configurations: c1, c3 (decode step), c4 / c4-3000 (LM forward), the generic pscan
+             and the batch-1 launches
 """
 import argparse
 import json
@@ -29,10 +32,18 @@ WORKLOADS = {
            "configs[2]: mamba-1.4b layer B=4 L=4096 ED=4096 N=16, bf16 I/O, fp32 state"),
 }
 
-# HBM bytes per launch of the backward entry point measured with rocprofv3 --pmc
-# (FETCH_SIZE + WRITE_SIZE, scaled by a copy kernel of known size); filled from the
-# summaries under profiles/.  None = not measured for that workload.
-MEASURED_TRAFFIC_BYTES = {"c2": 1.2196e9}
+def measured_traffic_bytes(workload):
+    """HBM bytes per launch of the backward entry point, measured with rocprofv3 --pmc (FETCH_SIZE
+    + WRITE_SIZE, scaled by a copy kernel of known size).  Read from the summary under profiles/
+    (a line `traffic_bytes_per_launch <workload> mpa_sscan_bwd = <number>`); None when that
+    workload has no summary."""
+    import re
+    path = os.path.join(ROOT, "profiles", f"sscan_fwd_bwd_{workload}_pmc.md")
+    try:
+        m = re.search(rf"traffic_bytes_per_launch\s+{workload}\s+mpa_sscan_bwd\s*=\s*([0-9.eE+-]+)", open(path).read())
+        return float(m.group(1)) if m else None
+    except OSError:
+        return None
 
 
 def algorithmic_bytes(B, L, ED, N, s):
@@ -45,39 +56,45 @@ def algorithmic_bytes(B, L, ED, N, s):
 
 
 def cpu_baseline(workload, torch):
-    """Time the reference's pure-PyTorch path (materialised tensors + Blelloch scan,
-    forward + backward, float32, all host threads) on a slice of the workload's channels:
-    channels are independent, so the slice is the same work per channel."""
-    B, L, ED, N, _, seed, _ = WORKLOADS[workload]
-    ed = min(ED, 512 if workload != "c0" else ED)
-    bs = min(B, 2)
+    """Time the reference's pure-PyTorch path (materialised (B,L,ED,N) tensors + Blelloch scan,
+    forward + backward, float32, all host threads: the oracle's restatement, kind "port") on
+    this host.  configs[0] and [1] run in full; configs[2] runs ONE of its four batch rows at
+    full width (batch rows are independent; ten live 1.07 GB tensors instead of 4.3 GB ones) and
+    the figures are per row: GB/s and tokens/s do not depend on the number of rows.  One warm-up,
+    then the median of three repetitions."""
     # the checker is imported here only: this leg times it, nothing else in the benchmark uses it
     from oracle import scan_oracle as so
     import synthetic_inputs
+    B, L, ED, N, _, seed, _ = WORKLOADS[workload]
+    bs = 1 if workload == "c2" else B
     threads = int(os.environ.get("OMP_NUM_THREADS") or os.cpu_count() or 1)
     torch.set_num_threads(threads)
-    inp = synthetic_inputs.make_inputs(bs, L, ed, N, seed=seed)
+    inp = synthetic_inputs.make_inputs(bs, L, ED, N, seed=seed)
     names = ("x", "delta", "A", "B", "C", "D")
 
-    def once():
+    def once(fn):
         args = [inp[k].clone().requires_grad_() for k in names]
-        y = so.selective_scan_blelloch(*args)
+        t0 = time.perf_counter()
+        y = fn(*args)
         y.backward(inp["dy"])
-        return y
+        return time.perf_counter() - t0
 
-    once()
-    reps, t0 = 0, time.perf_counter()
-    while reps < 3 or (time.perf_counter() - t0 < 12.0 and reps < 60):  # about 12 s of CPU work
-        once()
-        reps += 1
-    dt = (time.perf_counter() - t0) / reps
-    fwd, bwd = algorithmic_bytes(bs, L, ed, N, 4)
-    return {
+    once(so.selective_scan_blelloch)
+    ts = sorted(once(so.selective_scan_blelloch) for _ in range(3))
+    dt = ts[1]
+    fwd, bwd = algorithmic_bytes(bs, L, ED, N, 4)
+    out = {
         "value": (fwd + bwd) / dt / 1e9, "unit": "GB/s", "cores": threads, "kind": "port",
-        "sample": f"B={bs} L={L} ED={ed} of {ED} channels N={N} fp32, fwd+bwd, "
-                  f"{reps} reps, {dt * 1e3:.1f} ms each; GB/s on the same algorithmic-bytes formula",
-        "tokens_per_s_at_full_width": bs * L / dt * ed / ED,
+        "sample": f"B={bs}" + (f" of {B} batch rows" if bs != B else "") +
+                  f" L={L} ED={ED} N={N} fp32, fwd+bwd, 1 warm-up + median of 3, {dt * 1e3:.1f} ms each; "
+                  "GB/s on the same algorithmic-bytes formula",
+        "ms": dt * 1e3, "tokens_per_s": bs * L / dt,
     }
+    if workload == "c0":
+        # the reference's sequential twin (mambapy/mamba.py:297-327), timed at configs[0] only
+        once(so.selective_scan_ref)
+        out["sequential_loop_ms"] = sorted(once(so.selective_scan_ref) for _ in range(3))[1] * 1e3
+    return out
 
 
 def _timed(torch, fn, steps, warmup):
@@ -158,17 +175,17 @@ def bench_decode(args, torch, pkg, dev):
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": bytes_step / t_kgraph / 1e9 / HBM_PEAK_GBS,
                      "traffic": None},
     }
-    print(json.dumps(out))
+    return out
 
 
 def bench_pscan(args, torch, pkg, dev):
     """Generic PScan.apply(A, X) on materialised (B, L, ED, N) operands at the configs[1]
     shape, fp32: forward moves 3 tensors, backward 5."""
     B, L, ED, N = 8, 2048, 1536, 16
-    g = torch.Generator().manual_seed(1005)
-    A = (torch.rand(B, L, ED, N, generator=g) * 0.5 + 0.5).to(dev).requires_grad_()
-    X = torch.randn(B, L, ED, N, generator=g).to(dev).requires_grad_()
-    gH = torch.randn(B, L, ED, N, generator=g).to(dev)
+    g = torch.Generator(device=dev).manual_seed(1005)    # 1.6 GB per tensor: drawn on the GPU
+    A = (torch.rand(B, L, ED, N, generator=g, device=dev) * 0.5 + 0.5).requires_grad_()
+    X = torch.randn(B, L, ED, N, generator=g, device=dev).requires_grad_()
+    gH = torch.randn(B, L, ED, N, generator=g, device=dev)
     steps, warmup = max(3, args.steps // 5), 2
 
     def step(ev=None):
@@ -205,7 +222,7 @@ def bench_pscan(args, torch, pkg, dev):
         "forward": {"kernel": "pscan_fwd_kernel", "achieved": 3 * S / (fwd_ms * 1e-3) / 1e9, "unit": "GB/s",
                     "frac": 3 * S / (fwd_ms * 1e-3) / 1e9 / HBM_PEAK_GBS},
     }
-    print(json.dumps(out))
+    return out
 
 
 def bench_layer_kernels(args, torch, pkg, dev):
@@ -295,7 +312,7 @@ def bench_layer_kernels(args, torch, pkg, dev):
                      "unit": "GB/s", "frac": slow["frac"], "traffic": None},
         "kernels": per,
     }
-    print(json.dumps(out))
+    return out
 
 
 def bench_generate(args, torch, pkg, dev):
@@ -355,7 +372,7 @@ def bench_generate(args, torch, pkg, dev):
         "config": {"workload": "prefill once + one state-update step per token (HIP graph); batch 1 and 64"},
         "batch_1": rows[1], "batch_64": rows[64],
     }
-    print(json.dumps(out))
+    return out
 
 
 def bench_thin(args, torch, pkg, dev):
@@ -416,8 +433,10 @@ def bench_thin(args, torch, pkg, dev):
         "config": {"workload": "batch-1 launches: fused scan B=1 L=4096 ED=2048; generic pscan B=1 L=65536 ED=32"},
         "rows": rows,
     }
-    print(json.dumps(out))
     return out
+
+
+_CACHE = {}
 
 
 def bench_lm_forward(args, torch, pkg, dev, L):
@@ -425,8 +444,10 @@ def bench_lm_forward(args, torch, pkg, dev, L):
     activations, fp32 scan state, B=8, uniform-random token ids."""
     Bsz, vocab = 8, 50280
     cfg = pkg.MambaConfig(d_model=768, n_layers=24, d_state=16)
-    torch.manual_seed(1004)
-    model = pkg.LM(cfg, vocab, pad_vocab_size_multiple=8).to(dev).to(torch.bfloat16)
+    if "lm" not in _CACHE:           # the same random-init model serves L=4096 and L=3000
+        torch.manual_seed(1004)
+        _CACHE["lm"] = pkg.LM(cfg, vocab, pad_vocab_size_multiple=8).to(dev).to(torch.bfloat16)
+    model = _CACHE["lm"]
     ids = torch.randint(0, vocab, (Bsz, L), generator=torch.Generator().manual_seed(1004)).to(dev)
 
     def fwd():
@@ -446,48 +467,13 @@ def bench_lm_forward(args, torch, pkg, dev, L):
         "config": {"workload": f"configs[4]: LM forward 24 layers d_model=768 vocab 50280, B=8 L={L}",
                    "scan_algorithmic_bytes_all_layers": scan_bytes},
     }
-    print(json.dumps(out))
+    return out
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS) + ["c3", "c4", "c4-3000", "pscan", "layer", "generate", "thin"],
-                    help="c2 (default) is the headline workload; c3 = decode step, c4 = LM forward "
-                         "(reported with their own metric, same one-line schema)")
-    ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--copy-probe", action="store_true",
-                    help="also run a plain 256 MiB device copy (reference point that scales the "
-                         "FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
-    args = ap.parse_args()
-    if args.gpus != 1:
-        sys.exit("bench.py: this build runs on ONE GPU (one process, one MI355X); "
-                 "--gpus N with N > 1 is not supported.")
-
-    import torch
-    import __graft_entry__ as entry
+def bench_sscan(args, torch, pkg, dev, workload, steps, warmup, prewarm, cpu=True):
+    """configs[0..2]: forward + backward of the fused scan through the public selective_scan_fn."""
     import synthetic_inputs
-    pkg = entry.load_package()
-    if not torch.cuda.is_available():
-        sys.exit("bench.py: no GPU visible")
-    dev = torch.device("cuda:0")
-
-    if args.workload == "c3":
-        return bench_decode(args, torch, pkg, dev)
-    if args.workload == "pscan":
-        return bench_pscan(args, torch, pkg, dev)
-    if args.workload == "layer":
-        return bench_layer_kernels(args, torch, pkg, dev)
-    if args.workload == "generate":
-        return bench_generate(args, torch, pkg, dev)
-    if args.workload == "thin":
-        return bench_thin(args, torch, pkg, dev)
-    if args.workload.startswith("c4"):
-        return bench_lm_forward(args, torch, pkg, dev, 3000 if args.workload == "c4-3000" else 4096)
-
-    B, L, ED, N, dtname, seed, desc = WORKLOADS[args.workload]
+    B, L, ED, N, dtname, seed, desc = WORKLOADS[workload]
     dtype = getattr(torch, dtname)
     inp = synthetic_inputs.make_inputs(B, L, ED, N, seed=seed, dtype=dtype)
     names = ("x", "delta", "A", "B", "C", "D")
@@ -514,18 +500,22 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
-    for _ in range(args.warmup):
+    # Untimed start-up: the first tens of milliseconds of GPU work after an idle period run at
+    # ramping clocks and through a cold allocator (measured: 1.02 ms per step over the first 20
+    # steps, 0.96 ms from then on); `prewarm` steps bring the device to its steady state before
+    # the W warm-up and K timed steps of the contract.
+    for _ in range(prewarm + warmup):
         step()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for _ in range(args.steps):
+    for _ in range(steps):
         step()
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
-    ms_per_step = wall / args.steps * 1e3
+    ms_per_step = wall / steps * 1e3
 
     # per-entry-point GPU time from HIP events recorded on the launch stream
-    evs = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(args.steps)]
+    evs = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(steps)]
     for e in evs:
         step(e)
     torch.cuda.synchronize()
@@ -538,11 +528,11 @@ def main():
     bwd_gbs = bwd_b / (bwd_ms * 1e-3) / 1e9
     out = {
         "metric": "selective-scan fwd+bwd GB/s (% HBM peak) + tokens/s, "
-                  + ("1.4b layer L=4096" if args.workload == "c2" else desc),
+                  + ("1.4b layer L=4096" if workload == "c2" else desc),
         "value": gbs, "unit": "GB/s",
         "pct_hbm_peak": 100.0 * gbs / HBM_PEAK_GBS,
         "tokens_per_s": B * L / (ms_per_step * 1e-3),
-        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step,
+        "n_gpus": 1, "steps": steps, "warmup": warmup, "prewarm_steps": prewarm, "ms_per_step": ms_per_step,
         "fwd_ms": fwd_ms, "bwd_ms": bwd_ms,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32 state/accumulation, " + ("bf16" if s == 2 else "f32") + " I/O",
@@ -552,13 +542,82 @@ def main():
         "roofline": {"bound": "hbm", "kernel": "mpa_sscan_bwd (sscan_bwd_fast_kernel + sscan_bwd_finish_kernel)",
                      "achieved": bwd_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": bwd_gbs / HBM_PEAK_GBS,
-                     "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload)},
+                     "traffic": measured_traffic_bytes(workload)},
         "forward": {"kernel": "mpa_sscan_fwd (sscan_fwd_kernel)",
                     "achieved": fwd_b / (fwd_ms * 1e-3) / 1e9, "unit": "GB/s",
                     "frac": fwd_b / (fwd_ms * 1e-3) / 1e9 / HBM_PEAK_GBS},
     }
-    if not args.no_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline(args.workload, torch)
+    del gpu, dy, inp
+    torch.cuda.empty_cache()
+    if cpu:
+        out["cpu_baseline"] = cpu_baseline(workload, torch)
+    return out
+
+
+def _brief(rec, extra=()):
+    """The figures of a sub-record that belong into the headline line's `other` object."""
+    keep = ("metric", "value", "unit", "ms_per_step", "steps", "warmup", "dtype", "tokens_per_s", "pct_hbm_peak",
+            "fwd_ms", "bwd_ms", "cpu_baseline", "rows") + tuple(extra)
+    out = {k: rec[k] for k in keep if k in rec}
+    out["workload"] = rec["config"]["workload"]
+    if "roofline" in rec:
+        out["roofline"] = {k: rec["roofline"][k] for k in ("kernel", "achieved", "unit", "frac")}
+    return out
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--prewarm", type=int, default=40,
+                    help="untimed start-up steps before the W warm-up steps (device clocks, allocator)")
+    ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS) + ["c3", "c4", "c4-3000", "pscan", "layer", "generate", "thin"],
+                    help="c2 (default) is the headline workload; c3 = decode step, c4 = LM forward "
+                         "(reported with their own metric, same one-line schema)")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-other", action="store_true",
+                    help="default workload only: leave out the `other` records (c1, c3, c4, pscan, thin)")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="also run a plain 256 MiB device copy (reference point that scales the "
+                         "FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on ONE GPU (one process, one MI355X); "
+                 "--gpus N with N > 1 is not supported.")
+
+    import torch
+    import __graft_entry__ as entry
+    pkg = entry.load_package()
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible")
+    dev = torch.device("cuda:0")
+
+    single = {"c3": bench_decode, "pscan": bench_pscan, "layer": bench_layer_kernels,
+              "generate": bench_generate, "thin": bench_thin}
+    if args.workload in single:
+        out = single[args.workload](args, torch, pkg, dev)
+    elif args.workload.startswith("c4"):
+        out = bench_lm_forward(args, torch, pkg, dev, 3000 if args.workload == "c4-3000" else 4096)
+    else:
+        out = bench_sscan(args, torch, pkg, dev, args.workload, args.steps, args.warmup, args.prewarm,
+                          cpu=not args.no_cpu_baseline)
+        if args.workload == "c2" and not args.no_other:
+            # one timed record per remaining benchmark configuration, inside the same JSON line
+            other = {}
+            cpu = not args.no_cpu_baseline
+            other["c0"] = _brief(bench_sscan(args, torch, pkg, dev, "c0", max(10, args.steps), 3, 0, cpu=cpu))
+            other["c1"] = _brief(bench_sscan(args, torch, pkg, dev, "c1", max(10, args.steps // 2), 3, 10, cpu=cpu))
+            other["c3"] = _brief(bench_decode(args, torch, pkg, dev),
+                                 ("kernel_step_us_called_from_python", "block_step_us", "graphed_layer_step_us"))
+            torch.cuda.empty_cache()
+            other["c4"] = _brief(bench_lm_forward(args, torch, pkg, dev, 4096))
+            other["c4-3000"] = _brief(bench_lm_forward(args, torch, pkg, dev, 3000))
+            torch.cuda.empty_cache()
+            other["pscan"] = _brief(bench_pscan(args, torch, pkg, dev))
+            torch.cuda.empty_cache()
+            other["thin"] = _brief(bench_thin(args, torch, pkg, dev))
+            out["other"] = other
     print(json.dumps(out))
 
 
