@@ -97,9 +97,17 @@ def cpu_baseline(workload, torch):
     return out
 
 
-def _timed(torch, fn, steps, warmup):
-    for _ in range(warmup):
+def _timed(torch, fn, steps, warmup, settle_s=0.05):
+    """Wall time per call of fn over `steps` calls, after `warmup` calls and at least `settle_s`
+    seconds of the same work (device clocks and the allocator settle within tens of milliseconds;
+    a timed window that starts earlier reads 5-20 % slow)."""
+    t_start = time.perf_counter()
+    n = 0
+    while n < warmup or time.perf_counter() - t_start < settle_s:
         fn()
+        n += 1
+        if n >= warmup:
+            torch.cuda.synchronize()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for _ in range(steps):

@@ -153,13 +153,26 @@ __global__ void __launch_bounds__(256) pscan_carry_kernel(const float* __restric
     if (e >= dn) return;
     const int b = blockIdx.y;
     float v = 0.0f;
-    for (int c = 0; c < nchunk; ++c) {
-        const int64_t row = (int64_t)b * nchunk + c;
-        carry[row * dn + e] = v;
-        // (a zero value stays out of the product: it may have overflowed, and 0 * inf is not what
-        // the step-by-step recurrence computes)
-        const float hend = agg[(row * 2 + 1) * dn + e];
-        v = v == 0.0f ? hend : __builtin_fmaf(agg[row * 2 * dn + e], v, hend);
+    // the chain over the pieces is serial, its operands are not: eight pieces' aggregates are
+    // requested before the first of them is used (a launch has few lanes here, so nothing else
+    // would hide the memory latency of every step)
+    for (int c0 = 0; c0 < nchunk; c0 += kUnroll) {
+        float prod[kUnroll], hend[kUnroll];
+#pragma unroll
+        for (int k = 0; k < kUnroll; ++k) {
+            const int64_t row = (int64_t)b * nchunk + min(c0 + k, nchunk - 1);
+            prod[k] = agg[row * 2 * dn + e];
+            hend[k] = agg[(row * 2 + 1) * dn + e];
+        }
+#pragma unroll
+        for (int k = 0; k < kUnroll; ++k) {
+            if (c0 + k < nchunk) {
+                carry[((int64_t)b * nchunk + c0 + k) * dn + e] = v;
+                // (a zero value stays out of the product: it may have overflowed, and 0 * inf is
+                // not what the step-by-step recurrence computes)
+                v = v == 0.0f ? hend[k] : __builtin_fmaf(prod[k], v, hend[k]);
+            }
+        }
     }
 }
 

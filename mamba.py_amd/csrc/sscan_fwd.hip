@@ -331,7 +331,7 @@ __global__ void __launch_bounds__((kFwdWaves<NW, MODE>) * kWave) sscan_fwd_kerne
                         dv[j] = ok ? dv[j] : 0.0f;
                     }
                 }
-                dsum += (dv[0] + dv[1]) + (dv[2] + dv[3]);
+                if constexpr (MODE != kScan) dsum += (dv[0] + dv[1]) + (dv[2] + dv[3]);  // only the carry needs it
                 const int q4 = 4 * qi;
                 *reinterpret_cast<float4*>(&sDl[k & 1][ci][q4]) = make_float4(dv[0], dv[1], dv[2], dv[3]);
                 if (has_z) {
