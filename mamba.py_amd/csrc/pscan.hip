@@ -153,26 +153,36 @@ __global__ void __launch_bounds__(256) pscan_carry_kernel(const float* __restric
     if (e >= dn) return;
     const int b = blockIdx.y;
     float v = 0.0f;
-    // the chain over the pieces is serial, its operands are not: eight pieces' aggregates are
-    // requested before the first of them is used (a launch has few lanes here, so nothing else
-    // would hide the memory latency of every step)
-    for (int c0 = 0; c0 < nchunk; c0 += kUnroll) {
-        float prod[kUnroll], hend[kUnroll];
+    // The chain over the pieces is serial, its operands are not: the aggregates of the next kAhead
+    // pieces are requested while the chain runs over the kAhead before them (a launch has few
+    // lanes here, so nothing else would hide the memory latency of every step).
+    constexpr int kAhead = 16;
+    float prod[2][kAhead], hend[2][kAhead];
+    auto request = [&](int c0, float (&pr)[kAhead], float (&he)[kAhead]) {
 #pragma unroll
-        for (int k = 0; k < kUnroll; ++k) {
+        for (int k = 0; k < kAhead; ++k) {
             const int64_t row = (int64_t)b * nchunk + min(c0 + k, nchunk - 1);
-            prod[k] = agg[row * 2 * dn + e];
-            hend[k] = agg[(row * 2 + 1) * dn + e];
+            pr[k] = agg[row * 2 * dn + e];
+            he[k] = agg[(row * 2 + 1) * dn + e];
         }
+    };
+    auto chain = [&](int c0, const float (&pr)[kAhead], const float (&he)[kAhead]) {
 #pragma unroll
-        for (int k = 0; k < kUnroll; ++k) {
+        for (int k = 0; k < kAhead; ++k) {
             if (c0 + k < nchunk) {
                 carry[((int64_t)b * nchunk + c0 + k) * dn + e] = v;
                 // (a zero value stays out of the product: it may have overflowed, and 0 * inf is
                 // not what the step-by-step recurrence computes)
-                v = v == 0.0f ? hend[k] : __builtin_fmaf(prod[k], v, hend[k]);
+                v = v == 0.0f ? he[k] : __builtin_fmaf(pr[k], v, he[k]);
             }
         }
+    };
+    request(0, prod[0], hend[0]);
+    for (int c0 = 0; c0 < nchunk; c0 += 2 * kAhead) {
+        request(c0 + kAhead, prod[1], hend[1]);
+        chain(c0, prod[0], hend[0]);
+        request(c0 + 2 * kAhead, prod[0], hend[0]);
+        chain(c0 + kAhead, prod[1], hend[1]);
     }
 }
 
