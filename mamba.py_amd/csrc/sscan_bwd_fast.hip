@@ -54,9 +54,10 @@ __device__ __forceinline__ void tile_st(float* tile, int ch, int q, float a, flo
 // matching lane bit, so that at the end lane l holds the complete sum of value number l and
 // each value cost (32+16+8+4+2+1)/64 adds plus the data movement, all on the VALU (no LDS
 // round trip sits in the dependency chain of the reverse sweep).
-//   stage 1: v_permlane32_swap  (lane bit 5)     stage 4: DPP row_half_mirror (lane bit 2)
-//   stage 2: v_permlane16_swap  (lane bit 4)     stage 5: DPP quad_perm 3210  (lane bit 1)
-//   stage 3: DPP row_mirror     (lane bit 3)     stage 6: DPP quad_perm 1032  (lane bit 0)
+//   stage 1: DPP row_mirror      (lane bit 3)     stage 4: DPP quad_perm 1032  (lane bit 0)
+//   stage 2: DPP row_half_mirror (lane bit 2)     stage 5: v_permlane16_swap   (lane bit 4)
+//   stage 3: DPP quad_perm 3210  (lane bit 1)     stage 6: v_permlane32_swap   (lane bit 5)
+// (every stage's partner lane agrees with the lane in the bits of the stages before it)
 // `lo` is the value with index bit 0 (kept by lanes whose bit is clear), `hi` the other one.
 __device__ __forceinline__ float rs_swap32(float lo, float hi) {
     const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(lo), __float_as_uint(hi), false, false);
@@ -74,15 +75,43 @@ __device__ __forceinline__ float rs_dpp(float lo, float hi, bool lane_bit) {
         __builtin_amdgcn_update_dpp(0u, __float_as_uint(send), CTRL, 0xf, 0xf, false));
     return keep + got;
 }
-// stage number (1..6) -> combine
+// Stages 3 and 4 without selects: the lanes whose bit is clear form whole banks (groups of four
+// lanes) of a row, so two additions that each write only their banks do the work: lanes with the
+// bit clear get lo + lo[partner], the others hi + hi[partner].  (The compiler does not see into
+// inline assembly: the two wait states a DPP read needs after a VALU write of the same register
+// are written out.)
+__device__ __forceinline__ float rs_mirror8(float lo, float hi) {
+    float r;
+    asm("s_nop 1\n\t"
+        "v_add_f32_dpp %0, %1, %1 row_mirror row_mask:0xf bank_mask:0x3\n\t"
+        "v_add_f32_dpp %0, %2, %2 row_mirror row_mask:0xf bank_mask:0xc"
+        : "=&v"(r)
+        : "v"(lo), "v"(hi));
+    return r;
+}
+__device__ __forceinline__ float rs_mirror4(float lo, float hi) {
+    float r;
+    asm("s_nop 1\n\t"
+        "v_add_f32_dpp %0, %1, %1 row_half_mirror row_mask:0xf bank_mask:0x5\n\t"
+        "v_add_f32_dpp %0, %2, %2 row_half_mirror row_mask:0xf bank_mask:0xa"
+        : "=&v"(r)
+        : "v"(lo), "v"(hi));
+    return r;
+}
+// stage number (1..6) -> combine.  The stages inside a row of 16 lanes come first: they work on
+// the most values, and a DPP addition costs the SIMD half of what a lane swap across rows costs.
 template <int STAGE>
 __device__ __forceinline__ float rs_stage(float lo, float hi, int lane) {
-    if constexpr (STAGE == 1) return rs_swap32(lo, hi);
-    else if constexpr (STAGE == 2) return rs_swap16(lo, hi);
-    else if constexpr (STAGE == 3) return rs_dpp<0x140>(lo, hi, (lane & 8) != 0);
-    else if constexpr (STAGE == 4) return rs_dpp<0x141>(lo, hi, (lane & 4) != 0);
-    else if constexpr (STAGE == 5) return rs_dpp<0x1B>(lo, hi, (lane & 2) != 0);
-    else return rs_dpp<0xB1>(lo, hi, (lane & 1) != 0);
+    if constexpr (STAGE == 1) return rs_mirror8(lo, hi);
+    else if constexpr (STAGE == 2) return rs_mirror4(lo, hi);
+    else if constexpr (STAGE == 3) return rs_dpp<0x1B>(lo, hi, (lane & 2) != 0);
+    else if constexpr (STAGE == 4) return rs_dpp<0xB1>(lo, hi, (lane & 1) != 0);
+    else if constexpr (STAGE == 5) return rs_swap16(lo, hi);
+    else return rs_swap32(lo, hi);
+}
+// lane bit that decides, in stage 1..6, which of the two values a lane keeps
+__device__ __forceinline__ constexpr int rs_lane_bit(int stage) {
+    return stage == 1 ? 3 : stage == 2 ? 2 : stage == 3 ? 1 : stage == 4 ? 0 : stage == 5 ? 4 : 5;
 }
 
 constexpr int kSvc = 4;  // service waves per workgroup
@@ -168,7 +197,11 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
         const int item = sw * kWave + lane;  // 0 .. 255
         // with softplus or the gate the service waves carry long chains of transcendental
         // functions and would reach the tile barrier last: they then go first when ready
+#ifndef MPA_PRIO_SVC
+#define MPA_PRIO_SVC 1
+#endif
         if (HAS_Z || p.softplus) __builtin_amdgcn_s_setprio(2);
+        else __builtin_amdgcn_s_setprio(MPA_PRIO_SVC);
         constexpr uint32_t kES = sizeof(IO);
         const bool group_full = cmax == kWave - 1;
 
@@ -440,21 +473,33 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
         load_tile(4, rb);
         __syncthreads();  // tiles 0 and 1 are published
         __syncthreads();
-        for (int k = 0; k < ntiles; k += 3) {
+        // The steady-state loop has one exit, at its top: with exits between the intervals the
+        // compiler's wait-count bookkeeping sees an edge from the end of every interval back to
+        // the first one, takes the loads issued last for the ones a tile is staged from, and
+        // makes every interval wait for all loads and stores in flight.
+        int k = 0;
+        for (; k + 3 <= ntiles; k += 3) {
             if (k >= 1) reduce_tile(k - 1);
-            if (k + 2 < ntiles) stage_tile(k + 2, rc);
+            stage_tile(k + 2, rc);
             load_tile(k + 5, rc);
             __syncthreads();  // end of interval k
-            if (k + 1 >= ntiles) break;
             reduce_tile(k);
             if (k + 3 < ntiles) stage_tile(k + 3, ra);
             load_tile(k + 6, ra);
             __syncthreads();  // end of interval k + 1
-            if (k + 2 >= ntiles) break;
             reduce_tile(k + 1);
             if (k + 4 < ntiles) stage_tile(k + 4, rb);
             load_tile(k + 7, rb);
             __syncthreads();  // end of interval k + 2
+        }
+        // the last one or two intervals: every tile is staged already
+        if (k < ntiles) {
+            if (k >= 1) reduce_tile(k - 1);
+            __syncthreads();  // end of interval k
+            if (k + 1 < ntiles) {
+                reduce_tile(k);
+                __syncthreads();  // end of interval k + 1
+            }
         }
         reduce_tile(ntiles - 1);
         sDD[qi * kWave + ci] = dDacc;
@@ -530,11 +575,18 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
     };
 
     float hnext[NS];
+    float poison = 0.0f;
 
     auto tile_pass = [&](int k, const TileIn& in, TileIn& next) {
         float hin[NS];  // state at the tile start
 #pragma unroll
         for (int i = 0; i < NS; ++i) hin[i] = hnext[i];
+        // The two scan waves of a SIMD share its VALU.  The hardware prefers the older wave, which
+        // would then run the tile at the speed of a lone wave and wait at the barrier while the
+        // younger one does most of its work alone (a lone wave issues one instruction per five
+        // clocks, half of what the SIMD takes).  A wave's priority therefore falls as it advances
+        // through the tile: the wave that is behind goes first, both finish together.
+        __builtin_amdgcn_s_setprio(3);
 
         // ---- 1. recompute the tile forward, keeping a[t] and h[t] ----
         float aS[kTile][NS], hS[kTile][NS], dyq[2][4];
@@ -564,6 +616,7 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
         });
 
         // ---- 2. reverse sweep ----
+        __builtin_amdgcn_s_setprio(2);
         float gBv[kTile], ddv[kTile];
         float pend[4];
         int consumed = 0;
@@ -575,6 +628,8 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
                 const float4 v = tile_ld(sDy + (k & 3) * kTileF, lane, qn);
                 dyq[qn & 1][0] = v.x; dyq[qn & 1][1] = v.y; dyq[qn & 1][2] = v.z; dyq[qn & 1][3] = v.w;
             }
+            if (tt == 10) __builtin_amdgcn_s_setprio(1);
+            if (tt == 4) __builtin_amdgcn_s_setprio(0);
             const float dyv = dyq[(tt >> 2) & 1][tt & 3];
             float gB, dd = 0.0f;
             float pB[NS], pC[NS];
@@ -645,10 +700,12 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
                             if (done && sb == 0) {
                                 // lane l holds value number l: decode (step, dB|dC, state)
                                 const int ln = lane_now();
-                                const int which = ln >> 5;
-                                const int st = NS == 2 ? (ln >> 4) & 1 : (((ln >> 4) & 1) << 1) | ((ln >> 3) & 1);
-                                const int stp = NS == 2 ? (ln & 1) << 3 | (ln & 2) << 1 | (ln & 4) >> 1 | (ln & 8) >> 3
-                                                        : (ln & 1) << 2 | (ln & 2) | (ln & 4) >> 2;
+                                // value index bit j (stage j + 1) sits in lane bit rs_lane_bit(j + 1)
+                                auto vbit = [&](int stage) { return (ln >> rs_lane_bit(stage)) & 1; };
+                                const int which = vbit(1);
+                                const int st = NS == 2 ? vbit(2) : (vbit(2) << 1) | vbit(3);
+                                const int stp = NS == 2 ? vbit(3) | vbit(4) << 1 | vbit(5) << 2 | vbit(6) << 3
+                                                        : vbit(4) | vbit(5) << 1 | vbit(6) << 2;
                                 sRed[(k & 1) * kRedF + ((tt + stp) * 2 + which) * NP + w * NS + st] = r;
                             }
                         }
@@ -662,16 +719,22 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
         // spins forever); if the bound is ever reached the tiles may be overwritten while they
         // are still being read, so the wave poisons its sums of dA: the call then returns NaN
         // in dA for these channels instead of silently wrong gradients.
+        // (the sums of the sweep are pinned in front of the wait: left alone, the compiler moves
+        // part of the sweep's arithmetic behind the wait loop and copies the registers it needs)
+#pragma unroll
+        for (int i = 0; i < NS; ++i) asm volatile("" : "+v"(dAacc[i]));
+#pragma unroll
+        for (int tt = 0; tt < kTile; ++tt) asm volatile("" : "+v"(ddv[tt]));
         if (k >= 1) {
             int spins = 0;
             while (consumed < kSvc * k && ++spins < (1 << 20)) {
                 __builtin_amdgcn_s_sleep(1);
                 consumed = __hip_atomic_load(sConsumed, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP);
             }
-            if (consumed < kSvc * k || p.expire_waits) {
-#pragma unroll
-                for (int i = 0; i < NS; ++i) dAacc[i] = __builtin_nanf("");
-            }
+            // (added to the sums at the very end: an assignment here would make every dA
+            // product of the tile dead on this path, and the compiler then moves them behind the
+            // wait together with the registers they need)
+            if (consumed < kSvc * k || p.expire_waits) poison = __builtin_nanf("");
         }
 #pragma unroll
         for (int q = 0; q < NQ; ++q) {
@@ -696,7 +759,7 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
 #pragma unroll
         for (int i = 0; i < NS; ++i) {
             const int n = w * NS + i;
-            if (n < p.N) p.partA[((int64_t)bs * p.ED + d) * p.N + n] = dAacc[i];
+            if (n < p.N) p.partA[((int64_t)bs * p.ED + d) * p.N + n] = dAacc[i] + poison;
         }
     }
     __syncthreads();  // final
