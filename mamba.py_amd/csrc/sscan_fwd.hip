@@ -194,6 +194,7 @@ __global__ void __launch_bounds__((kFwdWaves<NW, MODE>) * kWave) sscan_fwd_kerne
         // transcendental functions and would reach the tile barrier last: they then go first
         // whenever they are ready (measured: -10 % with gate + softplus, +8 % without either)
         if (has_z || p.softplus) __builtin_amdgcn_s_setprio(2);
+        else __builtin_amdgcn_s_setprio(1);
         const int cmax = min(kWave, p.ED - d0) - 1;  // last valid channel of the group
         const int item = (sw & 3) * kWave + lane;    // 0 .. 255
         constexpr uint32_t kES = sizeof(IO);
@@ -369,18 +370,25 @@ __global__ void __launch_bounds__((kFwdWaves<NW, MODE>) * kWave) sscan_fwd_kerne
             load_tile(4, rb);
             __syncthreads();  // tiles 0 and 1 are published
             __syncthreads();  // the scan waves hold tile 0 in registers: its buffer is free
-            for (int k = 0; k < ntiles; k += 3) {
-                if (k + 2 < ntiles) stage_tile(k + 2, rc);
+            // The steady-state loop has one exit, at its top: with exits between the intervals
+            // the compiler's wait-count bookkeeping sees an edge from the end of every interval
+            // back to the first one and makes the wave wait for the loads it has just issued.
+            int k = 0;
+            for (; k + 3 <= ntiles; k += 3) {
+                stage_tile(k + 2, rc);
                 load_tile(k + 5, rc);
                 __syncthreads();
-                if (k + 1 >= ntiles) break;
                 if (k + 3 < ntiles) stage_tile(k + 3, ra);
                 load_tile(k + 6, ra);
                 __syncthreads();
-                if (k + 2 >= ntiles) break;
                 if (k + 4 < ntiles) stage_tile(k + 4, rb);
                 load_tile(k + 7, rb);
                 __syncthreads();
+            }
+            // the last one or two intervals: every tile is staged already
+            if (k < ntiles) {
+                __syncthreads();
+                if (k + 1 < ntiles) __syncthreads();
             }
             if (p.dsum && ci_ok) p.dsum[((int64_t)bs * NQ + qi) * p.ED + d0 + ci] = dsum;
         } else if constexpr (MODE == kScan) {
@@ -498,13 +506,21 @@ __global__ void __launch_bounds__((kFwdWaves<NW, MODE>) * kWave) sscan_fwd_kerne
     if constexpr (kBcast) {
         auto tile_compute = [&](int k, const TileRegs& cur, TileRegs& next) {
             CTile& yt = sY[(k & 1) * NW + w];
+            // The scan waves of a SIMD share its VALU and the hardware prefers the older one, which
+            // would run ahead and then wait at the barrier while the younger one works alone (a
+            // lone wave cannot keep the SIMD busy).  A wave's priority falls as it advances
+            // through the tile, so the wave that is behind goes first.
+            __builtin_amdgcn_s_setprio(3);
             const float4 y0 = scan_group_bcast<0, NS, MODE>(cur.dl, cur.uu, A2, h, cur.vb, cur.vc);
             if constexpr (MODE == kScan) *reinterpret_cast<float4*>(&yt[lane][0]) = y0;
             __builtin_amdgcn_sched_barrier(0);
             read_tile(k + 1, next);
             __builtin_amdgcn_sched_barrier(0);
+            __builtin_amdgcn_s_setprio(2);
             const float4 y1 = scan_group_bcast<1, NS, MODE>(cur.dl, cur.uu, A2, h, cur.vb, cur.vc);
+            __builtin_amdgcn_s_setprio(1);
             const float4 y2 = scan_group_bcast<2, NS, MODE>(cur.dl, cur.uu, A2, h, cur.vb, cur.vc);
+            __builtin_amdgcn_s_setprio(0);
             const float4 y3 = scan_group_bcast<3, NS, MODE>(cur.dl, cur.uu, A2, h, cur.vb, cur.vc);
             if constexpr (MODE == kScan) {
                 *reinterpret_cast<float4*>(&yt[lane][4]) = y1;
