@@ -580,7 +580,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--prewarm", type=int, default=40,
                     help="untimed start-up steps before the W warm-up steps (device clocks, allocator)")
-    ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS) + ["c3", "c4", "c4-3000", "pscan", "layer", "generate", "thin"],
+    ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS) + ["c3", "c4", "c4-3000", "pscan", "layer", "generate", "thin", "issue-probe"],
                     help="c2 (default) is the headline workload; c3 = decode step, c4 = LM forward "
                          "(reported with their own metric, same one-line schema)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -593,6 +593,15 @@ def main():
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU (one process, one MI355X); "
                  "--gpus N with N > 1 is not supported.")
+
+    if args.workload == "issue-probe":
+        # VALU issue-rate table of the SIMDs (mamba.py_amd/csrc/issue_probe.hip, built by build.py):
+        # a child process of its own, started before this process touches the GPU
+        import subprocess
+        exe = os.path.join(ROOT, "mamba.py_amd", "csrc", "issue_probe")
+        if not os.path.exists(exe):
+            sys.exit("bench.py: mamba.py_amd/csrc/issue_probe is not built (python mamba.py_amd/build.py)")
+        sys.exit(subprocess.run([exe]).returncode)
 
     import torch
     import __graft_entry__ as entry

@@ -48,6 +48,13 @@ def build(verbose: bool = False) -> str:
     res = subprocess.run(cmd, capture_output=True, text=True)
     if res.returncode != 0:
         raise RuntimeError(f"link failed:\n{res.stderr}")
+    # the issue-rate probe: a program of its own (a measuring tool, not linked into the library)
+    probe = [_hipcc(), "-O3", f"--offload-arch={ARCH}", "-std=c++17", "-Xclang", "-target-feature", "-Xclang",
+             "-packed-fp32-ops", "-Wno-unused-command-line-argument", os.path.join(CSRC, "issue_probe.hip"),
+             "-o", os.path.join(CSRC, "issue_probe")]
+    res = subprocess.run(probe, capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError(f"hipcc failed on issue_probe.hip:\n{res.stderr}")
     if verbose:
         print(LIB_PATH)
     return LIB_PATH
