@@ -444,6 +444,46 @@ def bench_thin(args, torch, pkg, dev):
     return out
 
 
+def bench_block(args, torch, pkg, dev):
+    """The regime of the reference's own plots (README.md:169-204: one whole MambaBlock, forward +
+    backward, batch 1, fp32, timed on an A100 80GB): d_model 1024 and 2048 at N=16, and d_model 1024
+    at N = 64, 128, 256, all at L=4096.  `published_ms_*` are the reference's figures read off its
+    PNG plots by eye (+-10-15 %, other hardware): context, not a like-for-like baseline."""
+    steps, warmup = max(3, args.steps // 5), 2
+    published = {  # (d_model, N): (mamba.py pscan, official CUDA kernel), milliseconds on A100
+        (1024, 16): (49, 26), (2048, 16): (110, 55), (1024, 64): (140, 28), (1024, 128): (260, 29),
+        (1024, 256): (500, 38)}
+    rows = {}
+    B, L = 1, 4096
+    for (d_model, N), (ref_ms, cuda_ms) in published.items():
+        torch.manual_seed(1020 + N)
+        blk = pkg.MambaBlock(pkg.MambaConfig(d_model=d_model, n_layers=1, d_state=N)).to(dev)
+        x = torch.randn(B, L, d_model, device=dev, requires_grad=True)
+
+        def step():
+            x.grad = None
+            for prm in blk.parameters():
+                prm.grad = None
+            blk(x).sum().backward()
+
+        t = _timed(torch, step, steps, warmup)
+        rows[f"d_model{d_model}_N{N}"] = {"ms": t * 1e3, "tokens_per_s": B * L / t,
+                                          "published_ms_mambapy_pscan_A100": ref_ms,
+                                          "published_ms_official_cuda_A100": cuda_ms}
+        del blk, x
+        torch.cuda.empty_cache()
+    head = rows["d_model1024_N16"]
+    return {
+        "metric": "MambaBlock forward+backward ms, batch 1, fp32, L=4096 (the regime of the reference's README plots)",
+        "value": head["ms"], "unit": "ms", "higher_is_better": False,
+        "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": head["ms"],
+        "scaling": "weak", "vs_baseline": None, "dtype": "f32",
+        "data": "synthetic (random-init weights, N(0,1) input)",
+        "config": {"workload": "one MambaBlock fwd+bwd, B=1 L=4096 fp32: d_model 1024 / 2048 at N=16, d_model 1024 at N=64 / 128 / 256"},
+        "rows": rows,
+    }
+
+
 _CACHE = {}
 
 
@@ -580,7 +620,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--prewarm", type=int, default=40,
                     help="untimed start-up steps before the W warm-up steps (device clocks, allocator)")
-    ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS) + ["c3", "c4", "c4-3000", "pscan", "layer", "generate", "thin", "issue-probe"],
+    ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS) + ["c3", "c4", "c4-3000", "pscan", "layer", "generate", "thin", "block", "issue-probe"],
                     help="c2 (default) is the headline workload; c3 = decode step, c4 = LM forward "
                          "(reported with their own metric, same one-line schema)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -611,7 +651,7 @@ def main():
     dev = torch.device("cuda:0")
 
     single = {"c3": bench_decode, "pscan": bench_pscan, "layer": bench_layer_kernels,
-              "generate": bench_generate, "thin": bench_thin}
+              "generate": bench_generate, "thin": bench_thin, "block": bench_block}
     if args.workload in single:
         out = single[args.workload](args, torch, pkg, dev)
     elif args.workload.startswith("c4"):
@@ -634,6 +674,8 @@ def main():
             other["pscan"] = _brief(bench_pscan(args, torch, pkg, dev))
             torch.cuda.empty_cache()
             other["thin"] = _brief(bench_thin(args, torch, pkg, dev))
+            torch.cuda.empty_cache()
+            other["block"] = _brief(bench_block(args, torch, pkg, dev))
             out["other"] = other
     print(json.dumps(out))
 

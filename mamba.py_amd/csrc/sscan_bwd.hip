@@ -480,13 +480,22 @@ static int bwd_states_per_lane(const mpa_sscan_shape* s) {
     const int ns = pick_states_per_lane(s->batch, s->dim, s->dstate, 4, s->plan_states_per_lane);
     return ns < 0 ? 4 : ns;
 }
-// The cut exists on the fast kernel only, i.e. up to 16 states.
+// The fast kernel holds 16 states.  A wider d_state runs on it as passes over blocks of 16 states
+// (the states are independent given x, delta, B, C; dx, ddelta add up over the passes), each pass cut
+// into segments like a 16-state call.  `blk` = the shape of one such pass.
+constexpr int kFastStates = 16;
+static mpa_sscan_shape fast_block_shape(const mpa_sscan_shape* s) {
+    mpa_sscan_shape blk = *s;
+    if (blk.dstate > kFastStates) blk.dstate = kFastStates;
+    return blk;
+}
+// The cut exists on the fast kernel only.
 static SegPlan bwd_seg_plan(const mpa_sscan_shape* s) {
-    const int ns = bwd_states_per_lane(s);
-    if (s->dstate > 16 || !bwd_fast_supported(ns, padded_states(s->dstate) / ns) ||
-        (s->plan_flags & MPA_PLAN_BWD_GENERAL))
+    const mpa_sscan_shape blk = fast_block_shape(s);
+    const int ns = bwd_states_per_lane(&blk);
+    if (!bwd_fast_supported(ns, padded_states(blk.dstate) / ns) || (s->plan_flags & MPA_PLAN_BWD_GENERAL))
         return SegPlan{1, 0, 0, 0, 0, 0};
-    return seg_plan(s, ns, kBwdThin);
+    return seg_plan(&blk, ns, kBwdThin);
 }
 
 constexpr int kStateBlock = 64;  // states one launch of the general kernel holds (4 per lane, 16 waves)
@@ -499,13 +508,16 @@ struct BwdWorkspace {
 static BwdWorkspace bwd_workspace(const mpa_sscan_shape* s) {
     BwdWorkspace w;
     w.seg = bwd_seg_plan(s);
-    // rows of the per-row partials: batch rows, times the segments of a cut sequence or the
-    // state blocks of a wide d_state (the two never combine)
-    const size_t nblk = (size_t)(s->dstate + kStateBlock - 1) / kStateBlock;
-    const size_t rows = (size_t)s->batch * (w.seg.nseg > 1 ? (size_t)w.seg.nseg : nblk);
+    // rows of the per-row partials of dD / ddelta_bias: batch rows, times the segments of a cut
+    // sequence, times the passes over state blocks of a wide d_state (16 states on the fast kernel,
+    // 64 on the general one, which is never cut: the larger count covers both); dA has one row per
+    // batch row and segment, every pass writes its own states of it
+    const size_t nseg = w.seg.nseg > 1 ? (size_t)w.seg.nseg : 1;
+    const size_t nblk = (size_t)(s->dstate + kFastStates - 1) / kFastStates;
+    const size_t rows = (size_t)s->batch * nseg * nblk;
     const size_t cg = (size_t)(s->dim + kWave - 1) / kWave;
     const size_t bln = (size_t)s->batch * s->seqlen * s->dstate;
-    const size_t ren = (w.seg.nseg > 1 ? rows : (size_t)s->batch) * s->dim * s->dstate;
+    const size_t ren = (size_t)s->batch * nseg * s->dim * s->dstate;
     const size_t re = rows * s->dim;
     auto up = [](size_t v) { return (v + 63) / 64 * 64; };  // 256-byte granules of floats
     // The partial sums of the channel groups for one (batch, step, state) are written at the same
@@ -606,40 +618,63 @@ extern "C" int mpa_sscan_bwd(const mpa_sscan_shape* s, const void* x, const void
     p.in_tmajor = (s->u_sd != 1 && s->u_sl == 1) ? 1 : 0;
     p.out_tmajor = (s->g_sd != 1 && s->g_sl == 1) ? 1 : 0;
 
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    // the fast kernel (16 states per launch, in passes over blocks of 16 for a wider d_state) unless
+    // the gate comes without the saved pre-gate output or the caller asks for the general kernel
+    const mpa_sscan_shape blk_shape = fast_block_shape(s);
+    const int fns = bwd_states_per_lane(&blk_shape);
+    const int fnw = padded_states(blk_shape.dstate) / fns;
+    const bool fast = (!z || p.ypre) && bwd_fast_supported(fns, fnw) && !(s->plan_flags & MPA_PLAN_BWD_GENERAL);
     const int np = padded_states(s->dstate);
     const int ns = bwd_states_per_lane(s);
     const int nw = np / ns;
-    hipStream_t st = static_cast<hipStream_t>(stream);
-    const bool fast = (!z || p.ypre) && bwd_fast_supported(ns, nw) && !(s->plan_flags & MPA_PLAN_BWD_GENERAL);
     int rows = p.batch, rows_a = p.batch;
     if (fast) {
-        if (ws.seg.nseg > 1) {
-            // Sequence cut into segments that run side by side.  The reverse recurrence
-            // ag[t] = a[t] * (ag[t+1] + C[t]*dy[t]) is linear in its state like the forward one,
-            // so the forward kernel in its carry mode, walking against the forward direction,
-            // finds every segment's end value from zero and its sum of delta; seg_carry_kernel
-            // chains them into the value that flows into each segment.
-            float* seg = wsf + ws.offSeg;
-            FwdParams g{};
-            g.x = dy; g.delta = delta; g.z = z; g.A = A; g.D = D; g.dbias = delta_bias;
-            g.Bm = C; g.C = C; g.bc_sb = s->bc_sb; g.bc_sl = s->bc_sl;
-            g.hlast = seg + ws.seg.off_hend; g.dsum = seg + ws.seg.off_dsum;
-            g.nseg = ws.seg.nseg; g.seg_tiles = ws.seg.seg_tiles;
-            g.batch = p.batch; g.L = p.L; g.ED = p.ED; g.N = p.N; g.nchunks = p.nchunks;
-            g.softplus = p.softplus; g.reverse = p.reverse ? 0 : 1;
-            g.u_sb = s->y_sb; g.u_sl = s->y_sl; g.u_sd = s->y_sd;
-            g.z_sb = s->z_sb; g.z_sl = s->z_sl; g.z_sd = s->z_sd;
-            g.d_sb = s->d_sb; g.d_sl = s->d_sl; g.d_sd = s->d_sd;
-            g.in_tmajor = (s->d_sd != 1 && s->d_sl == 1) ? 1 : 0;
-            rc = launch_fwd_any(g, s->io_dtype, ns, nw, kGCarry, st);
-            if (rc != MPA_OK) return rc;
-            rc = launch_seg_carry(A, nullptr, seg + ws.seg.off_hend, seg + ws.seg.off_dsum, seg + ws.seg.off_h0,
-                                  nullptr, p.batch, ws.seg.nseg, p.ED, p.N, st);
-            if (rc != MPA_OK) return rc;
-            p.nseg = ws.seg.nseg; p.seg_tiles = ws.seg.seg_tiles; p.ag0 = seg + ws.seg.off_h0;
-            rows = rows_a = p.batch * p.nseg;
+        const int nseg = ws.seg.nseg > 1 ? ws.seg.nseg : 1;
+        const int nblk = (p.N + kFastStates - 1) / kFastStates;
+        const size_t es_ = dtype_size(s->io_dtype);
+        for (int sb = 0; sb < nblk && rc == MPA_OK; ++sb) {
+            const int n0 = sb * kFastStates;
+            BwdParams q = p;
+            q.N = p.N - n0 < kFastStates ? p.N - n0 : kFastStates;
+            q.A = A + n0;
+            q.Bm = static_cast<const char*>(B) + n0 * es_;
+            q.C = static_cast<const char*>(C) + n0 * es_;
+            q.h0 = h0 ? h0 + n0 : nullptr;
+            q.ckpt = h_ckpt + (int64_t)n0 * p.ED;
+            q.partA = p.partA + n0; q.partB = p.partB + n0; q.partC = p.partC + n0;
+            q.accumulate = sb > 0 ? 1 : 0;
+            q.row0 = sb * p.batch * nseg;
+            if (nseg > 1) {
+                // Sequence cut into segments that run side by side.  The reverse recurrence
+                // ag[t] = a[t] * (ag[t+1] + C[t]*dy[t]) is linear in its state like the forward one,
+                // so the forward kernel in its carry mode, walking against the forward direction,
+                // finds every segment's end value from zero and its sum of delta; seg_carry_kernel
+                // chains them into the value that flows into each segment.
+                float* seg = wsf + ws.offSeg;
+                FwdParams g{};
+                g.x = dy; g.delta = delta; g.z = z; g.A = q.A; g.D = D; g.dbias = delta_bias;
+                g.Bm = q.C; g.C = q.C; g.bc_sb = s->bc_sb; g.bc_sl = s->bc_sl;
+                g.hlast = seg + ws.seg.off_hend; g.dsum = seg + ws.seg.off_dsum;
+                g.nseg = nseg; g.seg_tiles = ws.seg.seg_tiles;
+                g.batch = p.batch; g.L = p.L; g.ED = p.ED; g.N = q.N; g.nchunks = p.nchunks;
+                g.a_st = p.N; g.h_st = q.N; g.ck_st = q.N;
+                g.softplus = p.softplus; g.reverse = p.reverse ? 0 : 1;
+                g.u_sb = s->y_sb; g.u_sl = s->y_sl; g.u_sd = s->y_sd;
+                g.z_sb = s->z_sb; g.z_sl = s->z_sl; g.z_sd = s->z_sd;
+                g.d_sb = s->d_sb; g.d_sl = s->d_sl; g.d_sd = s->d_sd;
+                g.in_tmajor = (s->d_sd != 1 && s->d_sl == 1) ? 1 : 0;
+                rc = launch_fwd_any(g, s->io_dtype, fns, fnw, kGCarry, st);
+                if (rc != MPA_OK) return rc;
+                rc = launch_seg_carry(q.A, nullptr, seg + ws.seg.off_hend, seg + ws.seg.off_dsum, seg + ws.seg.off_h0,
+                                      nullptr, p.batch, nseg, p.ED, q.N, p.N, q.N, st);
+                if (rc != MPA_OK) return rc;
+                q.nseg = nseg; q.seg_tiles = ws.seg.seg_tiles; q.ag0 = seg + ws.seg.off_h0;
+            }
+            rc = launch_bwd_fast(q, fns, fnw, s->io_dtype, st);
         }
-        rc = launch_bwd_fast(p, ns, nw, s->io_dtype, st);
+        rows_a = p.batch * nseg;
+        rows = rows_a * nblk;
     } else {
         auto general = [&](const BwdParams& q, int qns, int qnw) {
             if (s->io_dtype == MPA_F32)

@@ -138,7 +138,9 @@ struct BwdFastLds {
 // HAS_Z: the forward multiplied its output by silu(z).  The service waves then read z and the
 // saved pre-gate output next to dy, publish dy*silu(z) as the dy tile (everything downstream is
 // unchanged) and store dz = dy * y_pre * d silu(z)/dz.
-template <typename IO, int NS, int NW, bool HAS_Z>
+// ACC: a pass after the first over the states of a wide d_state: it adds to the dx and ddelta
+// that are there and leaves D*dy, dD and dz to the first pass.
+template <typename IO, int NS, int NW, bool HAS_Z, bool ACC>
 __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(const BwdParams p) {
     constexpr int NP = NS * NW;
     constexpr int NQ = kTile / 4;
@@ -266,7 +268,9 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
         const int qo = p.out_tmajor ? item % NQ : item / kWave;
         const int qpo = rev ? NQ - 1 - qo : qo;
         const bool co_ok = co <= cmax;
-        const float Dr = p.D[d0 + min(co, cmax)];
+        // (a pass after the first over the states of a wide d_state adds to dx, ddelta; D*dy, dD and dz
+        // belong to the first one)
+        const float Dr = ACC ? 0.0f : p.D[d0 + min(co, cmax)];
         const uint32_t offg = ((uint32_t)(4 * qpo) * (uint32_t)p.g_sl + (uint32_t)min(co, cmax) * (uint32_t)p.g_sd) * kES;
         IO* const dxg = static_cast<IO*>(p.dx) + (b * p.g_sb + (int64_t)d0 * p.g_sd);
         IO* const ddg = static_cast<IO*>(p.ddelta) + (b * p.g_sb + (int64_t)d0 * p.g_sd);
@@ -279,9 +283,9 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
         const int fw_tt = fw_i / NP, fw_n = fw_i % NP;        // walk step, state
         const int fw_tp = rev ? kTile - 1 - fw_tt : fw_tt;    // physical step inside the chunk
         const int fw_e = (fw_tt * 2 + fw_which) * NP + fw_n;  // index inside the dB|dC tile in LDS
-        float* const fw_base = (fw_which ? p.partC : p.partB) + cg * p.part_gs + (int64_t)b * p.L * p.N;
-        const uint32_t fw_off = ((uint32_t)fw_tp * (uint32_t)p.N + (uint32_t)fw_n) * 4u;
-        const bool fw_vec = p.N == NP;  // rows of the partial buffers are then aligned for vector stores
+        float* const fw_base = (fw_which ? p.partC : p.partB) + cg * p.part_gs + (int64_t)b * p.L * p.Nst;
+        const uint32_t fw_off = ((uint32_t)fw_tp * (uint32_t)p.Nst + (uint32_t)fw_n) * 4u;
+        const bool fw_vec = p.N == NP && p.Nst % 4 == 0;  // rows of the partial buffers are then aligned for vector stores
 
         float dDacc = 0.0f, dDb = 0.0f;
 
@@ -355,7 +359,7 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
                 }
             }
             const bool ragged = !group_full || (ragged_seq && pc == last_chunk);
-            if constexpr (HAS_Z) {
+            if constexpr (HAS_Z && !ACC) {
                 IO* dzk = dzg + (int64_t)pc * kTile * p.g_sl;
                 if (!ragged) {
 #pragma unroll
@@ -379,7 +383,7 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
                 }
             }
 #pragma unroll
-            for (int j = 0; j < 4; ++j) dDacc = __builtin_fmaf(yv[j], xv[j], dDacc);
+            for (int j = 0; j < 4; ++j) dDacc = __builtin_fmaf(yv[j], xv[j], dDacc);  // (dropped at the end by a later pass)
             const int s4 = (k & 3) * kTileF;
             tile_st(sDl + s4, ci, qi, dv[0], dv[1], dv[2], dv[3]);
             tile_st(sU + (k & 1) * kTileF, ci, qi, dv[0] * xv[0], dv[1] * xv[1], dv[2] * xv[2], dv[3] * xv[3]);
@@ -392,6 +396,28 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
                 float* dst = sBC + (k & 1) * kBcF + bcn[r] * kTile + bct[r];
                 dst[0] = ok ? to_float(raw.b[r]) : 0.0f;
                 dst[NP * kTile] = ok ? to_float(raw.c[r]) : 0.0f;
+            }
+        };
+        // A pass after the first over the states of a wide d_state adds its share to the dx and
+        // ddelta that are there.  They are requested one interval before the tile is reduced, ahead
+        // of that interval's input loads: a wave's loads return in order, so a load that is
+        // waited for right after its issue would make the wave wait for every tile in flight.
+        struct Acc { IO dx[4], dd[4]; };
+        Acc acc;
+        auto load_acc = [&](int kk) {
+            if constexpr (!ACC) return;
+            const int pc = phys_of(chunk_of(min(kk, ntiles - 1)));
+            const IO* dxk = dxg + (int64_t)pc * kTile * p.g_sl;
+            const IO* ddk = ddg + (int64_t)pc * kTile * p.g_sl;
+            uint32_t wg = 0xffffffffu;
+            if (ragged_seq && pc == last_chunk) {
+                const int64_t end = (p.batch - 1) * p.g_sb + (p.L - 1) * p.g_sl + (p.ED - 1) * p.g_sd + 1;
+                wg = window_bytes(end, b * p.g_sb + (int64_t)pc * kTile * p.g_sl + (int64_t)d0 * p.g_sd, kES);
+            }
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                acc.dx[j] = ld_off(dxk, offg, sgj[j], wg);
+                acc.dd[j] = ld_off(ddk, offg, sgj[j], wg);
             }
         };
         auto reduce_tile = [&](int k) {
@@ -434,9 +460,16 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
                     dDb += dv[j];
                 }
             }
+            if constexpr (ACC) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    dxv[j] += to_float(acc.dx[j]);
+                    dv[j] += to_float(acc.dd[j]);
+                }
+            }
             IO* dxk = dxg + (int64_t)pc * kTile * p.g_sl;
             IO* ddk = ddg + (int64_t)pc * kTile * p.g_sl;
-            float* fwk = fw_base + (int64_t)pc * kTile * p.N;
+            float* fwk = fw_base + (int64_t)pc * kTile * p.Nst;
             if (group_full && !(ragged_seq && pc == last_chunk) && fw_vec) {
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
@@ -480,14 +513,17 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
         int k = 0;
         for (; k + 3 <= ntiles; k += 3) {
             if (k >= 1) reduce_tile(k - 1);
+            load_acc(k);
             stage_tile(k + 2, rc);
             load_tile(k + 5, rc);
             __syncthreads();  // end of interval k
             reduce_tile(k);
+            load_acc(k + 1);
             if (k + 3 < ntiles) stage_tile(k + 3, ra);
             load_tile(k + 6, ra);
             __syncthreads();  // end of interval k + 1
             reduce_tile(k + 1);
+            load_acc(k + 2);
             if (k + 4 < ntiles) stage_tile(k + 4, rb);
             load_tile(k + 7, rb);
             __syncthreads();  // end of interval k + 2
@@ -495,14 +531,16 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
         // the last one or two intervals: every tile is staged already
         if (k < ntiles) {
             if (k >= 1) reduce_tile(k - 1);
+            load_acc(k);
             __syncthreads();  // end of interval k
             if (k + 1 < ntiles) {
                 reduce_tile(k);
+                load_acc(k + 1);
                 __syncthreads();  // end of interval k + 1
             }
         }
         reduce_tile(ntiles - 1);
-        sDD[qi * kWave + ci] = dDacc;
+        sDD[qi * kWave + ci] = ACC ? 0.0f : dDacc;
         sDD[(4 + qo) * kWave + co] = dDb;
         __syncthreads();  // final
         // dD (and ddelta_bias): sum the four step groups of every channel
@@ -513,8 +551,8 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
                 s += sDD[q * kWave + lane];
                 sb += sDD[(4 + q) * kWave + lane];
             }
-            p.partD[(int64_t)bs * p.ED + d0 + lane] = s;
-            if (p.softplus) p.partDb[(int64_t)bs * p.ED + d0 + lane] = sb;
+            p.partD[(int64_t)(p.row0 + bs) * p.ED + d0 + lane] = s;
+            if (p.softplus) p.partDb[(int64_t)(p.row0 + bs) * p.ED + d0 + lane] = sb;
         }
         return;
     }
@@ -526,8 +564,10 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
 #pragma unroll
     for (int i = 0; i < NS; ++i) {
         const int n = w * NS + i;
+        // (A, h0, the checkpoints and the dA partials are rows of Nst states, the states of the whole
+        // call; this launch works on N of them, starting where the host put the pointers)
         const int64_t dn = (int64_t)min(d, p.ED - 1) * p.N + min(n, p.N - 1);
-        const float av = p.A[dn];
+        const float av = p.A[(int64_t)min(d, p.ED - 1) * p.Nst + min(n, p.N - 1)];
         const bool ok = dvalid && n < p.N;
         A2[i] = ok ? av * kLog2e : 0.0f;
         // a*g flowing in from the steps after this row's last one (zero at the sequence end)
@@ -540,14 +580,14 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
     auto load_state = [&](int k, float (&hs)[NS]) {
         const int c = chunk_of(min(k, ntiles - 1));
         const uint32_t ck_lane = (uint32_t)min(d0 + lane_now(), p.ED - 1);
-        const float* ck_base = p.ckpt + ((int64_t)b * p.nchunks + max(c - 1, 0)) * p.N * p.ED;
-        const float* h0_base = p.h0 ? p.h0 + (int64_t)b * p.ED * p.N : ck_base;
+        const float* ck_base = p.ckpt + ((int64_t)b * p.nchunks + max(c - 1, 0)) * p.Nst * p.ED;
+        const float* h0_base = p.h0 ? p.h0 + (int64_t)b * p.ED * p.Nst : ck_base;
         const bool first = c == 0;
 #pragma unroll
         for (int i = 0; i < NS; ++i) {
             const uint32_t n = (uint32_t)min(w * NS + i, p.N - 1);
             // branch-free: chunk 0 reads slot 0 (or h0) and the value is masked below
-            const uint32_t off = first && p.h0 ? ck_lane * (uint32_t)p.N + n : n * (uint32_t)p.ED + ck_lane;
+            const uint32_t off = first && p.h0 ? ck_lane * (uint32_t)p.Nst + n : n * (uint32_t)p.ED + ck_lane;
             const float v = (first ? h0_base : ck_base)[off];
             hs[i] = (!first || p.h0) ? v : 0.0f;
         }
@@ -759,38 +799,41 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
 #pragma unroll
         for (int i = 0; i < NS; ++i) {
             const int n = w * NS + i;
-            if (n < p.N) p.partA[((int64_t)bs * p.ED + d) * p.N + n] = dAacc[i] + poison;
+            if (n < p.N) p.partA[((int64_t)bs * p.ED + d) * p.Nst + n] = dAacc[i] + poison;
         }
     }
     __syncthreads();  // final
 }
 
-template <typename IO, int NS, int NW, bool HAS_Z>
+template <typename IO, int NS, int NW, bool HAS_Z, bool ACC>
 static int launch_fast(const BwdParams& p, hipStream_t stream) {
     dim3 grid((p.ED + kWave - 1) / kWave, p.batch * (p.nseg > 1 ? p.nseg : 1));
     dim3 block((NW + kSvc) * kWave);
     constexpr size_t lds = sizeof(float) * BwdFastLds<NS, NW>::floats;
     static_assert(lds <= 160 * 1024, "LDS budget");
     static LdsLimitOnce lds_limit;
-    const int attr_rc = lds_limit.ensure(sscan_bwd_fast_kernel<IO, NS, NW, HAS_Z>, lds);
+    const int attr_rc = lds_limit.ensure(sscan_bwd_fast_kernel<IO, NS, NW, HAS_Z, ACC>, lds);
     if (attr_rc != MPA_OK) return attr_rc;
-    hipLaunchKernelGGL((sscan_bwd_fast_kernel<IO, NS, NW, HAS_Z>), grid, block, lds, stream, p);
+    hipLaunchKernelGGL((sscan_bwd_fast_kernel<IO, NS, NW, HAS_Z, ACC>), grid, block, lds, stream, p);
     return check_launch();
 }
 
 bool bwd_fast_supported(int ns, int nw) { return (ns == 2 && nw == 8) || (ns == 4 && nw == 4); }
 
 int launch_bwd_fast(const BwdParams& p, int ns, int nw, int io_dtype, hipStream_t stream) {
-#define MPA_CASE(NS_, NW_)                                                                \
-    if (ns == NS_ && nw == NW_) {                                                         \
-        if (p.z)                                                                          \
-            return io_dtype == MPA_F32 ? launch_fast<float, NS_, NW_, true>(p, stream)    \
-                                       : launch_fast<bf16_t, NS_, NW_, true>(p, stream);  \
-        return io_dtype == MPA_F32 ? launch_fast<float, NS_, NW_, false>(p, stream)       \
-                                   : launch_fast<bf16_t, NS_, NW_, false>(p, stream);     \
+#define MPA_CASE2(NS_, NW_, Z_, ACC_)                                                    \
+    return io_dtype == MPA_F32 ? launch_fast<float, NS_, NW_, Z_, ACC_>(p, stream)        \
+                               : launch_fast<bf16_t, NS_, NW_, Z_, ACC_>(p, stream)
+#define MPA_CASE(NS_, NW_)                                          \
+    if (ns == NS_ && nw == NW_) {                                   \
+        if (p.z && p.accumulate) MPA_CASE2(NS_, NW_, true, true);   \
+        if (p.z) MPA_CASE2(NS_, NW_, true, false);                  \
+        if (p.accumulate) MPA_CASE2(NS_, NW_, false, true);         \
+        MPA_CASE2(NS_, NW_, false, false);                          \
     }
     MPA_CASE(2, 8) MPA_CASE(4, 4)
 #undef MPA_CASE
+#undef MPA_CASE2
     return MPA_ERR_BAD_SHAPE;
 }
 

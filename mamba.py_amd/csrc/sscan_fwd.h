@@ -26,6 +26,13 @@ struct FwdParams {
     int nseg;        // > 1: every batch row is cut into nseg segments of seg_tiles tiles, one
     int seg_tiles;   // workgroup row (blockIdx.y) per (batch row, segment)
     int batch, L, ED, N, nchunks;
+    // A wide d_state runs as passes over blocks of states: N = states of this launch, and the
+    // arrays indexed by state keep the row stride of the whole call, with their pointers advanced
+    // to the block's first state by the host: a_st = states per row of A, h_st = of h0 / hlast,
+    // ck_st = states per checkpoint.  A pass after the first gets D = NULL (no D*x term) and adds
+    // what `yacc` holds (strides of y) to its output before the gate.
+    int a_st, h_st, ck_st;
+    const void* yacc;
     int softplus;
     int reverse;     // the walk runs from the last physical step to the first
     int in_tmajor;   // x / delta have unit stride along time
@@ -61,7 +68,8 @@ SegPlan seg_plan(const mpa_sscan_shape* s, int ns, int thin);
 int launch_fwd_any(const FwdParams& p, int io_dtype, int ns, int nw, int mode, hipStream_t stream);
 // segh0[row] = state at the start of every segment, from the end states and delta sums of the
 // first pass; hlast (optional) = state after the last segment.
+// (A has rows of a_st states, the caller's h0 / hlast rows of h_st states; the segment buffers are dense)
 int launch_seg_carry(const float* A, const float* h0, const float* hend, const float* dsum, float* segh0,
-                     float* hlast, int batch, int nseg, int ED, int N, hipStream_t st);
+                     float* hlast, int batch, int nseg, int ED, int N, int a_st, int h_st, hipStream_t st);
 
 }  // namespace mpa

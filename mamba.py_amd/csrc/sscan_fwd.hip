@@ -205,7 +205,7 @@ __global__ void __launch_bounds__((kFwdWaves<NW, MODE>) * kWave) sscan_fwd_kerne
             const int qp = rev ? NQ - 1 - qi : qi;                  // its physical step group
             const bool ci_ok = ci <= cmax;
             const int cic = min(ci, cmax);
-            const float Dv = p.D[d0 + cic];
+            const float Dv = p.D ? p.D[d0 + cic] : 0.0f;  // (NULL: a pass after the first over a wide d_state)
             const float bias = p.dbias ? p.dbias[d0 + cic] : 0.0f;
             // wave-uniform chunk origins (scalar registers) + per-thread 32-bit element
             // offsets that do not change from tile to tile: one load per element and no
@@ -405,6 +405,23 @@ __global__ void __launch_bounds__((kFwdWaves<NW, MODE>) * kWave) sscan_fwd_kerne
             for (int j = 0; j < 4; ++j) syj[j] = __builtin_amdgcn_readfirstlane(jw(j) * (uint32_t)p.y_sl * kES);
             IO* const yg = static_cast<IO*>(p.y) + (b * p.y_sb + (int64_t)d0 * p.y_sd);
             IO* const ypg = static_cast<IO*>(p.ypre) + (b * p.y_sb + (int64_t)d0 * p.y_sd);
+            // What is already in the output (a pass after the first over a wide d_state adds to
+            // it): requested one interval before the tile is reduced, so that the wait for it
+            // is not a wait for a load just issued.
+            const IO* const yag = static_cast<const IO*>(p.yacc) + (b * p.y_sb + (int64_t)d0 * p.y_sd);
+            IO yav[4];
+            auto load_yacc = [&](int kk) {
+                if (!p.yacc) return;
+                const int pc = phys_chunk(min(kk, ntiles - 1));
+                uint32_t wy = 0xffffffffu;
+                if (ragged_seq && pc == last_chunk) {
+                    const int64_t end = (p.batch - 1) * p.y_sb + (p.L - 1) * p.y_sl + (p.ED - 1) * p.y_sd + 1;
+                    wy = window_bytes(end, b * p.y_sb + (int64_t)pc * kTile * p.y_sl + (int64_t)d0 * p.y_sd, kES);
+                }
+                const IO* yak = yag + (int64_t)pc * kTile * p.y_sl;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) yav[j] = ld_off(yak, offy, syj[j], wy);
+            };
             auto reduce_store = [&](int k) {
                 const int pc = phys_chunk(k);
                 IO* yk = yg + (int64_t)pc * kTile * p.y_sl;
@@ -414,6 +431,9 @@ __global__ void __launch_bounds__((kFwdWaves<NW, MODE>) * kWave) sscan_fwd_kerne
                 for (int ww = 0; ww < NW; ++ww) {
                     const float4 v = *reinterpret_cast<const float4*>(&sY[(k & 1) * NW + ww][co][q4]);
                     s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
+                }
+                if (p.yacc) {
+                    s.x += to_float(yav[0]); s.y += to_float(yav[1]); s.z += to_float(yav[2]); s.w += to_float(yav[3]);
                 }
                 const int t0 = pc * kTile + 4 * qpo;  // lowest physical step of the item
                 const bool whole = !(ragged_seq && pc == last_chunk) || t0 + 3 < p.L;
@@ -440,6 +460,7 @@ __global__ void __launch_bounds__((kFwdWaves<NW, MODE>) * kWave) sscan_fwd_kerne
             __syncthreads();
             for (int k = 0; k < ntiles; ++k) {
                 if (k >= 1) reduce_store(k - 1);
+                load_yacc(k);
                 __syncthreads();
             }
             reduce_store(ntiles - 1);
@@ -455,9 +476,9 @@ __global__ void __launch_bounds__((kFwdWaves<NW, MODE>) * kWave) sscan_fwd_kerne
     for (int i = 0; i < NS; ++i) {
         const int n = w * NS + i;
         const bool ok = dvalid && n < p.N;
-        const int64_t dn = (int64_t)min(d, p.ED - 1) * p.N + min(n, p.N - 1);
-        const float av = p.A[dn];
-        const float hv = p.h0 ? p.h0[(int64_t)bs * p.ED * p.N + dn] : 0.0f;
+        const int dc = min(d, p.ED - 1), nc = min(n, p.N - 1);
+        const float av = p.A[(int64_t)dc * p.a_st + nc];
+        const float hv = p.h0 ? p.h0[((int64_t)bs * p.ED + dc) * p.h_st + nc] : 0.0f;
         A2[i] = ok ? av * kLog2e : 0.0f;
         h[i] = ok ? hv : 0.0f;
     }
@@ -491,7 +512,7 @@ __global__ void __launch_bounds__((kFwdWaves<NW, MODE>) * kWave) sscan_fwd_kerne
 #pragma unroll
             for (int i = 0; i < NS; ++i) {
                 const int n = w * NS + i;
-                if (n < p.N) p.ckpt[(((int64_t)b * p.nchunks + tile0 + k) * p.N + n) * p.ED + d] = h[i];
+                if (n < p.N) p.ckpt[(((int64_t)b * p.nchunks + tile0 + k) * p.ck_st + n) * p.ED + d] = h[i];
             }
         }
     };
@@ -606,7 +627,7 @@ __global__ void __launch_bounds__((kFwdWaves<NW, MODE>) * kWave) sscan_fwd_kerne
 #pragma unroll
         for (int i = 0; i < NS; ++i) {
             const int n = w * NS + i;
-            if (n < p.N) p.hlast[((int64_t)bs * p.ED + d) * p.N + n] = h[i];
+            if (n < p.N) p.hlast[((int64_t)bs * p.ED + d) * p.h_st + n] = h[i];
         }
     }
 }
@@ -619,15 +640,16 @@ __global__ void __launch_bounds__((kFwdWaves<NW, MODE>) * kWave) sscan_fwd_kerne
 __global__ void __launch_bounds__(256) seg_carry_kernel(const float* __restrict__ A, const float* __restrict__ h0,
                                                         const float* __restrict__ hend, const float* __restrict__ dsum,
                                                         float* __restrict__ segh0, float* __restrict__ hlast,
-                                                        int batch, int nseg, int ED, int N) {
+                                                        int batch, int nseg, int ED, int N, int a_st, int h_st) {
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     const int64_t per_b = (int64_t)ED * N;
     if (i >= batch * per_b) return;
     const int b = (int)(i / per_b);
     const int64_t dn = i - b * per_b;
-    const int d = (int)(dn / N);
-    const float a2 = A[dn] * kLog2e;
-    float h = h0 ? h0[i] : 0.0f;
+    const int d = (int)(dn / N), n = (int)(dn - (int64_t)d * N);
+    const float a2 = A[(int64_t)d * a_st + n] * kLog2e;
+    const int64_t ih = ((int64_t)b * ED + d) * h_st + n;  // in the caller's h0 / hlast
+    float h = h0 ? h0[ih] : 0.0f;
     for (int sg = 0; sg < nseg; ++sg) {
         const int64_t row = (int64_t)b * nseg + sg;
         segh0[row * per_b + dn] = h;
@@ -638,7 +660,7 @@ __global__ void __launch_bounds__(256) seg_carry_kernel(const float* __restrict_
         const float e = hend[row * per_b + dn];
         h = h == 0.0f ? e : __builtin_fmaf(fast_exp2(a2 * sd), h, e);
     }
-    if (hlast) hlast[i] = h;
+    if (hlast) hlast[ih] = h;
 }
 
 // Segments per batch row.  The scan is serial in time, so a launch has only batch * dim/64
@@ -716,10 +738,10 @@ int launch_fwd_any(const FwdParams& p, int io_dtype, int ns, int nw, int mode, h
 }
 
 int launch_seg_carry(const float* A, const float* h0, const float* hend, const float* dsum, float* segh0,
-                     float* hlast, int batch, int nseg, int ED, int N, hipStream_t st) {
+                     float* hlast, int batch, int nseg, int ED, int N, int a_st, int h_st, hipStream_t st) {
     const int64_t total = (int64_t)batch * ED * N;
     hipLaunchKernelGGL(seg_carry_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, A, h0, hend, dsum,
-                       segh0, hlast, batch, nseg, ED, N);
+                       segh0, hlast, batch, nseg, ED, N, a_st, h_st);
     return check_launch();
 }
 
@@ -803,10 +825,26 @@ extern "C" int64_t mpa_sscan_ckpt_elems(const mpa_sscan_shape* s) {
 // forward cut: a third of the CUs or fewer covered (see seg_plan)
 static constexpr int kFwdThin = 3;
 
+// d_state above 64: the states are independent given x, delta, B, C, so the call runs as passes
+// over blocks of 64 states on the broadcast path (8 states per lane, 8 scan waves; cut into segments
+// like any other launch), each pass adding its readout to the output.  A caller that pins more than
+// 8 states per lane gets the single launch with packed B/C instead.
+static constexpr int kFwdStateBlock = 64;
+static bool fwd_in_state_blocks(const mpa_sscan_shape* s) {
+    return s->dstate > kFwdStateBlock && s->plan_states_per_lane <= 8;
+}
+
 extern "C" size_t mpa_sscan_fwd_workspace_bytes(const mpa_sscan_shape* s, int with_ckpt) {
     (void)with_ckpt;  // both kinds of call are cut by the same rule
     if (validate_shape(s) != MPA_OK) return 0;
     // the packed B/C exist only on the scalar-load path (more than 8 states per lane)
+    if (fwd_in_state_blocks(s)) {
+        // passes over blocks of kFwdStateBlock states: the first block needs the most
+        mpa_sscan_shape sb = *s;
+        sb.dstate = kFwdStateBlock;
+        const int nsb = pick_states_per_lane(sb.batch, sb.dim, sb.dstate, 8, sb.plan_states_per_lane);
+        return (seg_plan(&sb, nsb, kFwdThin).floats * sizeof(float) + 255) / 256 * 256 + 256;
+    }
     const int ns = pick_states_per_lane(s->batch, s->dim, s->dstate, 32, s->plan_states_per_lane);
     if (ns <= 8) return (seg_plan(s, ns, kFwdThin).floats * sizeof(float) + 255) / 256 * 256 + 256;
     return (bcpack_floats(s) * sizeof(float) + 255) / 256 * 256;
@@ -829,15 +867,8 @@ static int sscan_fwd_impl(const mpa_sscan_shape* s, const void* x, const void* d
         return MPA_ERR_MISALIGNED;
     if (workspace_bytes < mpa_sscan_fwd_workspace_bytes(s, h_ckpt != nullptr)) return MPA_ERR_WORKSPACE;
 
-    const int np = padded_states(s->dstate);
-    const int ns = pick_states_per_lane(s->batch, s->dim, s->dstate, 32, s->plan_states_per_lane);
-    if (ns < 0) return MPA_ERR_BAD_SHAPE;
-    const int nw = np / ns;
     hipStream_t st = static_cast<hipStream_t>(stream);
-    if (ns > 8) {  // !kBcastBC<NS>: B/C go through the scalar cache, repacked per scan wave
-        rc = launch_pack_bc(s, B, C, static_cast<float*>(workspace), ns, 1 /* FwdPack<NS>::kSS */, st);
-        if (rc != MPA_OK) return rc;
-    }
+    float* wsf = static_cast<float*>(workspace);
 
     FwdParams p{};
     p.x = x; p.delta = delta; p.z = z; p.A = A; p.D = D;
@@ -845,6 +876,7 @@ static int sscan_fwd_impl(const mpa_sscan_shape* s, const void* x, const void* d
     p.Bm = B; p.C = C; p.bc_sb = s->bc_sb; p.bc_sl = s->bc_sl;
     p.y = y; p.ypre = z ? y_pregate : nullptr; p.ckpt = h_ckpt; p.hlast = h_last;
     p.batch = (int)s->batch; p.L = (int)s->seqlen; p.ED = (int)s->dim; p.N = (int)s->dstate;
+    p.a_st = p.h_st = p.ck_st = p.N;
     p.nchunks = (p.L + kTile - 1) / kTile;
     p.softplus = softplus ? 1 : 0;
     p.reverse = (s->flags & MPA_SSCAN_REVERSE) ? 1 : 0;
@@ -854,24 +886,67 @@ static int sscan_fwd_impl(const mpa_sscan_shape* s, const void* x, const void* d
     p.y_sb = s->y_sb; p.y_sl = s->y_sl; p.y_sd = s->y_sd;
     p.in_tmajor = (s->u_sd != 1 && s->u_sl == 1) ? 1 : 0;
     p.out_tmajor = (s->y_sd != 1 && s->y_sl == 1) ? 1 : 0;
-    const SegPlan sp = seg_plan(s, ns, kFwdThin);
-    if (sp.nseg <= 1) return launch_fwd_any(p, s->io_dtype, ns, nw, kScan, st);
 
-    // segmented mode: end states of every segment from zero, carry, then the real pass
-    float* wsf = static_cast<float*>(workspace);
-    FwdParams p1 = p;
-    p1.nseg = sp.nseg; p1.seg_tiles = sp.seg_tiles;
-    p1.z = nullptr; p1.y = nullptr; p1.ypre = nullptr; p1.h0 = nullptr; p1.ckpt = nullptr;
-    p1.hlast = wsf + sp.off_hend; p1.dsum = wsf + sp.off_dsum;
-    rc = launch_fwd_any(p1, s->io_dtype, ns, nw, kCarry, st);
-    if (rc != MPA_OK) return rc;
-    rc = launch_seg_carry(A, h0, wsf + sp.off_hend, wsf + sp.off_dsum, wsf + sp.off_h0, h_last, p.batch, sp.nseg,
-                          p.ED, p.N, st);
-    if (rc != MPA_OK) return rc;
-    FwdParams p2 = p;
-    p2.nseg = sp.nseg; p2.seg_tiles = sp.seg_tiles;
-    p2.h0 = wsf + sp.off_h0; p2.hlast = nullptr;
-    return launch_fwd_any(p2, s->io_dtype, ns, nw, kScan, st);
+    // the launches for the states q describes (q.N of them, pointers at the first one): one
+    // launch, or a sequence cut into segments (end states of every segment from zero, carry,
+    // then the real pass)
+    auto run_states = [&](const FwdParams& q, int ns, int nw, const SegPlan& sp) -> int {
+        if (sp.nseg <= 1) return launch_fwd_any(q, s->io_dtype, ns, nw, kScan, st);
+        FwdParams p1 = q;
+        p1.nseg = sp.nseg; p1.seg_tiles = sp.seg_tiles;
+        p1.z = nullptr; p1.y = nullptr; p1.ypre = nullptr; p1.yacc = nullptr; p1.h0 = nullptr; p1.ckpt = nullptr;
+        p1.hlast = wsf + sp.off_hend; p1.dsum = wsf + sp.off_dsum; p1.h_st = q.N;
+        int r = launch_fwd_any(p1, s->io_dtype, ns, nw, kCarry, st);
+        if (r != MPA_OK) return r;
+        r = launch_seg_carry(q.A, q.h0, wsf + sp.off_hend, wsf + sp.off_dsum, wsf + sp.off_h0, q.hlast, q.batch,
+                             sp.nseg, q.ED, q.N, q.a_st, q.h_st, st);
+        if (r != MPA_OK) return r;
+        FwdParams p2 = q;
+        p2.nseg = sp.nseg; p2.seg_tiles = sp.seg_tiles;
+        p2.h0 = wsf + sp.off_h0; p2.hlast = nullptr; p2.h_st = q.N;
+        return launch_fwd_any(p2, s->io_dtype, ns, nw, kScan, st);
+    };
+
+    if (fwd_in_state_blocks(s)) {
+        // The passes before the last write the sum of their readouts where the last one finds it:
+        // in y_pregate when there is a gate and the caller wants that output, else in y.  The last
+        // pass adds its own, writes the pre-gate output and applies the gate.
+        void* const ysum = (z && y_pregate) ? y_pregate : y;
+        const int nblk = (p.N + kFwdStateBlock - 1) / kFwdStateBlock;
+        for (int blk = 0; blk < nblk; ++blk) {
+            const int n0 = blk * kFwdStateBlock;
+            mpa_sscan_shape sb = *s;
+            sb.dstate = p.N - n0 < kFwdStateBlock ? p.N - n0 : kFwdStateBlock;
+            const int ns = pick_states_per_lane(sb.batch, sb.dim, sb.dstate, 8, sb.plan_states_per_lane);
+            if (ns < 0) return MPA_ERR_BAD_SHAPE;
+            const int nw = padded_states(sb.dstate) / ns;
+            const bool last = blk == nblk - 1;
+            FwdParams q = p;
+            q.N = (int)sb.dstate;
+            q.A = A + n0;
+            q.Bm = static_cast<const char*>(B) + n0 * es;
+            q.C = static_cast<const char*>(C) + n0 * es;
+            q.h0 = h0 ? h0 + n0 : nullptr;
+            q.hlast = h_last ? h_last + n0 : nullptr;
+            q.ckpt = h_ckpt ? h_ckpt + (int64_t)n0 * p.ED : nullptr;
+            q.D = blk == 0 ? D : nullptr;
+            q.yacc = blk > 0 ? ysum : nullptr;
+            if (!last) { q.z = nullptr; q.y = ysum; q.ypre = nullptr; }
+            rc = run_states(q, ns, nw, seg_plan(&sb, ns, kFwdThin));
+            if (rc != MPA_OK) return rc;
+        }
+        return MPA_OK;
+    }
+
+    const int np = padded_states(s->dstate);
+    const int ns = pick_states_per_lane(s->batch, s->dim, s->dstate, 32, s->plan_states_per_lane);
+    if (ns < 0) return MPA_ERR_BAD_SHAPE;
+    const int nw = np / ns;
+    if (ns > 8) {  // !kBcastBC<NS>: B/C go through the scalar cache, repacked per scan wave
+        rc = launch_pack_bc(s, B, C, wsf, ns, 1 /* FwdPack<NS>::kSS */, st);
+        if (rc != MPA_OK) return rc;
+    }
+    return run_states(p, ns, nw, seg_plan(s, ns, kFwdThin));
 }
 
 extern "C" int mpa_sscan_fwd(const mpa_sscan_shape* s, const void* x, const void* delta,

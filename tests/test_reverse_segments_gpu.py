@@ -242,7 +242,7 @@ def test_batch_one_training_is_cut_by_the_library(pkg, dev):
 
 @pytest.mark.parametrize("N,ED,L", [(96, 70, 50), (128, 64, 130), (256, 64, 40), (100, 130, 33)])
 def test_forward_wide_state(pkg, dev, N, ED, L):
-    # 64 < d_state <= 256: 16 or 32 states per lane, B and C packed for scalar loads
+    # 64 < d_state <= 256: passes over blocks of 64 states, each adding its readout to the output
     inp = so.make_inputs(2, L, ED, N, seed=500 + N)
     g = torch.Generator().manual_seed(501 + N)
     h0 = torch.randn(2, ED, N, generator=g)
@@ -252,6 +252,32 @@ def test_forward_wide_state(pkg, dev, N, ED, L):
                                           return_last_state=True)
     assert rel_err(y, ref) <= TOL[torch.float32]
     assert rel_err(h_last, hl) <= TOL[torch.float32]
+    # a caller that pins 16 or 32 states per lane gets the single launch with packed B and C
+    with torch.no_grad(), pkg.plan_override(fwd_states_per_lane=32 if N > 128 else 16):
+        y2 = pkg.selective_scan_fn(*[inp[k].to(dev) for k in NAMES], h0=h0.to(dev))
+    assert rel_err(y2, ref) <= TOL[torch.float32]
+
+
+def test_forward_wide_state_gated_bf16_pregate(pkg, dev):
+    # gate + softplus at d_state 160 in bf16: the passes before the last add up in the pre-gate
+    # output, the last one applies the gate
+    Bs, L, ED, N = 2, 77, 96, 160
+    inp = so.make_inputs(Bs, L, ED, N, seed=540, dtype=torch.bfloat16)
+    g = torch.Generator().manual_seed(541)
+    z = torch.randn(Bs, L, ED, generator=g).to(torch.bfloat16)
+    raw = (torch.randn(Bs, L, ED, generator=g) * 0.5 - 4.0).to(torch.bfloat16)
+    bias = torch.randn(ED, generator=g) * 0.3
+    delta = so.softplus_ref(raw.double() + bias.double())
+    yr = so.selective_scan_ref(inp["x"].double(), delta, inp["A"].double(), inp["B"].double(), inp["C"].double(),
+                               inp["D"].double())
+    yr = yr * (z.double() * torch.sigmoid(z.double()))
+    args = [inp["x"].to(dev), raw.to(dev)] + [inp[k].to(dev) for k in ("A", "B", "C", "D")]
+    with torch.no_grad():
+        y = pkg.selective_scan_fn(*args, z=z.to(dev), delta_bias=bias.to(dev), delta_softplus=True)
+    assert rel_err(y, yr) <= TOL[torch.bfloat16]
+    t = [a.clone().requires_grad_() for a in args]
+    y2 = pkg.selective_scan_fn(*t, z=z.to(dev).requires_grad_(), delta_bias=bias.to(dev), delta_softplus=True)
+    assert rel_err(y2, yr) <= TOL[torch.bfloat16]
 
 
 # ---------------------------------------------------------------------------------------------
@@ -335,10 +361,47 @@ def test_pscan_thin_long_sequence_is_cut_by_the_library(pkg, dev):
     (80, 64, 17, torch.float32), (128, 96, 100, torch.bfloat16),
 ])
 def test_backward_wide_state(pkg, dev, N, ED, L, dtype):
+    # passes over blocks of 16 states on the fast kernel (dx, ddelta add up over the passes)
     inp = so.make_inputs(2, L, ED, N, seed=700 + N, dtype=dtype)
     ref = c_oracle.sscan_fwd_bwd(**inp)
     got = run_gpu_fwd_bwd(pkg, inp, dev)
     _check(got, ref, TOL[dtype], f"N={N}")
+
+
+@pytest.mark.parametrize("N,ED,L", [(32, 64, 48), (64, 65, 40), (24, 64, 129), (128, 64, 70), (200, 40, 33)])
+def test_backward_wide_state_general_kernel(pkg, dev, N, ED, L):
+    # the general kernel (32 or 64 states per launch, passes over blocks of 64 above that), which a
+    # gated call without the saved pre-gate output still uses
+    inp = so.make_inputs(2, L, ED, N, seed=760 + N)
+    ref = c_oracle.sscan_fwd_bwd(**inp)
+    with pkg.plan_override(bwd_general=True):
+        got = run_gpu_fwd_bwd(pkg, inp, dev)
+    _check(got, ref, TOL[torch.float32], f"general N={N}")
+
+
+@pytest.mark.parametrize("Bs,L,ED,N,nseg,reverse", [
+    (1, 160, 64, 48, 2, False), (2, 333, 70, 80, 3, True), (1, 1000, 96, 160, 7, False), (1, 517, 64, 256, 4, True),
+])
+def test_wide_state_cut_into_segments(pkg, dev, Bs, L, ED, N, nseg, reverse):
+    # state blocks and segments together: forward in passes of 64 states, backward in passes of 16,
+    # every pass cut into nseg segments with its own carry
+    inp = so.make_inputs(Bs, L, ED, N, seed=780 + N + nseg)
+    ref = _reverse_oracle(inp) if reverse else c_oracle.sscan_fwd_bwd(**inp)
+    with pkg.plan_override(fwd_segments=nseg, bwd_segments=nseg):
+        got = run_gpu_fwd_bwd(pkg, inp, dev, reverse=reverse)
+    _check(got, ref, TOL[torch.float32], f"N={N} nseg={nseg}")
+    with pkg.plan_override(fwd_segments=nseg, bwd_segments=nseg):
+        again = run_gpu_fwd_bwd(pkg, inp, dev, reverse=reverse)
+    for k in ("y",) + GRAD_KEYS:
+        assert torch.equal(got[k], again[k]), f"{k} differs between two runs"
+
+
+def test_batch_one_wide_state_is_cut_by_the_library(pkg, dev):
+    # the regime of the reference's d_state plot (README.md:181-196): batch 1, d_model 1024, N = 64
+    inp = so.make_inputs(1, 1024, 256, 64, seed=799, dtype=torch.bfloat16)
+    ref = c_oracle.sscan_fwd_bwd(**inp)
+    got = run_gpu_fwd_bwd(pkg, inp, dev)
+    _check(got, ref, TOL[torch.bfloat16], "B=1 N=64")
 
 
 def test_backward_wide_state_gated_softplus_reverse(pkg, dev):

@@ -69,9 +69,11 @@ def test_noalloc_forward_twice_second_call_smaller(pkg, dev):
 def test_noalloc_refuses_what_does_not_fit(pkg, dev):
     L_ = pkg._lib
     lib = L_.load()
-    # d_state 256 over a long sequence: the packed B/C alone are 8 * 512 * 2 * 16 * 256 floats
+    # d_state 256 over a long sequence as one launch (32 states per lane pinned): the packed B/C
+    # alone are 8 * 512 * 2 * 16 * 256 floats
     s = L_.SscanShape()
     s.batch, s.seqlen, s.dim, s.dstate = 8, 8192, 64, 256
+    s.plan_states_per_lane = 32
     assert lib.mpa_sscan_fwd_workspace_bytes(ctypes.byref(s), 0) > L_.MPA_NOALLOC_SCRATCH_BYTES
     assert lib.mpa_sscan_fwd_noalloc(ctypes.byref(s), *([None] * 13), None) == 6   # MPA_ERR_WORKSPACE
     assert lib.mpa_status_string(6) == b"workspace too small"
