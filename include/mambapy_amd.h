@@ -115,6 +115,8 @@ const char* mpa_status_string(int status);
  *   y_pregate  optional, only with z: the output before the gate (C.h + D*x), io_dtype, strides
  *            of y.  mpa_sscan_bwd needs it on its fast path; NULL when no gradient is needed.
  *   workspace  scratch of mpa_sscan_fwd_workspace_bytes() bytes.
+ * d_state above 64 runs in passes over blocks of 64 states, each adding its readout to y (in
+ * y_pregate when that is given) in io_dtype.
  * When batch * dim/64 workgroups would cover a fraction of the chip, the sequence is cut into
  * segments that run side by side (end states of all segments from zero, a carry pass, then the
  * real pass from the true initial states); checkpoints, h_last and y are the same as without the
@@ -143,8 +145,8 @@ size_t mpa_sscan_fwd_workspace_bytes(const mpa_sscan_shape* s, int with_ckpt);
  * every GPU it runs on, held until the process ends.  The call allocates and frees nothing.
  * A shape whose mpa_sscan_fwd_workspace_bytes() exceeds MPA_NOALLOC_SCRATCH_BYTES is refused with
  * MPA_ERR_WORKSPACE before anything is launched (sequences cut into segments need
- * 2 * batch * segments * dim * dstate floats and a little more; d_state above 64 needs the packed
- * B/C of the whole sequence).  All calls on one GPU share that GPU's array: calls that overlap
+ * 2 * batch * segments * dim * min(dstate, 64) floats and a little more; a caller that pins 16 or
+ * 32 states per lane needs the packed B/C of the whole sequence).  All calls on one GPU share that GPU's array: calls that overlap
  * on one GPU (different streams or threads) race; calls on one stream are ordered.
  */
 #define MPA_NOALLOC_SCRATCH_BYTES (16u << 20)
@@ -164,8 +166,10 @@ int mpa_sscan_fwd_noalloc(const mpa_sscan_shape* s, const void* x, const void* d
  * given.  y_pregate (strides of dy) is what the forward call wrote for the same inputs; with z
  * and y_pregate == NULL the pre-gate output is recomputed by a slower, more general kernel.
  * `workspace` needs mpa_sscan_bwd_workspace_bytes() bytes, 256-byte aligned.
- * d_state up to MPA_MAX_DSTATE.  Short batches of long sequences are cut into segments as in
- * the forward call (the carry runs from the end).
+ * d_state up to MPA_MAX_DSTATE; above 16 the call runs in passes over blocks of 16 states (the
+ * states are independent given x, delta, B, C), dx and ddelta being summed over the passes in
+ * io_dtype.  Short batches of long sequences are cut into segments as in the forward call (the
+ * carry runs from the end).
  * One kernel waits, with a bound, for a counter in shared memory; the wait cannot run out
  * unless the hardware scheduler misbehaves, and if it ever does the call does not return clean
  * numbers: dA of every channel whose sums may have been damaged is NaN.
