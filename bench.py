@@ -447,15 +447,16 @@ def bench_thin(args, torch, pkg, dev):
 def bench_block(args, torch, pkg, dev):
     """The regime of the reference's own plots (README.md:169-204: one whole MambaBlock, forward +
     backward, batch 1, fp32, timed on an A100 80GB): d_model 1024 and 2048 at N=16, and d_model 1024
-    at N = 64, 128, 256, all at L=4096.  `published_ms_*` are the reference's figures read off its
-    PNG plots by eye (+-10-15 %, other hardware): context, not a like-for-like baseline."""
+    at N = 64, 128, 256, all at L=4096, and d_model 1024, N=16 at L=65536.  `published_ms_*` are the
+    reference's figures read off its PNG plots by eye (+-10-15 %, other hardware): context, not a
+    like-for-like baseline."""
     steps, warmup = max(3, args.steps // 5), 2
-    published = {  # (d_model, N): (mamba.py pscan, official CUDA kernel), milliseconds on A100
-        (1024, 16): (49, 26), (2048, 16): (110, 55), (1024, 64): (140, 28), (1024, 128): (260, 29),
-        (1024, 256): (500, 38)}
+    published = {  # (d_model, N, L): (mamba.py pscan, official CUDA kernel), milliseconds on A100
+        (1024, 16, 4096): (49, 26), (2048, 16, 4096): (110, 55), (1024, 64, 4096): (140, 28),
+        (1024, 128, 4096): (260, 29), (1024, 256, 4096): (500, 38), (1024, 16, 65536): (760, 410)}
     rows = {}
-    B, L = 1, 4096
-    for (d_model, N), (ref_ms, cuda_ms) in published.items():
+    B = 1
+    for (d_model, N, L), (ref_ms, cuda_ms) in published.items():
         torch.manual_seed(1020 + N)
         blk = pkg.MambaBlock(pkg.MambaConfig(d_model=d_model, n_layers=1, d_state=N)).to(dev)
         x = torch.randn(B, L, d_model, device=dev, requires_grad=True)
@@ -467,9 +468,9 @@ def bench_block(args, torch, pkg, dev):
             blk(x).sum().backward()
 
         t = _timed(torch, step, steps, warmup)
-        rows[f"d_model{d_model}_N{N}"] = {"ms": t * 1e3, "tokens_per_s": B * L / t,
-                                          "published_ms_mambapy_pscan_A100": ref_ms,
-                                          "published_ms_official_cuda_A100": cuda_ms}
+        rows[f"d_model{d_model}_N{N}" + ("" if L == 4096 else f"_L{L}")] = {
+            "ms": t * 1e3, "tokens_per_s": B * L / t,
+            "published_ms_mambapy_pscan_A100": ref_ms, "published_ms_official_cuda_A100": cuda_ms}
         del blk, x
         torch.cuda.empty_cache()
     head = rows["d_model1024_N16"]
@@ -479,7 +480,7 @@ def bench_block(args, torch, pkg, dev):
         "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": head["ms"],
         "scaling": "weak", "vs_baseline": None, "dtype": "f32",
         "data": "synthetic (random-init weights, N(0,1) input)",
-        "config": {"workload": "one MambaBlock fwd+bwd, B=1 L=4096 fp32: d_model 1024 / 2048 at N=16, d_model 1024 at N=64 / 128 / 256"},
+        "config": {"workload": "one MambaBlock fwd+bwd, B=1 fp32: L=4096 with d_model 1024 / 2048 at N=16 and d_model 1024 at N=64 / 128 / 256; L=65536 with d_model 1024, N=16"},
         "rows": rows,
     }
 
