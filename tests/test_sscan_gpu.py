@@ -365,6 +365,18 @@ def test_errors_are_reported_not_undefined(pkg, dev):
 def test_random_shapes_layouts_and_options(pkg, dev, seed):
     # seeded sweep over ragged shapes, both memory layouts, fp32 / bf16, gate + softplus + bias, initial
     # state: forward, last state and every gradient against the float64 definition
+    _random_case(pkg, dev, seed, wide=False)
+
+
+@pytest.mark.parametrize("seed", range(100, 116))
+def test_random_wide_state_directions_and_segments(pkg, dev, seed):
+    # the same sweep at d_state 40 ... 256 (passes over blocks of states), in either direction and with
+    # the sequence cut into segments
+    _random_case(pkg, dev, seed, wide=True)
+
+
+def _random_case(pkg, dev, seed, wide):
+    import contextlib
     import random
     rnd = random.Random(1234 + seed)
     Bs, L = rnd.randint(1, 3), rnd.choice([1, 2, 15, 16, 17, 31, 33, 47, 64, 65, 100, 129, 200])
@@ -372,6 +384,12 @@ def test_random_shapes_layouts_and_options(pkg, dev, seed):
     N = rnd.choice([1, 2, 4, 7, 8, 12, 15, 16, 16, 16, 16, 24, 32, 64])
     dtype = rnd.choice([torch.float32, torch.float32, torch.bfloat16])
     gated, tmajor, with_h0 = rnd.random() < 0.5, rnd.random() < 0.4, rnd.random() < 0.5
+    reverse, nseg = False, None
+    if wide:
+        N = rnd.choice([40, 65, 80, 96, 128, 130, 200, 256])
+        ED = rnd.choice([3, 31, 64, 65, 96])
+        L = rnd.choice([1, 17, 33, 64, 100, 129])
+        reverse, nseg = rnd.random() < 0.5, rnd.choice([None, None, 2, 3])
     inp = so.make_inputs(Bs, L, ED, N, seed=9000 + seed, dtype=dtype)
     g = torch.Generator().manual_seed(9100 + seed)
     z = torch.randn(Bs, L, ED, generator=g).to(dtype)
@@ -382,8 +400,10 @@ def test_random_shapes_layouts_and_options(pkg, dev, seed):
     x, dl, A, Bm, C, D = map(f64, (inp["x"], raw if gated else inp["delta"], inp["A"], inp["B"], inp["C"], inp["D"]))
     zz, bb = f64(z), f64(bias)
     delta = so.softplus_ref(dl + bb) if gated else dl
-    yr, hl = so.selective_scan_ref(x, delta, A, Bm, C, D, h0=None if h0 is None else h0.double(),
+    fl = (lambda t: t.flip(1)) if reverse else (lambda t: t)
+    yr, hl = so.selective_scan_ref(fl(x), fl(delta), A, fl(Bm), fl(C), D, h0=None if h0 is None else h0.double(),
                                    return_last_state=True)
+    yr = fl(yr)
     if gated:
         yr = yr * (zz * torch.sigmoid(zz))
     yr.backward(inp["dy"].double())
@@ -399,14 +419,16 @@ def test_random_shapes_layouts_and_options(pkg, dev, seed):
     gz = lay(z).requires_grad_()
     gA, gB, gC, gD, gb = (t.to(dev).requires_grad_() for t in (inp["A"], inp["B"], inp["C"], inp["D"], bias))
     kw = dict(z=gz, delta_bias=gb, delta_softplus=True) if gated else {}
-    y, hg = pkg.selective_scan_fn(gx, gd, gA, gB, gC, gD, h0=None if h0 is None else h0.to(dev),
-                                  return_last_state=True, **kw)
-    y.backward(inp["dy"].to(dev))
+    plan = pkg.plan_override(fwd_segments=nseg, bwd_segments=nseg) if nseg else contextlib.nullcontext()
+    with plan:
+        y, hg = pkg.selective_scan_fn(gx, gd, gA, gB, gC, gD, h0=None if h0 is None else h0.to(dev),
+                                      return_last_state=True, reverse=reverse, **kw)
+        y.backward(inp["dy"].to(dev))
     got = dict(y=y, hl=hg, dx=gx.grad, ddelta=gd.grad, dA=gA.grad, dB=gB.grad, dC=gC.grad, dD=gD.grad)
     if gated:
         got.update(dz=gz.grad, dbias=gb.grad)
     tol = TOL[dtype]
-    what = f"B{Bs} L{L} ED{ED} N{N} {dtype} gated={gated} tmajor={tmajor} h0={with_h0}"
+    what = f"B{Bs} L{L} ED{ED} N{N} {dtype} gated={gated} tmajor={tmajor} h0={with_h0} reverse={reverse} nseg={nseg}"
     for k in ref:
         scale = ref[k].abs().max().item()
         if scale == 0.0:
