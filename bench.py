@@ -46,6 +46,36 @@ def measured_traffic_bytes(workload):
         return None
 
 
+def measured_valu_insts(workload, entry):
+    """Wave-level VALU instructions per launch of an entry point's scan kernel (rocprofv3 --pmc
+    SQ_INSTS_VALU), read from the same summary (a line `valu_insts_per_launch <workload> <entry>
+    = <number>`); None when there is none."""
+    import re
+    path = os.path.join(ROOT, "profiles", f"sscan_fwd_bwd_{workload}_pmc.md")
+    try:
+        m = re.search(rf"valu_insts_per_launch\s+{workload}\s+{entry}\s*=\s*([0-9.eE+-]+)", open(path).read())
+        return float(m.group(1)) if m else None
+    except OSError:
+        return None
+
+
+# Plain fp32 wave64 instructions per second the chip can issue: 1024 SIMDs x 2.4 GHz / 2 clocks
+# (the published 157.3 TFLOP/s divided by the 128 flops of one wave-wide FMA).
+VALU_PEAK_GINST = 1024 * 2.4 / 2.0
+
+
+def valu_issue(workload, entry, ms):
+    """What actually bounds the scan kernels: the rate of VALU instructions, against the rate of
+    plain fp32 instructions (a DPP operand costs about twice, exp2 and lane swaps four times a plain
+    instruction, so the attainable fraction of this peak is well below one)."""
+    n = measured_valu_insts(workload, entry)
+    if n is None:
+        return None
+    ach = n / (ms * 1e-3) / 1e9
+    return {"wave_insts_per_launch": n, "achieved": ach, "peak": VALU_PEAK_GINST,
+            "unit": "G wave64 instructions/s", "frac": ach / VALU_PEAK_GINST}
+
+
 def algorithmic_bytes(B, L, ED, N, s):
     """Bytes that must cross HBM: fwd reads x, delta, B, C, A, D and writes y; bwd reads
     x, delta, dy, B, C, A, D and writes dx, ddelta, dB, dC, dA, dD (s = I/O element size;
@@ -591,10 +621,12 @@ def bench_sscan(args, torch, pkg, dev, workload, steps, warmup, prewarm, cpu=Tru
         "roofline": {"bound": "hbm", "kernel": "mpa_sscan_bwd (sscan_bwd_fast_kernel + sscan_bwd_finish_kernel)",
                      "achieved": bwd_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": bwd_gbs / HBM_PEAK_GBS,
-                     "traffic": measured_traffic_bytes(workload)},
+                     "traffic": measured_traffic_bytes(workload),
+                     "valu_issue": valu_issue(workload, "mpa_sscan_bwd", bwd_ms)},
         "forward": {"kernel": "mpa_sscan_fwd (sscan_fwd_kernel)",
                     "achieved": fwd_b / (fwd_ms * 1e-3) / 1e9, "unit": "GB/s",
-                    "frac": fwd_b / (fwd_ms * 1e-3) / 1e9 / HBM_PEAK_GBS},
+                    "frac": fwd_b / (fwd_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                    "valu_issue": valu_issue(workload, "mpa_sscan_fwd", fwd_ms)},
     }
     del gpu, dy, inp
     torch.cuda.empty_cache()
