@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the selective-scan hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c1|c0|c3|c4|c4-3000|pscan|thin|layer|generate]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c1|c0|c3|c4|c4-3000|pscan|thin|block|gated|layer|generate|issue-probe]
 
 One step = one forward + one backward of the fused selective scan over one batch of
 seeded synthetic input that is already resident in HBM.  Prints ONE JSON line.
@@ -353,6 +353,75 @@ def bench_layer_kernels(args, torch, pkg, dev):
     return out
 
 
+def bench_gated(args, torch, pkg, dev):
+    """The fused form of the scan as a layer calls it (mambapy/mamba.py:252-261 reaches it through
+    `use_cuda`): softplus(delta + bias) and the gate y * silu(z) inside the kernels, forward +
+    backward, at the configs[2] shape and at the configs[4] layer shape, bf16 I/O.  Beside it the
+    same computation with the two element-wise steps left to PyTorch around the plain scan (what the
+    reference's pscan path does, mamba.py:264-270 and :229-231): four more passes over (B, L, ED)
+    tensors per direction."""
+    import torch.nn.functional as F
+    import synthetic_inputs
+    rows = {}
+    steps = max(5, args.steps // 2)
+    for name, (B, L, ED, N) in (("B4_L4096_ED4096", (4, 4096, 4096, 16)), ("B8_L4096_ED1536", (8, 4096, 1536, 16))):
+        inp = synthetic_inputs.make_inputs(B, L, ED, N, seed=1007, dtype=torch.bfloat16)
+        g = torch.Generator().manual_seed(1008)
+        leaf = lambda t: t.to(dev).requires_grad_()
+        x, A, Bm, C, D = (leaf(inp[k]) for k in ("x", "A", "B", "C", "D"))
+        raw = leaf((torch.randn(B, L, ED, generator=g) * 0.5 - 4.0).to(torch.bfloat16))
+        z = leaf(torch.randn(B, L, ED, generator=g).to(torch.bfloat16))
+        bias = leaf(torch.randn(ED, generator=g) * 0.3)
+        dy = inp["dy"].to(dev)
+        leaves = (x, raw, A, Bm, C, D, z, bias)
+
+        def fused(ev=None):
+            for t in leaves:
+                t.grad = None
+            if ev:
+                ev[0].record()
+            y = pkg.selective_scan_fn(x, raw, A, Bm, C, D, z=z, delta_bias=bias, delta_softplus=True)
+            if ev:
+                ev[1].record()
+            y.backward(dy)
+            if ev:
+                ev[2].record()
+
+        def unfused():
+            for t in leaves:
+                t.grad = None
+            delta = F.softplus(raw + bias.to(raw.dtype))
+            y = pkg.selective_scan_fn(x, delta, A, Bm, C, D) * F.silu(z)
+            y.backward(dy)
+
+        t_f = _timed(torch, fused, steps, 3, settle_s=0.3)
+        evs = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(steps)]
+        for e in evs:
+            fused(e)
+        torch.cuda.synchronize()
+        fwd_ms = sum(e[0].elapsed_time(e[1]) for e in evs) / len(evs)
+        bwd_ms = sum(e[1].elapsed_time(e[2]) for e in evs) / len(evs)
+        t_u = _timed(torch, unfused, steps, 3, settle_s=0.3)
+        # fused: fwd reads x, delta, z, B, C and writes y; bwd reads x, delta, z, dy, B, C and
+        # writes dx, ddelta, dz, dB, dC (the saved pre-gate output is not counted)
+        s_ = 2
+        alg = s_ * (4 * B * L * ED + 2 * B * L * N) + s_ * (7 * B * L * ED + 4 * B * L * N) + 4 * (3 * ED * N + 5 * ED)
+        rows[name] = {"ms_fused": t_f * 1e3, "fwd_ms": fwd_ms, "bwd_ms": bwd_ms, "ms_elementwise_outside": t_u * 1e3,
+                      "speedup": t_u / t_f, "GBps_fused": alg / t_f / 1e9, "tokens_per_s_fused": B * L / t_f}
+        del x, raw, z, dy, leaves, inp
+        torch.cuda.empty_cache()
+    first = rows["B4_L4096_ED4096"]
+    return {
+        "metric": "fused softplus(delta+bias) + scan + gate fwd+bwd GB/s, B=4 L=4096 ED=4096 N=16 bf16",
+        "value": first["GBps_fused"], "unit": "GB/s", "higher_is_better": True, "n_gpus": 1, "steps": steps, "warmup": 3,
+        "ms_per_step": first["ms_fused"], "fwd_ms": first["fwd_ms"], "bwd_ms": first["bwd_ms"],
+        "pct_hbm_peak": 100.0 * first["GBps_fused"] / HBM_PEAK_GBS, "tokens_per_s": first["tokens_per_s_fused"],
+        "scaling": "weak", "vs_baseline": None, "dtype": "f32 state/accumulation, bf16 I/O", "data": "synthetic (seeded)",
+        "rows": rows,
+        "config": {"workload": "scan with softplus, bias and gate inside the kernels: configs[2] shape and configs[4] layer shape"},
+    }
+
+
 def bench_generate(args, torch, pkg, dev):
     """Generation with the mamba-130m architecture (random-init, bf16): one prefill of a 512-token
     prompt, then 128 greedy tokens, (a) with LM.step per token, (b) with the step replayed as a
@@ -653,7 +722,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--prewarm", type=int, default=40,
                     help="untimed start-up steps before the W warm-up steps (device clocks, allocator)")
-    ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS) + ["c3", "c4", "c4-3000", "pscan", "layer", "generate", "thin", "block", "issue-probe"],
+    ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS) + ["c3", "c4", "c4-3000", "pscan", "layer", "generate", "thin", "block", "gated", "issue-probe"],
                     help="c2 (default) is the headline workload; c3 = decode step, c4 = LM forward "
                          "(reported with their own metric, same one-line schema)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -684,7 +753,7 @@ def main():
     dev = torch.device("cuda:0")
 
     single = {"c3": bench_decode, "pscan": bench_pscan, "layer": bench_layer_kernels,
-              "generate": bench_generate, "thin": bench_thin, "block": bench_block}
+              "generate": bench_generate, "thin": bench_thin, "block": bench_block, "gated": bench_gated}
     if args.workload in single:
         out = single[args.workload](args, torch, pkg, dev)
     elif args.workload.startswith("c4"):
@@ -709,6 +778,8 @@ def main():
             other["thin"] = _brief(bench_thin(args, torch, pkg, dev))
             torch.cuda.empty_cache()
             other["block"] = _brief(bench_block(args, torch, pkg, dev))
+            torch.cuda.empty_cache()
+            other["gated"] = _brief(bench_gated(args, torch, pkg, dev))
             out["other"] = other
     print(json.dumps(out))
 
