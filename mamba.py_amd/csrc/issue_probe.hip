@@ -32,7 +32,9 @@ enum Stream {
 
 // 64 VALU instructions per loop iteration in every stream
 template <int STREAM>
-__global__ void probe_kernel(float* out, int iters) {
+__global__ void probe_kernel(float* out, long long* ticks, int iters) {
+    // shader-clock and constant 100 MHz counters around the stream: the clock the part really runs at
+    const long long c0 = __builtin_readcyclecounter(), w0 = wall_clock64();
     float v0 = threadIdx.x * 1e-6f + 1.0f, v1 = v0 + 1, v2 = v0 + 2, v3 = v0 + 3, v4 = v0 + 4, v5 = v0 + 5, v6 = v0 + 6,
           v7 = v0 + 7;
     const float c = 0.999f, d = 1e-3f;
@@ -133,11 +135,16 @@ __global__ void probe_kernel(float* out, int iters) {
         }
     }
     out[blockIdx.x * blockDim.x + threadIdx.x] = v0 + v1 + v2 + v3 + v4 + v5 + v6 + v7;
+    if (blockIdx.x == gridDim.x / 2 && threadIdx.x == 0) {
+        ticks[0] = __builtin_readcyclecounter() - c0;
+        ticks[1] = wall_clock64() - w0;
+    }
 }
 
 template <int STREAM>
-static int run(const char* name, float* out, double clock_hz) {
+static int run(const char* name, float* out, long long* ticks, double clock_hz) {
     const int iters = 2000;
+    double mhz3 = 0.0, mhz8 = 0.0;
     printf("%-34s", name);
     for (int waves_per_simd : {1, 2, 3, 4, 8}) {
         dim3 block(64 * 4 * waves_per_simd), grid(256);
@@ -151,7 +158,7 @@ static int run(const char* name, float* out, double clock_hz) {
         float best = 1e30f;
         for (int rep = 0; rep < 3; ++rep) {
             CK(hipEventRecord(e0));
-            hipLaunchKernelGGL(probe_kernel<STREAM>, grid, block, 0, 0, out, iters);
+            hipLaunchKernelGGL(probe_kernel<STREAM>, grid, block, 0, 0, out, ticks, iters);
             CK(hipEventRecord(e1));
             CK(hipEventSynchronize(e1));
             float ms;
@@ -161,8 +168,12 @@ static int run(const char* name, float* out, double clock_hz) {
         CK(hipEventDestroy(e0));
         CK(hipEventDestroy(e1));
         printf(" %6.2f", best * 1e-3 * clock_hz / (64.0 * iters * waves_per_simd));
+        long long t[2];
+        CK(hipMemcpy(t, ticks, sizeof(t), hipMemcpyDeviceToHost));
+        if (waves_per_simd == 3 && t[1] > 0) mhz3 = 100.0 * (double)t[0] / (double)t[1];
+        if (waves_per_simd == 8 && t[1] > 0) mhz8 = 100.0 * (double)t[0] / (double)t[1];
     }
-    printf("\n");
+    printf("   | %5.0f %5.0f MHz\n", mhz3, mhz8);
     return 0;
 }
 
@@ -171,20 +182,24 @@ int main() {
     CK(hipGetDeviceProperties(&prop, 0));
     const double clock_hz = prop.clockRate * 1e3;  // the nominal shader clock; the part may run below it
     float* out;
+    long long* ticks;
     CK(hipMalloc(&out, 4 << 20));
+    CK(hipMalloc(&ticks, 2 * sizeof(long long)));
     printf("%s, %d CUs, nominal shader clock %.0f MHz\n", prop.gcnArchName, prop.multiProcessorCount, clock_hz / 1e6);
-    printf("clocks per wave64 VALU instruction and SIMD, with 1 / 2 / 3 / 4 / 8 waves on the SIMD\n");
+    printf("clocks per wave64 VALU instruction and SIMD (kernel time x nominal clock), with 1 / 2 / 3 / 4 / 8 waves on\n"
+           "the SIMD; last columns: shader clock read inside the kernel (cycle counter / 100 MHz counter) at 3 and at 8 waves\n");
     int rc = 0;
-    rc |= run<kFmaIndependent>("v_fma_f32, 8 independent chains", out, clock_hz);
-    rc |= run<kFmaDependent>("v_fma_f32, one dependent chain", out, clock_hz);
-    rc |= run<kExp>("v_exp_f32, independent", out, clock_hz);
-    rc |= run<kExpDependent>("v_exp_f32, one dependent chain", out, clock_hz);
-    rc |= run<kDppBroadcast>("v_fmac_f32_dpp row_newbcast", out, clock_hz);
-    rc |= run<kLaneSwap32>("v_permlane32_swap_b32", out, clock_hz);
-    rc |= run<kForwardMix>("forward step mix, DPP broadcast", out, clock_hz);
-    rc |= run<kForwardMixPlain>("forward step mix, plain operands", out, clock_hz);
-    rc |= run<kBackwardMix>("backward step mix, DPP broadcast", out, clock_hz);
-    rc |= run<kBackwardMixPlain>("backward step mix, plain operands", out, clock_hz);
+    rc |= run<kFmaIndependent>("v_fma_f32, 8 independent chains", out, ticks, clock_hz);
+    rc |= run<kFmaDependent>("v_fma_f32, one dependent chain", out, ticks, clock_hz);
+    rc |= run<kExp>("v_exp_f32, independent", out, ticks, clock_hz);
+    rc |= run<kExpDependent>("v_exp_f32, one dependent chain", out, ticks, clock_hz);
+    rc |= run<kDppBroadcast>("v_fmac_f32_dpp row_newbcast", out, ticks, clock_hz);
+    rc |= run<kLaneSwap32>("v_permlane32_swap_b32", out, ticks, clock_hz);
+    rc |= run<kForwardMix>("forward step mix, DPP broadcast", out, ticks, clock_hz);
+    rc |= run<kForwardMixPlain>("forward step mix, plain operands", out, ticks, clock_hz);
+    rc |= run<kBackwardMix>("backward step mix, DPP broadcast", out, ticks, clock_hz);
+    rc |= run<kBackwardMixPlain>("backward step mix, plain operands", out, ticks, clock_hz);
     CK(hipFree(out));
+    CK(hipFree(ticks));
     return rc;
 }
