@@ -122,3 +122,53 @@ def test_host_threads_on_their_own_streams_get_the_serial_bits(pkg, dev):
         t.join(timeout=100)
     assert not any(t.is_alive() for t in threads)
     assert errors == []
+
+
+@pytest.mark.parametrize("gated", [False, True])
+def test_forward_backward_captured_in_a_hip_graph(pkg, dev, gated):
+    """The entry points allocate nothing, clear nothing with memset nodes and wait for nothing, so a
+    training step of the scan can be recorded once and replayed: three replays on new input values,
+    with eager calls and synchronisations in between, each equal to the eager result bit for bit."""
+    shape, dtype = (2, 300, 130, 16), torch.bfloat16 if gated else torch.float32
+    names = ("x", "delta", "A", "B", "C", "D")
+
+    def values(seed):
+        inp = so.make_inputs(*shape, seed=seed, dtype=dtype)
+        g = torch.Generator().manual_seed(seed + 1)
+        z = torch.randn(shape[0], shape[1], shape[2], generator=g).to(dtype)
+        bias = torch.randn(shape[2], generator=g) * 0.3
+        return [inp[k] for k in names] + [z, bias, inp["dy"]]
+
+    def call(t):
+        kw = dict(z=t[6], delta_bias=t[7], delta_softplus=True) if gated else {}
+        y = pkg.selective_scan_fn(*t[:6], **kw)
+        leaves = t[:8] if gated else t[:6]
+        return (y,) + torch.autograd.grad(y, leaves, t[8])
+
+    static = [v.to(dev) for v in values(100)]
+    for t in static[:8]:
+        t.requires_grad_()
+    side = torch.cuda.Stream(device=dev)
+    side.wait_stream(torch.cuda.current_stream(dev))
+    with torch.cuda.stream(side):
+        for _ in range(3):
+            call(static)
+    torch.cuda.current_stream(dev).wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        outs = call(static)
+    for rep in range(3):
+        new = [v.to(dev) for v in values(200 + rep)]
+        with torch.no_grad():
+            for s_, n_ in zip(static, new):
+                s_.copy_(n_)
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [o.clone() for o in outs]
+        for t in new[:8]:
+            t.requires_grad_()
+        want = call(new)                      # eager, between the replays
+        torch.cuda.synchronize()
+        for i, (a, b) in enumerate(zip(got, want)):
+            assert torch.equal(a, b), (rep, i)
