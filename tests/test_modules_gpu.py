@@ -295,3 +295,59 @@ def test_block_with_inner_layernorms_matches_float64_layer(pkg, dev):
             yt, cache = blk.step(x[:, t].to(dev), cache)
             ys.append(yt)
         assert rel_err(torch.stack(ys, 1), yr[:, :12]) <= 1e-4
+
+
+def test_lm_training_step_matches_float64_model_and_learns(pkg, dev):
+    """The whole training path the reference's examples drive (mambapy/lm.py:97-117 forward,
+    cross-entropy on the logits, backward through every layer): loss and the gradient of every
+    parameter against a float64 restatement of the model built from the oracle's scan, then a few
+    AdamW steps on a repeating sequence, which must bring the loss down."""
+    torch.manual_seed(21)
+    cfg = pkg.MambaConfig(d_model=32, n_layers=2, d_state=16)
+    V, Bs, L = 53, 3, 45
+    lm = pkg.LM(cfg, V).to(dev)
+    tok = torch.randint(1, V, (Bs, L + 1))
+    inp, tgt = tok[:, :-1], tok[:, 1:]
+
+    # float64 restatement on CPU copies of the weights
+    p = {k: v.detach().double().cpu().requires_grad_() for k, v in lm.named_parameters()}
+
+    def rms(x, w):
+        return x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + cfg.rms_norm_eps) * w
+
+    x = F.embedding(inp, p["embedding.weight"])
+    for i in range(cfg.n_layers):
+        pre = "mamba.layers.%d." % i
+        h = rms(x, p[pre + "norm.weight"])
+        q = {k[len(pre) + 6:]: v for k, v in p.items() if k.startswith(pre + "mixer.")}
+        xz = F.linear(h, q["in_proj.weight"])
+        xin, z = xz.chunk(2, dim=-1)
+        xc = F.conv1d(xin.transpose(1, 2), q["conv1d.weight"], q["conv1d.bias"], padding=cfg.d_conv - 1,
+                      groups=cfg.d_inner)[:, :, :L].transpose(1, 2)
+        xs = F.silu(xc)
+        dlow, Bm, C = torch.split(F.linear(xs, q["x_proj.weight"]), [cfg.dt_rank, cfg.d_state, cfg.d_state], dim=-1)
+        delta = so.softplus_ref(F.linear(dlow, q["dt_proj.weight"], q["dt_proj.bias"]))
+        y = so.selective_scan_ref(xs, delta, -torch.exp(q["A_log"]), Bm, C, q["D"])
+        x = x + F.linear(y * F.silu(z), q["out_proj.weight"])
+    logits_ref = F.linear(rms(x, p["norm_f.weight"]), p["lm_head.weight"])
+    loss_ref = F.cross_entropy(logits_ref.reshape(-1, V), tgt.reshape(-1))
+    loss_ref.backward()
+
+    logits = lm(inp.to(dev))
+    loss = F.cross_entropy(logits.reshape(-1, V), tgt.to(dev).reshape(-1))
+    loss.backward()
+    assert rel_err(logits, logits_ref) <= 1e-4
+    assert abs(loss.item() - loss_ref.item()) <= 1e-5 * abs(loss_ref.item())
+    for k, v in lm.named_parameters():
+        assert v.grad is not None, k
+        assert rel_err(v.grad, p[k].grad) <= 1e-3, k
+
+    opt = torch.optim.AdamW(lm.parameters(), lr=3e-3)
+    first = loss.item()
+    for _ in range(30):
+        opt.zero_grad()
+        out = lm(inp.to(dev))
+        cur = F.cross_entropy(out.reshape(-1, V), tgt.to(dev).reshape(-1))
+        cur.backward()
+        opt.step()
+    assert torch.isfinite(cur) and cur.item() < 0.8 * first
