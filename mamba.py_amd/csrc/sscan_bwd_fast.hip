@@ -23,7 +23,7 @@
 //     per-tile code is short and has one uniform branch for the ragged edge: a lone wave
 //     issues an instruction only every ~6 clocks and pays tens of clocks per branch, and every
 //     instruction it issues takes a VALU slot away from the scan waves of its SIMD.
-// Tiles in LDS are [64 channels][16 steps] float32 at a pitch of 20 floats.
+// Tiles in LDS are float32 planes of [64 channels][4 steps] (see tile_off).
 // Reductions over channel groups, batch and time go through deterministic partial buffers
 // summed by sscan_bwd_finish_kernel (no floating-point atomics: results are bitwise
 // reproducible).
@@ -33,13 +33,17 @@
 
 namespace mpa {
 
-constexpr int kPitchT = kTile + 4;         // row pitch (floats) of a [channel][step] LDS tile: rows stay
-                                          // 16-byte aligned and 16-byte accesses are conflict-free
-constexpr int kTileF = kWave * kPitchT;   // floats per LDS tile
-
+// A tile of (64 channels x kTile steps) in LDS is kTile/4 planes; plane q holds steps 4q..4q+3 of every
+// channel, the channel index fastest (16 bytes per channel).  A wave that reads or writes one plane with
+// one channel per lane touches 1 KB of consecutive addresses: no bank conflicts and no padding inside the
+// plane (a [channel][step] tile needs a pitch of 20 floats for that).  Planes are 8 floats further apart
+// than their 256 floats, so that threads that walk the planes of a few channels (the step-major item map
+// of the service waves) do not all start in the same bank.
+constexpr int kPlane = kWave * 4 + 8;
+constexpr int kTileF = (kTile / 4) * kPlane;  // floats per LDS tile
 
 // float index of the 16-byte column q (4 steps) of channel ch inside a tile
-__device__ __forceinline__ int tile_off(int ch, int q) { return ch * kPitchT + 4 * q; }
+__device__ __forceinline__ int tile_off(int ch, int q) { return q * kPlane + ch * 4; }
 
 __device__ __forceinline__ float4 tile_ld(const float* tile, int ch, int q) {
     return *reinterpret_cast<const float4*>(tile + tile_off(ch, q));
@@ -125,14 +129,19 @@ __device__ __forceinline__ void static_for(F&& f) {
     }
 }
 
+// dB/dC products of one scan wave and tile, summed over groups of 2*NS lanes by the wave's in-register
+// stages: [kTile steps][64 lanes]; four floats between the waves' blocks, so that service threads that
+// read the same row of different waves start in different banks
+constexpr int kRpW = kTile * kWave + 4;
+
 template <int NS, int NW>
 struct BwdFastLds {
     static constexpr int NP = NS * NW;
     static constexpr size_t kInputs = 3 * 4 + 2;     // delta, x, dy: four buffers each; u: two
-    // + partial sums per scan wave, dB|dC tile sums [2][kTile][2][NP], B|C tiles
+    // + partial sums per scan wave, dB|dC lane-group sums [NW][kRpW], B|C tiles
     // [2][2][NP][kTile], consumption flags
     static constexpr size_t floats =
-        (kInputs + 2 * NW) * kTileF + 2 * kTile * 2 * NP + 2 * 2 * NP * kTile + 4;
+        (kInputs + 2 * NW) * kTileF + NW * kRpW + 2 * 2 * NP * kTile + 4;
 };
 
 // HAS_Z: the forward multiplied its output by silu(z).  The service waves then read z and the
@@ -145,11 +154,12 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
     constexpr int NP = NS * NW;
     constexpr int NQ = kTile / 4;
     static_assert(kSvc == NQ, "one service thread per (channel, 4 steps) item of a tile");
-    // channel reduction of dB/dC: 64 values (2 * NS per step, kBatch steps) per reduce-scatter
-    constexpr int kStepBits = NS == 2 ? 2 : 3;  // stages spent inside one step: log2(2*NS)
-    constexpr int kBatch = 64 / (2 * NS);       // steps per batch
+    // channel reduction of dB/dC: the 2 * NS products of a step are summed over groups of 2 * NS lanes in
+    // registers (reduce-scatter stages inside a row of 16 lanes); kLanesPer lanes of every row then hold
+    // partial sums of one (dB|dC, state) value, and the service waves add those up
     static_assert(NS == 2 || NS == 4, "reduce-scatter layout written for 2 or 4 states per lane");
-    constexpr int kRedF = kTile * 2 * NP;       // floats of one dB|dC tile
+    constexpr int kLanesPer = 16 / (2 * NS);
+    constexpr int kRedF = kTile * 2 * NP;       // dB|dC values of one tile
     constexpr int kBcF = 2 * NP * kTile;        // floats of one B|C tile
 
     extern __shared__ float4 smem4[];
@@ -160,8 +170,8 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
     float* const sU = sDy + 4 * kTileF;           // [2] u = delta*x
     float* const sP1 = sU + 2 * kTileF;           // [NW] sum_n g*B
     float* const sP2 = sP1 + NW * kTileF;         // [NW] sum_n g*a*h[t-1]*A*log2(e)
-    float* const sRed = sP2 + NW * kTileF;        // [2][kTile][2][NP] dB | dC tile sums
-    float* const sBC = sRed + 2 * kRedF;          // [2][B|C][NP][kTile]
+    float* const sRP = sP2 + NW * kTileF;         // [NW][kTile][64] dB | dC lane-group sums
+    float* const sBC = sRP + NW * kRpW;           // [2][B|C][NP][kTile]
     // counts (service wave, tile) pairs whose partial sums have been consumed: kSvc * (k + 1)
     // once every service wave is done with tile k
     int* const sConsumed = reinterpret_cast<int*>(sBC + 2 * kBcF);
@@ -282,7 +292,10 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
         const int fw_i = ((sw >> 1) * kWave + lane) * kFw;  // index inside the [kTile][NP] half
         const int fw_tt = fw_i / NP, fw_n = fw_i % NP;        // walk step, state
         const int fw_tp = rev ? kTile - 1 - fw_tt : fw_tt;    // physical step inside the chunk
-        const int fw_e = (fw_tt * 2 + fw_which) * NP + fw_n;  // index inside the dB|dC tile in LDS
+        // its values in a scan wave's block of lane-group sums: row fw_tt, lanes (of every row of 16)
+        // fw_which * 8 + (state inside the wave) * kLanesPer onwards, kFw * kLanesPer of them
+        static_assert(kFw == 2 && NS % kFw == 0, "a thread forwards two states of one scan wave");
+        const int fw_rp = (fw_n / NS) * kRpW + fw_tt * kWave + fw_which * 8 + (fw_n % NS) * kLanesPer;
         float* const fw_base = (fw_which ? p.partC : p.partB) + cg * p.part_gs + (int64_t)b * p.L * p.Nst;
         const uint32_t fw_off = ((uint32_t)fw_tp * (uint32_t)p.Nst + (uint32_t)fw_n) * 4u;
         const bool fw_vec = p.N == NP && p.Nst % 4 == 0;  // rows of the partial buffers are then aligned for vector stores
@@ -422,6 +435,34 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
         };
         auto reduce_tile = [&](int k) {
             const int pc = phys_of(chunk_of(k));
+            // this thread's share of the tile's dB / dC sums over the 64 channels: the four rows of
+            // lanes, then the lanes of a state's group, always in this order
+            float fw[kFw];
+            {
+                const float* rp = sRP + fw_rp;
+                float4 s0 = *reinterpret_cast<const float4*>(rp), s1 = make_float4(0.f, 0.f, 0.f, 0.f);
+                if constexpr (kLanesPer == 4) s1 = *reinterpret_cast<const float4*>(rp + 4);
+#pragma unroll
+                for (int r = 1; r < 4; ++r) {
+                    const float4 v = *reinterpret_cast<const float4*>(rp + 16 * r);
+                    s0.x += v.x; s0.y += v.y; s0.z += v.z; s0.w += v.w;
+                    if constexpr (kLanesPer == 4) {
+                        const float4 u = *reinterpret_cast<const float4*>(rp + 16 * r + 4);
+                        s1.x += u.x; s1.y += u.y; s1.z += u.z; s1.w += u.w;
+                    }
+                }
+                if constexpr (kLanesPer == 4) {
+                    fw[0] = (s0.x + s0.y) + (s0.z + s0.w);
+                    fw[1] = (s1.x + s1.y) + (s1.z + s1.w);
+                } else {
+                    fw[0] = s0.x + s0.y;
+                    fw[1] = s0.z + s0.w;
+                }
+            }
+            // (summed before the loads below are issued: together the two groups of loads hold more
+            // registers than the wave has)
+            asm volatile("" : "+v"(fw[0]), "+v"(fw[1]));
+            __builtin_amdgcn_sched_barrier(0);
             float4 gB = make_float4(0.f, 0.f, 0.f, 0.f), dd = gB;
 #pragma unroll
             for (int ww = 0; ww < NW; ++ww) {
@@ -437,11 +478,6 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
             const float4 dl4 = tile_ld(sDl + (k & 3) * kTileF, co, qo);
             const float4 x4 = tile_ld(sX + (k & 3) * kTileF, co, qo);
             const float4 dy4 = tile_ld(sDy + (k & 3) * kTileF, co, qo);
-            // this thread's share of the tile's dB / dC sums over the 64 channels
-            const float* red = sRed + (k & 1) * kRedF + fw_e;
-            float fw[kFw];
-#pragma unroll
-            for (int i = 0; i < kFw; ++i) fw[i] = red[i];
             const float gBv[4] = {gB.x, gB.y, gB.z, gB.w}, ddv[4] = {dd.x, dd.y, dd.z, dd.w};
             const float dlv[4] = {dl4.x, dl4.y, dl4.z, dl4.w}, xvv[4] = {x4.x, x4.y, x4.z, x4.w};
             const float dyv[4] = {dy4.x, dy4.y, dy4.z, dy4.w};
@@ -630,6 +666,7 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
 
         // ---- 1. recompute the tile forward, keeping a[t] and h[t] ----
         float aS[kTile][NS], hS[kTile][NS], dyq[2][4];
+        int consumed = 0;
         static_for<0, kTile>([&](auto TT) {
             constexpr int tt = decltype(TT)::value;
 #pragma unroll
@@ -648,6 +685,9 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
                 __builtin_amdgcn_sched_barrier(0);
             }
             if (tt == kTile - 4) {
+                // first look at the consumption counter (see the wait below), early enough to hide the
+                // LDS latency
+                consumed = __hip_atomic_load(sConsumed, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP);
                 // dy of the last four steps, needed when the reverse sweep starts
                 const float4 v = tile_ld(sDy + (k & 3) * kTileF, lane, NQ - 1);
                 dyq[(NQ - 1) & 1][0] = v.x; dyq[(NQ - 1) & 1][1] = v.y;
@@ -656,10 +696,25 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
         });
 
         // ---- 2. reverse sweep ----
+        // The sweep writes this wave's single-buffered LDS blocks: the dB/dC lane-group sums step by
+        // step, the partial sums over the states at its end.  The service waves read those of tile
+        // k-1 at the start of this interval and publish that in sConsumed; by the end of the
+        // recomputation that has normally happened, so this wait falls through.  It is bounded (a
+        // wave never spins forever); if the bound is ever reached the blocks may be overwritten while
+        // they are still being read, so the wave poisons its sums of dA: the call then returns NaN
+        // in dA for these channels instead of silently wrong gradients.
+        if (k >= 1) {
+            int spins = 0;
+            while (consumed < kSvc * k && ++spins < (1 << 20)) {
+                __builtin_amdgcn_s_sleep(1);
+                consumed = __hip_atomic_load(sConsumed, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP);
+            }
+            // (added to the sums at the very end of the kernel)
+            if (consumed < kSvc * k || p.expire_waits) poison = __builtin_nanf("");
+        }
         __builtin_amdgcn_s_setprio(2);
         float gBv[kTile], ddv[kTile];
-        float pend[4];
-        int consumed = 0;
+        float* const rp_lane = sRP + w * kRpW + lane_now();
         static_for<0, kTile>([&](auto RT) {
             constexpr int tt = kTile - 1 - decltype(RT)::value;
             if constexpr ((tt & 3) == 3 && tt >= 4) {
@@ -692,20 +747,16 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
             gBv[tt] = gB;
             ddv[tt] = dd;
 
-            if (tt == 4) {
-                // first look at the consumption counter, early enough to hide the LDS latency
-                consumed = __hip_atomic_load(sConsumed, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP);
-            }
             if (tt == 2) {
                 // fetch delta, u, B, C of the next tile (published two intervals ahead)
                 __builtin_amdgcn_sched_barrier(0);
                 read_fwd_inputs(k + 1, next);
                 __builtin_amdgcn_sched_barrier(0);
             }
-            // ---- channel reduction of this step's dB / dC products (see rs_stage) ----
-            // value index bits, from stage 1 up: dB|dC, the state index, then the step index
-            // inside the batch; steps arrive in descending order, so a step with a set index
-            // bit waits in `pend` for its partner with the bit clear
+            // ---- channel reduction of this step's dB / dC products, first part (see rs_stage) ----
+            // value index bits, from stage 1 up: dB|dC, then the state index.  The lanes of a row then
+            // hold 16 / (2 * NS) partial sums of each of the step's 2 * NS values; they go to this
+            // wave's block of sRP as they are, and the service waves add them up one tile later.
             {
                 float r;
                 if constexpr (NS == 2) {
@@ -715,67 +766,9 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
                     const float a2 = rs_stage<1>(pB[2], pC[2], lane), a3 = rs_stage<1>(pB[3], pC[3], lane);
                     r = rs_stage<3>(rs_stage<2>(a0, a2, lane), rs_stage<2>(a1, a3, lane), lane);
                 }
-                constexpr int sb = tt % kBatch;  // step inside the batch
-                if constexpr ((sb & 1) != 0) {
-                    pend[0] = r;
-                } else {
-                    r = rs_stage<kStepBits + 1>(r, pend[0], lane);
-                    if constexpr ((sb & 2) != 0) {
-                        pend[1] = r;
-                    } else {
-                        r = rs_stage<kStepBits + 2>(r, pend[1], lane);
-                        if constexpr ((sb & 4) != 0) {
-                            pend[2] = r;
-                        } else {
-                            r = rs_stage<kStepBits + 3>(r, pend[2], lane);
-                            bool done = true;
-                            if constexpr (kBatch == 16) {
-                                if constexpr ((sb & 8) != 0) {
-                                    pend[3] = r;
-                                    done = false;
-                                } else {
-                                    r = rs_stage<6>(r, pend[3], lane);
-                                }
-                            }
-                            if (done && sb == 0) {
-                                // lane l holds value number l: decode (step, dB|dC, state)
-                                const int ln = lane_now();
-                                // value index bit j (stage j + 1) sits in lane bit rs_lane_bit(j + 1)
-                                auto vbit = [&](int stage) { return (ln >> rs_lane_bit(stage)) & 1; };
-                                const int which = vbit(1);
-                                const int st = NS == 2 ? vbit(2) : (vbit(2) << 1) | vbit(3);
-                                const int stp = NS == 2 ? vbit(3) | vbit(4) << 1 | vbit(5) << 2 | vbit(6) << 3
-                                                        : vbit(4) | vbit(5) << 1 | vbit(6) << 2;
-                                sRed[(k & 1) * kRedF + ((tt + stp) * 2 + which) * NP + w * NS + st] = r;
-                            }
-                        }
-                    }
-                }
+                rp_lane[tt * kWave] = r;
             }
         });
-        // The partial sums go to single-buffered LDS tiles.  The service waves read tile k-1 at
-        // the start of this interval and publish that in sConsumed; by the end of the sweep
-        // that has normally happened, so this wait falls through.  It is bounded (a wave never
-        // spins forever); if the bound is ever reached the tiles may be overwritten while they
-        // are still being read, so the wave poisons its sums of dA: the call then returns NaN
-        // in dA for these channels instead of silently wrong gradients.
-        // (the sums of the sweep are pinned in front of the wait: left alone, the compiler moves
-        // part of the sweep's arithmetic behind the wait loop and copies the registers it needs)
-#pragma unroll
-        for (int i = 0; i < NS; ++i) asm volatile("" : "+v"(dAacc[i]));
-#pragma unroll
-        for (int tt = 0; tt < kTile; ++tt) asm volatile("" : "+v"(ddv[tt]));
-        if (k >= 1) {
-            int spins = 0;
-            while (consumed < kSvc * k && ++spins < (1 << 20)) {
-                __builtin_amdgcn_s_sleep(1);
-                consumed = __hip_atomic_load(sConsumed, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP);
-            }
-            // (added to the sums at the very end: an assignment here would make every dA
-            // product of the tile dead on this path, and the compiler then moves them behind the
-            // wait together with the registers they need)
-            if (consumed < kSvc * k || p.expire_waits) poison = __builtin_nanf("");
-        }
 #pragma unroll
         for (int q = 0; q < NQ; ++q) {
             tile_st(sP1 + w * kTileF, lane, q, gBv[4 * q], gBv[4 * q + 1], gBv[4 * q + 2], gBv[4 * q + 3]);
