@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the selective-scan hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c1|c0|c3|c4|c4-3000|pscan|thin|block|gated|layer|generate|issue-probe]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c1|c0|c3|c4|c4-3000|pscan|thin|block|gated|layer|generate]
 
 One step = one forward + one backward of the fused selective scan over one batch of
 seeded synthetic input that is already resident in HBM.  Prints ONE JSON line.
@@ -32,31 +32,49 @@ WORKLOADS = {
            "configs[2]: mamba-1.4b layer B=4 L=4096 ED=4096 N=16, bf16 I/O, fp32 state"),
 }
 
+LIBRARY_SHA = None  # mpa_source_hash() of the library that is timed, set in main()
+
+
+def profile_state(workload):
+    """The hardware-counter summary of a workload under profiles/ and whether it describes the
+    kernels that run: the summary carries a line `source_sha = <hash of the kernel sources it was
+    measured on>`, the loaded library reports the hash of the sources it was built from."""
+    import re
+    path = os.path.join(ROOT, "profiles", f"sscan_fwd_bwd_{workload}_pmc.md")
+    try:
+        text = open(path).read()
+    except OSError:
+        return None, {"file": None, "stale": None}
+    m = re.search(r"^\s*source_sha\s*=\s*([0-9a-f]+)", text, flags=re.M)
+    sha = m.group(1) if m else None
+    stale = sha is None or LIBRARY_SHA is None or sha != LIBRARY_SHA
+    return text, {"file": os.path.relpath(path, ROOT), "source_sha": sha, "library_sha": LIBRARY_SHA,
+                  "stale": stale}
+
+
+def _profile_number(workload, pattern):
+    import re
+    text, st = profile_state(workload)
+    if text is None or st["stale"]:
+        return None
+    m = re.search(pattern, text)
+    return float(m.group(1)) if m else None
+
+
 def measured_traffic_bytes(workload):
     """HBM bytes per launch of the backward entry point, measured with rocprofv3 --pmc (FETCH_SIZE
     + WRITE_SIZE, scaled by a copy kernel of known size).  Read from the summary under profiles/
     (a line `traffic_bytes_per_launch <workload> mpa_sscan_bwd = <number>`); None when that
-    workload has no summary."""
-    import re
-    path = os.path.join(ROOT, "profiles", f"sscan_fwd_bwd_{workload}_pmc.md")
-    try:
-        m = re.search(rf"traffic_bytes_per_launch\s+{workload}\s+mpa_sscan_bwd\s*=\s*([0-9.eE+-]+)", open(path).read())
-        return float(m.group(1)) if m else None
-    except OSError:
-        return None
+    workload has no summary or the summary was measured on other kernel sources than the library
+    that is being timed (see profile_state)."""
+    return _profile_number(workload, rf"traffic_bytes_per_launch\s+{workload}\s+mpa_sscan_bwd\s*=\s*([0-9.eE+-]+)")
 
 
 def measured_valu_insts(workload, entry):
     """Wave-level VALU instructions per launch of an entry point's scan kernel (rocprofv3 --pmc
     SQ_INSTS_VALU), read from the same summary (a line `valu_insts_per_launch <workload> <entry>
-    = <number>`); None when there is none."""
-    import re
-    path = os.path.join(ROOT, "profiles", f"sscan_fwd_bwd_{workload}_pmc.md")
-    try:
-        m = re.search(rf"valu_insts_per_launch\s+{workload}\s+{entry}\s*=\s*([0-9.eE+-]+)", open(path).read())
-        return float(m.group(1)) if m else None
-    except OSError:
-        return None
+    = <number>`); None when there is none or it is stale."""
+    return _profile_number(workload, rf"valu_insts_per_launch\s+{workload}\s+{entry}\s*=\s*([0-9.eE+-]+)")
 
 
 # Plain fp32 wave64 instructions per second the chip can issue: 1024 SIMDs x 2.4 GHz / 2 clocks
@@ -691,6 +709,7 @@ def bench_sscan(args, torch, pkg, dev, workload, steps, warmup, prewarm, cpu=Tru
                      "achieved": bwd_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": bwd_gbs / HBM_PEAK_GBS,
                      "traffic": measured_traffic_bytes(workload),
+                     "traffic_source": profile_state(workload)[1],
                      "valu_issue": valu_issue(workload, "mpa_sscan_bwd", bwd_ms)},
         "forward": {"kernel": "mpa_sscan_fwd (sscan_fwd_kernel)",
                     "achieved": fwd_b / (fwd_ms * 1e-3) / 1e9, "unit": "GB/s",
@@ -722,7 +741,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--prewarm", type=int, default=40,
                     help="untimed start-up steps before the W warm-up steps (device clocks, allocator)")
-    ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS) + ["c3", "c4", "c4-3000", "pscan", "layer", "generate", "thin", "block", "gated", "issue-probe"],
+    ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS) + ["c3", "c4", "c4-3000", "pscan", "layer", "generate", "thin", "block", "gated"],
                     help="c2 (default) is the headline workload; c3 = decode step, c4 = LM forward "
                          "(reported with their own metric, same one-line schema)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -736,18 +755,11 @@ def main():
         sys.exit("bench.py: this build runs on ONE GPU (one process, one MI355X); "
                  "--gpus N with N > 1 is not supported.")
 
-    if args.workload == "issue-probe":
-        # VALU issue-rate table of the SIMDs (mamba.py_amd/csrc/issue_probe.hip, built by build.py):
-        # a child process of its own, started before this process touches the GPU
-        import subprocess
-        exe = os.path.join(ROOT, "mamba.py_amd", "csrc", "issue_probe")
-        if not os.path.exists(exe):
-            sys.exit("bench.py: mamba.py_amd/csrc/issue_probe is not built (python mamba.py_amd/build.py)")
-        sys.exit(subprocess.run([exe]).returncode)
-
     import torch
     import __graft_entry__ as entry
     pkg = entry.load_package()
+    global LIBRARY_SHA
+    LIBRARY_SHA = pkg._lib.load().mpa_source_hash().decode()
     if not torch.cuda.is_available():
         sys.exit("bench.py: no GPU visible")
     dev = torch.device("cuda:0")

@@ -10,11 +10,14 @@
  *     enqueued on it and nothing synchronises the device;
  *   - sizes are in elements, strides are ELEMENT strides of the tensor they describe;
  *   - io_dtype selects the storage type of x, delta, B, C, z, y, dy and of their
- *     gradients; A, D, delta_bias, the recurrent state and every accumulation are float32;
+ *     gradients (delta and its gradient may be float32 next to bfloat16 tensors, see
+ *     MPA_DELTA_F32); A, D, delta_bias, the recurrent state and every accumulation are float32;
  *   - the return value is MPA_OK or one of the MPA_ERR_* codes; nothing is thrown.
- * All entry points are reentrant and keep no global state: nothing is read from the
- * environment, every choice the library makes is a function of the arguments (the
- * workspace queries and the calls they size therefore always agree).
+ * All entry points are reentrant: nothing is read from the environment, every choice the
+ * library makes is a function of the arguments (the workspace queries and the calls they size
+ * therefore always agree).  They keep no global state, with two exceptions: a per-device flag
+ * that remembers that a kernel's dynamic-LDS limit has been raised, and mpa_sscan_fwd_noalloc,
+ * which owns a static device array per GPU and the address of it (see there).
  */
 #ifndef MAMBAPY_AMD_H
 #define MAMBAPY_AMD_H
@@ -26,7 +29,7 @@
 extern "C" {
 #endif
 
-#define MPA_VERSION 200 /* major*10000 + minor*100 + patch */
+#define MPA_VERSION 20100 /* major*10000 + minor*100 + patch: 2.1.0 */
 
 enum mpa_status {
     MPA_OK = 0,
@@ -74,8 +77,15 @@ typedef struct mpa_sscan_shape {
     int32_t plan_states_per_lane; /* states of d_state kept by one lane: a power of two */
     int32_t plan_segments;        /* pieces the sequence is cut into (1 = never cut) */
     int32_t plan_flags;           /* bit set of MPA_PLAN_* */
-    int32_t reserved;             /* 0 */
+    int32_t delta_dtype;          /* 0: delta and ddelta have io_dtype; MPA_DELTA_F32: see below */
 } mpa_sscan_shape;
+
+/* mpa_sscan_shape.delta_dtype: delta (read) and ddelta (written) are float32 whatever io_dtype is
+ * (d_* and g_* remain element strides).  This is the call the reference makes under
+ * torch.autocast: softplus leaves delta in float32 while x, B, C are bfloat16
+ * (mambapy/mamba.py:264-265 with :284-287).  Fast kernels only: mpa_sscan_bwd returns
+ * MPA_ERR_BAD_DTYPE where it would need its general kernel. */
+#define MPA_DELTA_F32 1
 
 /* delta = softplus(delta + delta_bias) is applied inside the kernel (mamba.py:264-265);
  * without the flag `delta` is used as given and delta_bias must be NULL. */
@@ -96,6 +106,10 @@ typedef struct mpa_sscan_shape {
 int mpa_version(void);
 /* Host string naming the GPU architecture the kernels were compiled for ("gfx950"). */
 const char* mpa_arch(void);
+/* Host string: hash of the kernel sources this library was built from (16 hex digits, "unknown"
+ * when the build did not say).  Measurements that are kept next to the sources (hardware-counter
+ * summaries) quote it, so that a reader can tell whether they describe the kernels that run. */
+const char* mpa_source_hash(void);
 /* Host string describing a status code. */
 const char* mpa_status_string(int status);
 
@@ -148,6 +162,9 @@ size_t mpa_sscan_fwd_workspace_bytes(const mpa_sscan_shape* s, int with_ckpt);
  * 2 * batch * segments * dim * min(dstate, 64) floats and a little more; a caller that pins 16 or
  * 32 states per lane needs the packed B/C of the whole sequence).  All calls on one GPU share that GPU's array: calls that overlap
  * on one GPU (different streams or threads) race; calls on one stream are ordered.
+ * The first call on a device looks up the array's address and raises the kernels' dynamic-LDS limit
+ * (host calls that do not belong into a stream capture): make one call per device and kernel variant
+ * (same dtype, gate and states per lane) before capturing.
  */
 #define MPA_NOALLOC_SCRATCH_BYTES (16u << 20)
 int mpa_sscan_fwd_noalloc(const mpa_sscan_shape* s, const void* x, const void* delta, const float* A,

@@ -14,13 +14,14 @@ MPA_SSCAN_DELTA_SOFTPLUS = 1
 MPA_SSCAN_REVERSE = 2
 MPA_PLAN_BWD_GENERAL = 1
 MPA_PLAN_EXPIRE_WAITS = 2
+MPA_DELTA_F32 = 1
 MPA_CONV_SILU = 1
 MPA_CKPT_STEPS = 16
 MPA_MAX_DSTATE = 256
 
 MPA_NOALLOC_SCRATCH_BYTES = 16 << 20
 
-EXPORTS = ("mpa_version", "mpa_arch", "mpa_status_string", "mpa_sscan_fwd", "mpa_sscan_fwd_noalloc",
+EXPORTS = ("mpa_version", "mpa_arch", "mpa_source_hash", "mpa_status_string", "mpa_sscan_fwd", "mpa_sscan_fwd_noalloc",
            "mpa_sscan_ckpt_elems", "mpa_sscan_fwd_workspace_bytes", "mpa_sscan_bwd", "mpa_sscan_bwd_workspace_bytes",
            "mpa_pscan_fwd", "mpa_pscan_bwd", "mpa_pscan_workspace_bytes", "mpa_ssm_step",
            "mpa_conv1d_fwd", "mpa_conv1d_bwd", "mpa_conv1d_bwd_workspace_bytes",
@@ -33,7 +34,7 @@ class SscanShape(ctypes.Structure):
                [(n, ctypes.c_int64) for n in (
                    "u_sb", "u_sl", "u_sd", "z_sb", "z_sl", "z_sd", "d_sb", "d_sl", "d_sd", "y_sb", "y_sl", "y_sd",
                    "g_sb", "g_sl", "g_sd", "bc_sb", "bc_sl", "dbc_sb", "dbc_sl")] + \
-               [(n, ctypes.c_int32) for n in ("plan_states_per_lane", "plan_segments", "plan_flags", "reserved")]
+               [(n, ctypes.c_int32) for n in ("plan_states_per_lane", "plan_segments", "plan_flags", "delta_dtype")]
 
 
 class ConvShape(ctypes.Structure):
@@ -69,6 +70,7 @@ def load():
     vp, i64, i32, sz = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int32, ctypes.c_size_t
     lib.mpa_version.restype = ctypes.c_int
     lib.mpa_arch.restype = ctypes.c_char_p
+    lib.mpa_source_hash.restype = ctypes.c_char_p
     lib.mpa_status_string.restype = ctypes.c_char_p
     lib.mpa_status_string.argtypes = [ctypes.c_int]
     sp = ctypes.POINTER(SscanShape)

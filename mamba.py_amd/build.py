@@ -5,6 +5,7 @@
 The library is built in-tree (csrc/libmambapy_amd.so) with hipcc; packed-FP32 code
 generation is switched off for the device pass.
 """
+import hashlib
 import os
 import subprocess
 import sys
@@ -27,9 +28,21 @@ def _hipcc() -> str:
     raise RuntimeError("hipcc not found")
 
 
+def source_hash() -> str:
+    """sha256 over the kernel sources (csrc/*.hip, csrc/*.h and the public header, by name).  The
+    library is built with this string inside (mpa_source_hash()); a profile summary that quotes
+    counters of a kernel names the hash of the sources it was measured on."""
+    h = hashlib.sha256()
+    files = sorted(f for f in os.listdir(CSRC) if f.endswith((".hip", ".h")))
+    for path in [os.path.join(CSRC, f) for f in files] + [os.path.join(_HERE, "..", "include", "mambapy_amd.h")]:
+        h.update(os.path.basename(path).encode() + b"\0")
+        h.update(open(path, "rb").read())
+    return h.hexdigest()[:16]
+
+
 def _compile(src: str) -> str:
     obj = os.path.join(CSRC, os.path.splitext(src)[0] + ".o")
-    cmd = [_hipcc(), *HIPCC_FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
+    cmd = [_hipcc(), *HIPCC_FLAGS, f'-DMPA_SOURCE_SHA="{source_hash()}"', "-c", os.path.join(CSRC, src), "-o", obj]
     res = subprocess.run(cmd, capture_output=True, text=True)
     noise = "is not a recognized feature for this target"
     err = "\n".join(l for l in res.stderr.splitlines() if noise not in l)
@@ -48,13 +61,6 @@ def build(verbose: bool = False) -> str:
     res = subprocess.run(cmd, capture_output=True, text=True)
     if res.returncode != 0:
         raise RuntimeError(f"link failed:\n{res.stderr}")
-    # the issue-rate probe: a program of its own (a measuring tool, not linked into the library)
-    probe = [_hipcc(), "-O3", f"--offload-arch={ARCH}", "-std=c++17", "-Xclang", "-target-feature", "-Xclang",
-             "-packed-fp32-ops", "-Wno-unused-command-line-argument", os.path.join(CSRC, "issue_probe.hip"),
-             "-o", os.path.join(CSRC, "issue_probe")]
-    res = subprocess.run(probe, capture_output=True, text=True)
-    if res.returncode != 0:
-        raise RuntimeError(f"hipcc failed on issue_probe.hip:\n{res.stderr}")
     if verbose:
         print(LIB_PATH)
     return LIB_PATH

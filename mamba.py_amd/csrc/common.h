@@ -95,6 +95,15 @@ __device__ __forceinline__ void st_off(float* base, uint32_t voff, float v, uint
 __device__ __forceinline__ void st_off(bf16_t* base, uint32_t voff, bf16_t v, uint32_t soff = 0) {
     __builtin_amdgcn_raw_buffer_store_b16(__builtin_bit_cast(unsigned short, v), make_rsrc(base), voff, soff, 0);
 }
+// A delta element as loaded (see the service waves): float32 bits, or bfloat16 bits in the low half;
+// `shift` is 16 for the latter, 0 for the former (wave-uniform, one instruction either way).
+__device__ __forceinline__ uint32_t ld_bits32(const void* base, uint32_t voff, uint32_t soff, uint32_t bytes) {
+    return (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(make_rsrc(base, bytes), voff, soff, 0);
+}
+__device__ __forceinline__ uint32_t ld_bits16(const void* base, uint32_t voff, uint32_t soff, uint32_t bytes) {
+    return (uint32_t)(uint16_t)__builtin_amdgcn_raw_buffer_load_b16(make_rsrc(base, bytes), voff, soff, 0);
+}
+__device__ __forceinline__ float bits_to_float(uint32_t bits, uint32_t shift) { return __uint_as_float(bits << shift); }
 typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
 typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
 __device__ __forceinline__ void st_off(float2* base, uint32_t voff, float2 v, uint32_t soff = 0) {

@@ -42,6 +42,7 @@ struct BwdParams {
     // overwriting them and contributes nothing to dD; row0 = its first row in partD / partDb
     int Nst, accumulate, row0;
     int softplus;
+    int delta_f32;  // delta and ddelta are float32 whatever the I/O type (MPA_DELTA_F32)
     int in_tmajor, dy_tmajor, out_tmajor;
     int64_t u_sb, u_sl, u_sd;
     int64_t z_sb, z_sl, z_sd;

@@ -585,8 +585,9 @@ extern "C" int mpa_sscan_bwd(const mpa_sscan_shape* s, const void* x, const void
     if (!softplus && (delta_bias || ddelta_bias)) return MPA_ERR_BAD_SHAPE;
     if (delta_bias && !ddelta_bias) return MPA_ERR_NULL_POINTER;
     const size_t es = dtype_size(s->io_dtype);
-    if (!aligned_to(x, es) || !aligned_to(delta, es) || !aligned_to(B, es) || !aligned_to(C, es) ||
-        !aligned_to(dy, es) || !aligned_to(dx, es) || !aligned_to(ddelta, es) ||
+    const size_t esd = s->delta_dtype == MPA_DELTA_F32 ? 4 : es;
+    if (!aligned_to(x, es) || !aligned_to(delta, esd) || !aligned_to(B, es) || !aligned_to(C, es) ||
+        !aligned_to(dy, es) || !aligned_to(dx, es) || !aligned_to(ddelta, esd) ||
         !aligned_to(dB, es) || !aligned_to(dC, es) || (z && !aligned_to(z, es)) ||
         (dz && !aligned_to(dz, es)) || (y_pregate && !aligned_to(y_pregate, es)) ||
         !aligned_to(workspace, 256))
@@ -609,6 +610,7 @@ extern "C" int mpa_sscan_bwd(const mpa_sscan_shape* s, const void* x, const void
     p.nchunks = (p.L + kTile - 1) / kTile;
     p.Nst = p.N;
     p.softplus = softplus ? 1 : 0;
+    p.delta_f32 = s->delta_dtype == MPA_DELTA_F32 ? 1 : 0;
     p.u_sb = s->u_sb; p.u_sl = s->u_sl; p.u_sd = s->u_sd;
     p.z_sb = s->z_sb; p.z_sl = s->z_sl; p.z_sd = s->z_sd;
     p.d_sb = s->d_sb; p.d_sl = s->d_sl; p.d_sd = s->d_sd;
@@ -629,6 +631,8 @@ extern "C" int mpa_sscan_bwd(const mpa_sscan_shape* s, const void* x, const void
     const int ns = bwd_states_per_lane(s);
     const int nw = np / ns;
     int rows = p.batch, rows_a = p.batch;
+    // (float32 delta next to bfloat16 tensors exists on the fast kernels only)
+    if (!fast && p.delta_f32 && s->io_dtype != MPA_F32) return MPA_ERR_BAD_DTYPE;
     if (fast) {
         const int nseg = ws.seg.nseg > 1 ? ws.seg.nseg : 1;
         const int nblk = (p.N + kFastStates - 1) / kFastStates;
@@ -659,7 +663,7 @@ extern "C" int mpa_sscan_bwd(const mpa_sscan_shape* s, const void* x, const void
                 g.nseg = nseg; g.seg_tiles = ws.seg.seg_tiles;
                 g.batch = p.batch; g.L = p.L; g.ED = p.ED; g.N = q.N; g.nchunks = p.nchunks;
                 g.a_st = p.N; g.h_st = q.N; g.ck_st = q.N;
-                g.softplus = p.softplus; g.reverse = p.reverse ? 0 : 1;
+                g.softplus = p.softplus; g.delta_f32 = p.delta_f32; g.reverse = p.reverse ? 0 : 1;
                 g.u_sb = s->y_sb; g.u_sl = s->y_sl; g.u_sd = s->y_sd;
                 g.z_sb = s->z_sb; g.z_sl = s->z_sl; g.z_sd = s->z_sd;
                 g.d_sb = s->d_sb; g.d_sl = s->d_sl; g.d_sd = s->d_sd;

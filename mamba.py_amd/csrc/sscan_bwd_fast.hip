@@ -231,7 +231,11 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
         // byte offset of the item's lowest physical step (one vector register per tensor); walk
         // step j of the item is jw(j) row strides further, which goes into the scalar offset
         const uint32_t offx = ((uint32_t)(4 * qp) * (uint32_t)p.u_sl + (uint32_t)cic * (uint32_t)p.u_sd) * kES;
-        const uint32_t offd = ((uint32_t)(4 * qp) * (uint32_t)p.d_sl + (uint32_t)cic * (uint32_t)p.d_sd) * kES;
+        // (delta and ddelta may be float32 next to bfloat16 tensors: element size and conversion shift of their own)
+        const bool d_wide = sizeof(IO) == 4 || p.delta_f32;
+        const uint32_t kESd = d_wide ? 4u : 2u;
+        const uint32_t dshift = __builtin_amdgcn_readfirstlane(d_wide ? 0u : 16u);
+        const uint32_t offd = ((uint32_t)(4 * qp) * (uint32_t)p.d_sl + (uint32_t)cic * (uint32_t)p.d_sd) * kESd;
         const uint32_t offy = ((uint32_t)(4 * qp) * (uint32_t)p.y_sl + (uint32_t)cic * (uint32_t)p.y_sd) * kES;
         const uint32_t offzi = ((uint32_t)(4 * qp) * (uint32_t)p.z_sl + (uint32_t)cic * (uint32_t)p.z_sd) * kES;
         const uint32_t offz = ((uint32_t)(4 * qp) * (uint32_t)p.g_sl + (uint32_t)cic * (uint32_t)p.g_sd) * kES;  // dz
@@ -242,14 +246,14 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             sxj[j] = __builtin_amdgcn_readfirstlane(jw(j) * (uint32_t)p.u_sl * kES);
-            sdj[j] = __builtin_amdgcn_readfirstlane(jw(j) * (uint32_t)p.d_sl * kES);
+            sdj[j] = __builtin_amdgcn_readfirstlane(jw(j) * (uint32_t)p.d_sl * kESd);
             syj[j] = __builtin_amdgcn_readfirstlane(jw(j) * (uint32_t)p.y_sl * kES);
             szj[j] = __builtin_amdgcn_readfirstlane(jw(j) * (uint32_t)p.z_sl * kES);
             sgj[j] = __builtin_amdgcn_readfirstlane(jw(j) * (uint32_t)p.g_sl * kES);
         }
         // tensor origins of this (batch row, channel group)
         const IO* const xb = static_cast<const IO*>(p.x) + (b * p.u_sb + (int64_t)d0 * p.u_sd);
-        const IO* const db = static_cast<const IO*>(p.delta) + (b * p.d_sb + (int64_t)d0 * p.d_sd);
+        const char* const db = static_cast<const char*>(p.delta) + (b * p.d_sb + (int64_t)d0 * p.d_sd) * (int64_t)kESd;
         const IO* const yb = static_cast<const IO*>(p.dy) + (b * p.y_sb + (int64_t)d0 * p.y_sd);
         const IO* const zb = static_cast<const IO*>(p.z) + (b * p.z_sb + (int64_t)d0 * p.z_sd);
         const IO* const ypb = static_cast<const IO*>(p.ypre) + (b * p.y_sb + (int64_t)d0 * p.y_sd);
@@ -284,6 +288,9 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
         const uint32_t offg = ((uint32_t)(4 * qpo) * (uint32_t)p.g_sl + (uint32_t)min(co, cmax) * (uint32_t)p.g_sd) * kES;
         IO* const dxg = static_cast<IO*>(p.dx) + (b * p.g_sb + (int64_t)d0 * p.g_sd);
         IO* const ddg = static_cast<IO*>(p.ddelta) + (b * p.g_sb + (int64_t)d0 * p.g_sd);
+        // ddelta as float32 next to bfloat16 tensors: same element offsets, twice the bytes
+        const bool dd_wide = sizeof(IO) == 2 && p.delta_f32;
+        float* const ddgf = static_cast<float*>(p.ddelta) + (b * p.g_sb + (int64_t)d0 * p.g_sd);
         // dB/dC forwarding: kFw consecutive states of one (step, dB|dC) per thread
         constexpr int kFw = kRedF / (kSvc * kWave);
         static_assert(kRedF % (kSvc * kWave) == 0 && NP % kFw == 0 && (kFw == 2 || kFw == 4), "forwarding layout");
@@ -304,14 +311,14 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
 
         // Raw values of three tiles in flight (see the forward kernel: HBM latency under load
         // is longer than one tile interval)
-        struct Raw { IO x[4], d[4], y[4], z[HAS_Z ? 4 : 1], yp[HAS_Z ? 4 : 1], b[kBcPer], c[kBcPer]; };
+        struct Raw { IO x[4], y[4], z[HAS_Z ? 4 : 1], yp[HAS_Z ? 4 : 1], b[kBcPer], c[kBcPer]; uint32_t d[4]; };
         auto load_tile = [&](int kk, Raw& raw) {
             // tiles beyond the last one are clamped to it; steps beyond the sequence end are read
             // as whatever follows inside the tensor (or zero past its end) and masked at staging
             const int k = min(kk, ntiles - 1);
             const int pc = phys_of(chunk_of(k));
             const IO* xk = xb + (int64_t)pc * kTile * p.u_sl;
-            const IO* dk = db + (int64_t)pc * kTile * p.d_sl;
+            const char* dk = db + ((int64_t)pc * kTile * p.d_sl) * kESd;
             const IO* yk = yb + (int64_t)pc * kTile * p.y_sl;
             const IO* zk = zb + (int64_t)pc * kTile * p.z_sl;
             const IO* ypk = ypb + (int64_t)pc * kTile * p.y_sl;
@@ -321,12 +328,12 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
             if (ragged_seq && pc == last_chunk) {
                 // elements from this chunk's origin to one past the tensor's last element
                 const int64_t tb = (int64_t)pc * kTile;
-                auto left = [&](int64_t sb_, int64_t sl_, int64_t sd_, int64_t width) {
+                auto left = [&](int64_t sb_, int64_t sl_, int64_t sd_, int64_t width, int es = (int)sizeof(IO)) {
                     const int64_t end = (p.batch - 1) * sb_ + (p.L - 1) * sl_ + (width - 1) * sd_ + 1;
-                    return window_bytes(end, b * sb_ + tb * sl_ + (int64_t)d0 * sd_, kES);
+                    return window_bytes(end, b * sb_ + tb * sl_ + (int64_t)d0 * sd_, es);
                 };
                 wx = left(p.u_sb, p.u_sl, p.u_sd, p.ED);
-                wd = left(p.d_sb, p.d_sl, p.d_sd, p.ED);
+                wd = left(p.d_sb, p.d_sl, p.d_sd, p.ED, kESd);
                 wy = left(p.y_sb, p.y_sl, p.y_sd, p.ED);
                 wz = left(p.z_sb, p.z_sl, p.z_sd, p.ED);
                 wbc = window_bytes((p.batch - 1) * p.bc_sb + (p.L - 1) * p.bc_sl + p.N, b * p.bc_sb + tb * p.bc_sl, kES);
@@ -334,12 +341,18 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 raw.x[j] = ld_off(xk, offx, sxj[j], wx);
-                raw.d[j] = ld_off(dk, offd, sdj[j], wd);
                 raw.y[j] = ld_off(yk, offy, syj[j], wy);
                 if constexpr (HAS_Z) {
                     raw.z[j] = ld_off(zk, offzi, szj[j], wz);
                     raw.yp[j] = ld_off(ypk, offy, syj[j], wy);
                 }
+            }
+            if (d_wide) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) raw.d[j] = ld_bits32(dk, offd, sdj[j], wd);
+            } else {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) raw.d[j] = ld_bits16(dk, offd, sdj[j], wd);
             }
 #pragma unroll
             for (int r = 0; r < kBcPer; ++r) {
@@ -353,7 +366,7 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 xv[j] = to_float(raw.x[j]);
-                dv[j] = to_float(raw.d[j]);
+                dv[j] = bits_to_float(raw.d[j], dshift);
                 yv[j] = to_float(raw.y[j]);
             }
             if (p.softplus) {
@@ -415,22 +428,30 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
         // ddelta that are there.  They are requested one interval before the tile is reduced, ahead
         // of that interval's input loads: a wave's loads return in order, so a load that is
         // waited for right after its issue would make the wave wait for every tile in flight.
-        struct Acc { IO dx[4], dd[4]; };
+        struct Acc { IO dx[4]; uint32_t dd[4]; };
         Acc acc;
         auto load_acc = [&](int kk) {
             if constexpr (!ACC) return;
             const int pc = phys_of(chunk_of(min(kk, ntiles - 1)));
             const IO* dxk = dxg + (int64_t)pc * kTile * p.g_sl;
             const IO* ddk = ddg + (int64_t)pc * kTile * p.g_sl;
-            uint32_t wg = 0xffffffffu;
+            uint32_t wg = 0xffffffffu, wgd = 0xffffffffu;
             if (ragged_seq && pc == last_chunk) {
                 const int64_t end = (p.batch - 1) * p.g_sb + (p.L - 1) * p.g_sl + (p.ED - 1) * p.g_sd + 1;
                 wg = window_bytes(end, b * p.g_sb + (int64_t)pc * kTile * p.g_sl + (int64_t)d0 * p.g_sd, kES);
+                wgd = window_bytes(end, b * p.g_sb + (int64_t)pc * kTile * p.g_sl + (int64_t)d0 * p.g_sd, kESd);
             }
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                acc.dx[j] = ld_off(dxk, offg, sgj[j], wg);
-                acc.dd[j] = ld_off(ddk, offg, sgj[j], wg);
+            for (int j = 0; j < 4; ++j) acc.dx[j] = ld_off(dxk, offg, sgj[j], wg);
+            if (dd_wide) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc.dd[j] = ld_bits32(ddgf + (int64_t)pc * kTile * p.g_sl, offg * 2u, sgj[j] * 2u, wgd);
+            } else if (sizeof(IO) == 4) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc.dd[j] = ld_bits32(ddk, offg, sgj[j], wgd);
+            } else {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc.dd[j] = ld_bits16(ddk, offg, sgj[j], wgd);
             }
         };
         auto reduce_tile = [&](int k) {
@@ -500,17 +521,22 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
                     dxv[j] += to_float(acc.dx[j]);
-                    dv[j] += to_float(acc.dd[j]);
+                    dv[j] += bits_to_float(acc.dd[j], dshift);
                 }
             }
             IO* dxk = dxg + (int64_t)pc * kTile * p.g_sl;
             IO* ddk = ddg + (int64_t)pc * kTile * p.g_sl;
+            float* ddkf = ddgf + (int64_t)pc * kTile * p.g_sl;
+            auto st_dd = [&](int j, float v) {
+                if (dd_wide) st_off(ddkf, offg * 2u, v, sgj[j] * 2u);
+                else st_off(ddk, offg, from_float<IO>(v), sgj[j]);
+            };
             float* fwk = fw_base + (int64_t)pc * kTile * p.Nst;
             if (group_full && !(ragged_seq && pc == last_chunk) && fw_vec) {
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
                     st_off(dxk, offg, from_float<IO>(dxv[j]), sgj[j]);
-                    st_off(ddk, offg, from_float<IO>(dv[j]), sgj[j]);
+                    st_dd(j, dv[j]);
                 }
                 if constexpr (kFw == 2)
                     st_off(reinterpret_cast<float2*>(fwk), fw_off, make_float2(fw[0], fw[1]));
@@ -521,7 +547,7 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
                 for (int j = 0; j < 4; ++j)
                     if (co_ok && t0 + (int)jw(j) < p.L) {
                         st_off(dxk, offg, from_float<IO>(dxv[j]), sgj[j]);
-                        st_off(ddk, offg, from_float<IO>(dv[j]), sgj[j]);
+                        st_dd(j, dv[j]);
                     }
                 for (int i = 0; i < kFw; ++i)
                     if (pc * kTile + (rev ? kTile - 1 - fw_tt : fw_tt) < p.L && fw_n + i < p.N)
@@ -702,7 +728,8 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
         // recomputation that has normally happened, so this wait falls through.  It is bounded (a
         // wave never spins forever); if the bound is ever reached the blocks may be overwritten while
         // they are still being read, so the wave poisons its sums of dA: the call then returns NaN
-        // in dA for these channels instead of silently wrong gradients.
+        // in dA for these channels (and in one element of dx and ddelta per channel, see the end of the
+        // kernel) instead of silently wrong gradients.
         if (k >= 1) {
             int spins = 0;
             while (consumed < kSvc * k && ++spins < (1 << 20)) {
@@ -796,6 +823,15 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
         }
     }
     __syncthreads();  // final
+    // A caller that drops dA (a frozen A) must still see an expired wait: the wave also overwrites one
+    // element of dx and of ddelta per channel with NaN, in the tile the row ends with (the barrier
+    // above orders these stores after the service waves' stores of that tile).
+    if (poison != poison && dvalid) {
+        const int64_t at = b * p.g_sb + (int64_t)phys_of(chunk_of(ntiles - 1)) * kTile * p.g_sl + (int64_t)d * p.g_sd;
+        static_cast<IO*>(p.dx)[at] = from_float<IO>(poison);
+        if (sizeof(IO) == 2 && p.delta_f32) static_cast<float*>(p.ddelta)[at] = poison;
+        else static_cast<IO*>(p.ddelta)[at] = from_float<IO>(poison);
+    }
 }
 
 template <typename IO, int NS, int NW, bool HAS_Z, bool ACC>

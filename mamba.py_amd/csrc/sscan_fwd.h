@@ -34,6 +34,7 @@ struct FwdParams {
     int a_st, h_st, ck_st;
     const void* yacc;
     int softplus;
+    int delta_f32;   // delta is float32 whatever the I/O type (MPA_DELTA_F32)
     int reverse;     // the walk runs from the last physical step to the first
     int in_tmajor;   // x / delta have unit stride along time
     int out_tmajor;  // y has unit stride along time

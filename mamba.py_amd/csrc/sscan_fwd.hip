@@ -212,13 +212,17 @@ __global__ void __launch_bounds__((kFwdWaves<NW, MODE>) * kWave) sscan_fwd_kerne
             // offsets that do not change from tile to tile: one load per element and no
             // address arithmetic in the loop
             const IO* const xg = static_cast<const IO*>(p.x) + (b * p.u_sb + (int64_t)d0 * p.u_sd);
-            const IO* const dg = static_cast<const IO*>(p.delta) + (b * p.d_sb + (int64_t)d0 * p.d_sd);
+            const char* const dg = static_cast<const char*>(p.delta) + (b * p.d_sb + (int64_t)d0 * p.d_sd) * (int64_t)(sizeof(IO) == 4 || p.delta_f32 ? 4 : 2);
             const IO* const zg = static_cast<const IO*>(p.z) + (b * p.z_sb + (int64_t)d0 * p.z_sd);
             // byte offset of the item's lowest physical step (one vector register per tensor, see
             // ld_off); walk step j of the item is jw(j) row strides further, which goes into the
             // scalar offset of the access
             const uint32_t offx = ((uint32_t)(4 * qp) * (uint32_t)p.u_sl + (uint32_t)cic * (uint32_t)p.u_sd) * kES;
-            const uint32_t offd = ((uint32_t)(4 * qp) * (uint32_t)p.d_sl + (uint32_t)cic * (uint32_t)p.d_sd) * kES;
+            // (delta may be float32 next to bfloat16 tensors: element size and conversion shift of its own)
+            const bool d_wide = sizeof(IO) == 4 || p.delta_f32;
+            const uint32_t kESd = d_wide ? 4u : 2u;
+            const uint32_t dshift = __builtin_amdgcn_readfirstlane(d_wide ? 0u : 16u);
+            const uint32_t offd = ((uint32_t)(4 * qp) * (uint32_t)p.d_sl + (uint32_t)cic * (uint32_t)p.d_sd) * kESd;
             const uint32_t offz = ((uint32_t)(4 * qp) * (uint32_t)p.z_sl + (uint32_t)cic * (uint32_t)p.z_sd) * kES;
             auto jw = [&](int j) { return (uint32_t)(rev ? 3 - j : j); };
             // scalar byte offsets of the item's four walk steps, computed once (scalar registers)
@@ -228,7 +232,7 @@ __global__ void __launch_bounds__((kFwdWaves<NW, MODE>) * kWave) sscan_fwd_kerne
                 // (readfirstlane: told to the compiler as wave-uniform, so that they stay in scalar
                 // registers; an offset it takes for per-lane costs a loop over its values per access)
                 sxj[j] = __builtin_amdgcn_readfirstlane(jw(j) * (uint32_t)p.u_sl * kES);
-                sdj[j] = __builtin_amdgcn_readfirstlane(jw(j) * (uint32_t)p.d_sl * kES);
+                sdj[j] = __builtin_amdgcn_readfirstlane(jw(j) * (uint32_t)p.d_sl * kESd);
                 szj[j] = __builtin_amdgcn_readfirstlane(jw(j) * (uint32_t)p.z_sl * kES);
             }
             // Loads of the ragged chunk run past the sequence end.  That is harmless (the values
@@ -264,14 +268,14 @@ __global__ void __launch_bounds__((kFwdWaves<NW, MODE>) * kWave) sscan_fwd_kerne
                 kBcast ? nullptr
                        : reinterpret_cast<const float4*>(p.bcpack) + (int64_t)b * ntiles * kPackVec + min(item, kPackVec - 1);
             float dsum = 0.0f;  // delta summed over the thread's steps of the row
-            struct Raw { IO x[4], d[4], z[4], b[kBcPer > 0 ? kBcPer : 1], c[kBcPer > 0 ? kBcPer : 1]; float4 warm; };
+            struct Raw { IO x[4], z[4], b[kBcPer > 0 ? kBcPer : 1], c[kBcPer > 0 ? kBcPer : 1]; uint32_t d[4]; float4 warm; };
             auto load_tile = [&](int kk, Raw& raw) {
                 // tiles beyond the last one are clamped to it; the loads are unconditional (a
                 // branch around them would force a wait on their data)
                 const int k = min(kk, ntiles - 1);
                 const int pc = phys_chunk(k);
                 const IO* xk = xg + (int64_t)pc * kTile * p.u_sl;
-                const IO* dk = dg + (int64_t)pc * kTile * p.d_sl;
+                const char* dk = dg + ((int64_t)pc * kTile * p.d_sl) * kESd;
                 const IO* zk = zg + (int64_t)pc * kTile * p.z_sl;
                 const IO* Bk = Bg + (int64_t)pc * kTile * p.bc_sl;
                 const IO* Ck = Cg + (int64_t)pc * kTile * p.bc_sl;
@@ -279,20 +283,26 @@ __global__ void __launch_bounds__((kFwdWaves<NW, MODE>) * kWave) sscan_fwd_kerne
                 if (ragged_seq && pc == last_chunk) {
                     // elements from this chunk's origin to one past the tensor's last element
                     const int64_t tb = (int64_t)pc * kTile;
-                    auto left = [&](int64_t sb_, int64_t sl_, int64_t sd_, int64_t width) {
+                    auto left = [&](int64_t sb_, int64_t sl_, int64_t sd_, int64_t width, int es = (int)sizeof(IO)) {
                         const int64_t end = (p.batch - 1) * sb_ + (p.L - 1) * sl_ + (width - 1) * sd_ + 1;
-                        return window_bytes(end, b * sb_ + tb * sl_ + (int64_t)d0 * sd_, kES);
+                        return window_bytes(end, b * sb_ + tb * sl_ + (int64_t)d0 * sd_, es);
                     };
                     wx = left(p.u_sb, p.u_sl, p.u_sd, p.ED);
-                    wd = left(p.d_sb, p.d_sl, p.d_sd, p.ED);
+                    wd = left(p.d_sb, p.d_sl, p.d_sd, p.ED, kESd);
                     wz = left(p.z_sb, p.z_sl, p.z_sd, p.ED);
                     wbc = window_bytes((p.batch - 1) * p.bc_sb + (p.L - 1) * p.bc_sl + p.N, b * p.bc_sb + tb * p.bc_sl, kES);
                 }
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
                     raw.x[j] = ld_off(xk, offx, sxj[j], wx);
-                    raw.d[j] = ld_off(dk, offd, sdj[j], wd);
                     if (has_z) raw.z[j] = ld_off(zk, offz, szj[j], wz);
+                }
+                if (d_wide) {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) raw.d[j] = ld_bits32(dk, offd, sdj[j], wd);
+                } else {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) raw.d[j] = ld_bits16(dk, offd, sdj[j], wd);
                 }
 #pragma unroll
                 for (int r = 0; r < kBcPer; ++r) {
@@ -316,7 +326,7 @@ __global__ void __launch_bounds__((kFwdWaves<NW, MODE>) * kWave) sscan_fwd_kerne
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
                     xv[j] = to_float(raw.x[j]);
-                    dv[j] = to_float(raw.d[j]);
+                    dv[j] = bits_to_float(raw.d[j], dshift);
                 }
                 if (p.softplus) {
 #pragma unroll
@@ -752,7 +762,8 @@ int validate_shape(const mpa_sscan_shape* s) {
     if (s->dstate > MPA_MAX_DSTATE || s->batch > 65535) return MPA_ERR_BAD_SHAPE;
     if (s->seqlen > (int64_t)1 << 30 || s->dim > (int64_t)1 << 30) return MPA_ERR_BAD_SHAPE;
     if (s->io_dtype != MPA_F32 && s->io_dtype != MPA_BF16) return MPA_ERR_BAD_DTYPE;
-    if (s->plan_states_per_lane < 0 || s->plan_segments < 0 || s->reserved != 0) return MPA_ERR_BAD_SHAPE;
+    if (s->plan_states_per_lane < 0 || s->plan_segments < 0) return MPA_ERR_BAD_SHAPE;
+    if (s->delta_dtype != 0 && s->delta_dtype != MPA_DELTA_F32) return MPA_ERR_BAD_DTYPE;
     const int64_t st[] = {s->z_sb, s->z_sl, s->z_sd, s->u_sb, s->u_sl, s->u_sd, s->d_sb, s->d_sl, s->d_sd, s->y_sb, s->y_sl,
                           s->y_sd, s->g_sb, s->g_sl, s->g_sd, s->bc_sb, s->bc_sl, s->dbc_sb, s->dbc_sl};
     for (int64_t v : st)
@@ -862,7 +873,7 @@ static int sscan_fwd_impl(const mpa_sscan_shape* s, const void* x, const void* d
     const bool softplus = (s->flags & MPA_SSCAN_DELTA_SOFTPLUS) != 0;
     if (!softplus && delta_bias) return MPA_ERR_BAD_SHAPE;
     const size_t es = dtype_size(s->io_dtype);
-    if (!aligned_to(x, es) || !aligned_to(delta, es) || !aligned_to(B, es) || !aligned_to(C, es) ||
+    if (!aligned_to(x, es) || !aligned_to(delta, s->delta_dtype == MPA_DELTA_F32 ? 4 : es) || !aligned_to(B, es) || !aligned_to(C, es) ||
         !aligned_to(y, es) || (z && !aligned_to(z, es)) || (y_pregate && !aligned_to(y_pregate, es)) || !aligned_to(A, 4) || !aligned_to(D, 4) ||
         !aligned_to(workspace, 256))
         return MPA_ERR_MISALIGNED;
@@ -880,6 +891,7 @@ static int sscan_fwd_impl(const mpa_sscan_shape* s, const void* x, const void* d
     p.a_st = p.h_st = p.ck_st = p.N;
     p.nchunks = (p.L + kTile - 1) / kTile;
     p.softplus = softplus ? 1 : 0;
+    p.delta_f32 = s->delta_dtype == MPA_DELTA_F32 ? 1 : 0;
     p.reverse = (s->flags & MPA_SSCAN_REVERSE) ? 1 : 0;
     p.u_sb = s->u_sb; p.u_sl = s->u_sl; p.u_sd = s->u_sd;
     p.z_sb = s->z_sb; p.z_sl = s->z_sl; p.z_sd = s->z_sd;

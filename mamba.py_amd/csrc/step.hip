@@ -188,6 +188,10 @@ extern "C" int mpa_ssm_step(const void* x, const void* delta, const float* A, co
 
 extern "C" int mpa_version(void) { return MPA_VERSION; }
 extern "C" const char* mpa_arch(void) { return "gfx950"; }
+#ifndef MPA_SOURCE_SHA
+#define MPA_SOURCE_SHA "unknown"
+#endif
+extern "C" const char* mpa_source_hash(void) { return MPA_SOURCE_SHA; }
 extern "C" const char* mpa_status_string(int status) {
     switch (status) {
         case MPA_OK: return "ok";

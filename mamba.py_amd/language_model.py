@@ -73,7 +73,10 @@ class LM(nn.Module):
         Where the reference runs the whole sequence through forward again for every token, this
         runs the prompt once and then one state-update step per token."""
         if num_tokens <= 0:
-            return prompt[:, :0]
+            # nothing is appended and the reference's final slice `generated[:, -num_tokens:]` then
+            # returns the prompt (from position -num_tokens on); the module ends in train mode there too
+            self.train()
+            return prompt.clone()[:, -num_tokens:]
         if top_k is not None:
             top_k = min(top_k, self.vocab_size)
         input_device = prompt.device

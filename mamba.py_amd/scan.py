@@ -103,6 +103,8 @@ def plan_override(**kw):
 
 
 def _sscan_shape(x, delta, Bm, y_like, g_like, dbc_like, N, flags, z=None, backward=False):
+    """Shape struct of one call.  delta may be float32 next to bfloat16 tensors (the reference's call
+    under autocast, mambapy/mamba.py:264-265): the library then reads it, and writes ddelta, as float32."""
     s = _lib.SscanShape()
     s.batch, s.seqlen, s.dim = x.shape
     s.dstate = N
@@ -112,6 +114,7 @@ def _sscan_shape(x, delta, Bm, y_like, g_like, dbc_like, N, flags, z=None, backw
     if z is not None:
         s.z_sb, s.z_sl, s.z_sd = z.stride()
     s.d_sb, s.d_sl, s.d_sd = delta.stride()
+    s.delta_dtype = _lib.MPA_DELTA_F32 if (delta.dtype == torch.float32 and x.dtype != torch.float32) else 0
     s.y_sb, s.y_sl, s.y_sd = y_like.stride()
     s.g_sb, s.g_sl, s.g_sd = g_like.stride()
     s.bc_sb, s.bc_sl = Bm.stride(0), Bm.stride(1)
@@ -144,7 +147,13 @@ class SelectiveScanFn(torch.autograd.Function):
         if h0 is not None and h0.requires_grad and need_grad:
             raise RuntimeError("selective_scan_fn: no gradient is computed for h0; pass h0.detach()")
         x_ = x.detach()
-        delta_ = delta.detach().to(dt)
+        # float32 delta next to bfloat16 x, B, C is what the reference passes under autocast (softplus
+        # promotes to float32): it is read as it is, unrounded and without a copy (the general
+        # backward kernel, which only a pinned plan selects, has no such path)
+        if delta.dtype == torch.float32 and dt == torch.bfloat16 and not plan.bwd_general:
+            delta_ = delta.detach()
+        else:
+            delta_ = delta.detach().to(dt)
         B_ = _rows_unit_stride(B.detach().to(dt))
         C_ = _rows_unit_stride(C.detach().to(dt))
         if C_.stride() != B_.stride():
@@ -196,7 +205,7 @@ class SelectiveScanFn(torch.autograd.Function):
         if y_pre is not None and dy.stride() != y_pre.stride():
             dy = dy.contiguous()  # the saved pre-gate output is addressed with dy's strides
         dx = torch.empty((Bsz, L, ED), dtype=dt, device=x.device)
-        ddelta = torch.empty_like(dx)
+        ddelta = torch.empty((Bsz, L, ED), dtype=delta.dtype, device=x.device)   # float32 with a float32 delta
         dz = torch.empty_like(dx) if z is not None else None
         dA = torch.empty((ED, N), dtype=torch.float32, device=x.device)
         dD = torch.empty((ED,), dtype=torch.float32, device=x.device)

@@ -29,7 +29,14 @@ def test_library_exports_every_declared_symbol(pkg):
         assert hasattr(lib, n), f"{n} is declared in the header but not exported"
     assert set(pkg._lib.EXPORTS) == set(_declared_functions())
     assert lib.mpa_arch() == b"gfx950"
-    assert lib.mpa_version() == 200
+    assert lib.mpa_version() == 20100   # major*10000 + minor*100 + patch
+    # the library names the sources it was built from; after a build in this tree that is the tree's hash
+    import importlib.util
+    spec = importlib.util.spec_from_file_location("_mpa_build", os.path.join(ROOT, "mamba.py_amd", "build.py"))
+    b = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(b)
+    assert re.fullmatch(r"[0-9a-f]{16}", lib.mpa_source_hash().decode())
+    assert lib.mpa_source_hash().decode() == b.source_hash(), "csrc/ changed since the library was built"
 
 
 def test_status_codes_without_launch(pkg):

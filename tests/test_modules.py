@@ -52,3 +52,14 @@ def test_block_initial_values(pkg):
 def test_vocab_padding(pkg):
     m = pkg.LM(pkg.MambaConfig(d_model=16, n_layers=1), 50277, pad_vocab_size_multiple=8)
     assert m.lm_head.weight.shape[0] == 50280
+
+
+def test_generate_without_new_tokens_returns_the_prompt(pkg):
+    # mambapy/lm.py:119-155 with num_tokens = 0: the loop does not run and `generated[:, -0:]` is the
+    # whole prompt; a negative count slices the prompt from that position on; the module ends in train mode
+    m = pkg.LM(pkg.MambaConfig(d_model=16, n_layers=1), 11)
+    prompt = torch.tensor([[1, 2, 3, 4, 5]])
+    m.eval()
+    out = m.generate(prompt, 0)
+    assert torch.equal(out, prompt) and out.data_ptr() != prompt.data_ptr() and m.training
+    assert torch.equal(m.generate(prompt, -2), prompt[:, 2:])

@@ -470,3 +470,129 @@ def test_config2_shape_gated_softplus_bf16_channel_slice(pkg, dev):
     assert rel_err(gA.grad[sl], A.grad) <= tol
     assert rel_err(gD.grad[sl], Dd.grad) <= tol
     assert rel_err(gb.grad[sl], bb.grad) <= tol
+
+
+def _gated_reference_from_c_oracle(inp, raw, z, bias):
+    """Gate + softplus + bias around the float64 C oracle by the chain rule: the oracle runs the plain
+    scan on delta = softplus(raw + bias) with the upstream gradient dy * silu(z); dz, d raw and d bias
+    follow element-wise in float64.  Everything a fused call returns, at any size the C oracle handles."""
+    rd, zd, dyd = raw.double(), z.double(), inp["dy"].double()
+    pre = rd + bias.double()
+    delta = so.softplus_ref(pre)
+    sg = torch.sigmoid(zd)
+    silu = zd * sg
+    ref = c_oracle.sscan_fwd_bwd(inp["x"], delta, inp["A"], inp["B"], inp["C"], inp["D"], dyd * silu)
+    y_pre = ref["y"]
+    out = dict(ref)
+    out["y"] = y_pre * silu
+    out["dz"] = dyd * y_pre * (sg * (1 + zd * (1 - sg)))
+    out["ddelta"] = ref["ddelta"] * torch.sigmoid(pre)      # d softplus(v)/dv = sigmoid(v)
+    out["dbias"] = out["ddelta"].sum(dim=(0, 1))
+    return out
+
+
+def test_gated_reference_composition_is_the_autograd_oracle():
+    # pins the helper above (no GPU work): on a small case it equals plain float64 autograd through the
+    # definition with gate and softplus written out
+    inp = so.make_inputs(2, 37, 20, 16, seed=71)
+    g = torch.Generator().manual_seed(72)
+    z = torch.randn(2, 37, 20, generator=g)
+    raw = torch.randn(2, 37, 20, generator=g) * 0.5 - 4.0
+    bias = torch.randn(20, generator=g) * 0.3
+    ref = _gated_reference_from_c_oracle(inp, raw, z, bias)
+    f64 = lambda v: v.double().requires_grad_()
+    x, r, A, Bm, C, D, zz, bb = map(f64, (inp["x"], raw, inp["A"], inp["B"], inp["C"], inp["D"], z, bias))
+    y = so.selective_scan_ref(x, so.softplus_ref(r + bb), A, Bm, C, D) * (zz * torch.sigmoid(zz))
+    y.backward(inp["dy"].double())
+    want = dict(y=y, dx=x.grad, ddelta=r.grad, dA=A.grad, dB=Bm.grad, dC=C.grad, dD=D.grad, dz=zz.grad, dbias=bb.grad)
+    for k, v in want.items():
+        assert rel_err(ref[k], v) <= 1e-6, k      # (the C oracle takes its inputs as float32)
+
+
+def test_config2_full_size_gated_softplus_bf16(pkg, dev):
+    # configs[2] in the fused form a Mamba layer calls (gate, softplus, bias inside the kernels), bf16
+    # I/O, EVERY output at full size against the float64 C oracle: dB and dC are sums over all 4096
+    # channels and a channel slice cannot check them
+    Bs, L, ED, N = 4, 4096, 4096, 16
+    dt = torch.bfloat16
+    inp = so.make_inputs(Bs, L, ED, N, seed=1002, dtype=dt)
+    g = torch.Generator().manual_seed(2002)
+    z = torch.randn(Bs, L, ED, generator=g).to(dt)
+    raw = (torch.randn(Bs, L, ED, generator=g) * 0.5 - 4.0).to(dt)
+    bias = torch.randn(ED, generator=g) * 0.3
+    ref = _gated_reference_from_c_oracle(inp, raw, z, bias)
+    t = lambda v: v.to(dev).requires_grad_()
+    gx, gr, gA, gB, gC, gD, gz, gb = map(t, (inp["x"], raw, inp["A"], inp["B"], inp["C"], inp["D"], z, bias))
+    y = pkg.selective_scan_fn(gx, gr, gA, gB, gC, gD, z=gz, delta_bias=gb, delta_softplus=True)
+    y.backward(inp["dy"].to(dev))
+    got = dict(y=y, dx=gx.grad, ddelta=gr.grad, dA=gA.grad, dB=gB.grad, dC=gC.grad, dD=gD.grad, dz=gz.grad,
+               dbias=gb.grad)
+    for k in ref:
+        e = rel_err(got[k], ref[k])
+        assert e <= TOL[dt], f"gated config2: {k} rel err {e:.3e}"
+
+
+# ---------------------------------------------------------------------------------------------
+# float32 delta next to bfloat16 tensors (the reference's call under torch.autocast)
+# ---------------------------------------------------------------------------------------------
+
+def _mixed_inputs(Bs, L, ED, N, seed):
+    """x, B, C, dy rounded to bfloat16, delta kept in float32: what MambaBlock.selective_scan receives
+    under autocast (softplus output is float32, mambapy/mamba.py:264-265)."""
+    inp = so.make_inputs(Bs, L, ED, N, seed=seed)
+    for k in ("x", "B", "C", "dy"):
+        inp[k] = inp[k].to(torch.bfloat16)
+    return inp
+
+
+@pytest.mark.parametrize("tmajor", [False, True])
+@pytest.mark.parametrize("Bs,L,ED,N", [(2, 300, 192, 16), (1, 77, 100, 16), (2, 64, 70, 40)])
+def test_bf16_tensors_with_float32_delta(pkg, dev, Bs, L, ED, N, tmajor):
+    inp = _mixed_inputs(Bs, L, ED, N, seed=4000 + L)
+    ref = c_oracle.sscan_fwd_bwd(**inp)          # on the UNROUNDED delta
+
+    def lay(v):
+        v = v.to(dev)
+        return (v.transpose(1, 2).contiguous().transpose(1, 2) if tmajor else v).requires_grad_()
+    gx, gd = lay(inp["x"]), lay(inp["delta"])
+    gA, gB, gC, gD = (inp[k].to(dev).requires_grad_() for k in ("A", "B", "C", "D"))
+    y = pkg.selective_scan_fn(gx, gd, gA, gB, gC, gD)
+    y.backward(inp["dy"].to(dev))
+    assert y.dtype == torch.bfloat16 and gd.grad.dtype == torch.float32 and gx.grad.dtype == torch.bfloat16
+    got = dict(y=y, dx=gx.grad, ddelta=gd.grad, dA=gA.grad, dB=gB.grad, dC=gC.grad, dD=gD.grad)
+    for k in ref:
+        # ddelta, dA and dD leave the kernels as float32: the float32 bar applies to them
+        tol = TOL[torch.float32] if k in ("ddelta", "dA", "dD") else TOL[torch.bfloat16]
+        e = rel_err(got[k], ref[k])
+        assert e <= tol, f"{k} rel err {e:.3e} > {tol}"
+    # and the unrounded delta is what was used: with delta rounded to bfloat16 the float32 outputs
+    # are further from this oracle than the bar above
+    rounded = dict(inp, delta=inp["delta"].to(torch.bfloat16))
+    far = run_gpu_fwd_bwd(pkg, rounded, dev)
+    assert rel_err(far["dA"], ref["dA"]) > 10 * rel_err(got["dA"], ref["dA"])
+
+
+def test_float32_delta_gated_reverse_and_cut(pkg, dev):
+    # the same with softplus + bias + gate inside the kernels, the walk reversed and the sequence cut
+    Bs, L, ED, N = 2, 200, 130, 16
+    inp = _mixed_inputs(Bs, L, ED, N, seed=4100)
+    g = torch.Generator().manual_seed(4101)
+    z = torch.randn(Bs, L, ED, generator=g).to(torch.bfloat16)
+    raw = torch.randn(Bs, L, ED, generator=g) * 0.5 - 4.0       # float32
+    bias = torch.randn(ED, generator=g) * 0.3
+    fl = lambda v: v.flip(1)
+    finp = {k: (fl(v) if v.dim() == 3 else v) for k, v in inp.items()}
+    ref = _gated_reference_from_c_oracle(finp, fl(raw), fl(z), bias)
+    ref = {k: (fl(v) if v.dim() == 3 else v) for k, v in ref.items()}
+    t = lambda v: v.to(dev).requires_grad_()
+    gx, gr, gA, gB, gC, gD, gz, gb = map(t, (inp["x"], raw, inp["A"], inp["B"], inp["C"], inp["D"], z, bias))
+    with pkg.plan_override(fwd_segments=3, bwd_segments=3):
+        y = pkg.selective_scan_fn(gx, gr, gA, gB, gC, gD, z=gz, delta_bias=gb, delta_softplus=True, reverse=True)
+        y.backward(inp["dy"].to(dev))
+    assert gr.grad.dtype == torch.float32
+    got = dict(y=y, dx=gx.grad, ddelta=gr.grad, dA=gA.grad, dB=gB.grad, dC=gC.grad, dD=gD.grad, dz=gz.grad,
+               dbias=gb.grad)
+    for k in ref:
+        tol = TOL[torch.float32] if k in ("ddelta", "dA", "dD", "dbias") else TOL[torch.bfloat16]
+        e = rel_err(got[k], ref[k])
+        assert e <= tol, f"{k} rel err {e:.3e} > {tol}"

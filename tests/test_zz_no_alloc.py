@@ -35,9 +35,15 @@ def _call_both(pkg, dev, Bs, L, ED, N, seed, with_ckpt, dtype=torch.float32):
         args = [ctypes.byref(shape)] + [p(t[k]) for k in NAMES] + [None, None, None, p(y), None, p(ck), p(hl)]
         stream = scan._stream(dev)
         if noalloc:
-            before = torch.cuda.memory_allocated(dev)
+            # one call first (the very first one on a device resolves the array's address and may make
+            # the runtime materialise the array); after that a call must leave the DRIVER's count of
+            # free device memory alone: torch's own counters would not see a hipMalloc inside the library
+            assert lib.mpa_sscan_fwd_noalloc(*args, stream) == 0
+            torch.cuda.synchronize()
+            free_before = torch.cuda.mem_get_info(dev)[0]
             rc = lib.mpa_sscan_fwd_noalloc(*args, stream)
-            assert torch.cuda.memory_allocated(dev) == before
+            torch.cuda.synchronize()
+            assert torch.cuda.mem_get_info(dev)[0] == free_before
         else:
             ws = torch.empty(need, dtype=torch.uint8, device=dev)
             rc = lib.mpa_sscan_fwd(*args, p(ws), need, stream)
@@ -64,6 +70,49 @@ def test_noalloc_forward_twice_second_call_smaller(pkg, dev):
     # the training form (checkpoints) and bf16, again larger then smaller
     _call_both(pkg, dev, 2, 2048, 128, 16, seed=8103, with_ckpt=True, dtype=torch.bfloat16)
     _call_both(pkg, dev, 1, 600, 64, 8, seed=8104, with_ckpt=True)
+
+
+def test_noalloc_inside_a_hip_graph(pkg, dev):
+    # The callers the entry point is for include code under HIP graph capture.  Its first call on a
+    # device (address look-up, LDS limit of the kernels) happens outside the capture; the capture then
+    # records kernels only, and every replay, on new input values and with eager work in between, equals
+    # the eager mpa_sscan_fwd bit for bit.
+    L_ = pkg._lib
+    lib = L_.load()
+    scan = pkg.scan
+    Bs, L, ED, N = 1, 2048, 256, 16
+    inp = so.make_inputs(Bs, L, ED, N, seed=8110)
+    t = {k: inp[k].to(dev) for k in NAMES}
+    y = torch.zeros(Bs, L, ED, device=dev)
+    hl = torch.zeros(Bs, ED, N, device=dev)
+    shape = scan._sscan_shape(t["x"], t["delta"], t["B"], y, y, t["B"], N, 0)
+    need = lib.mpa_sscan_fwd_workspace_bytes(ctypes.byref(shape), 0)
+    assert 256 < need <= L_.MPA_NOALLOC_SCRATCH_BYTES
+    p = scan._ptr
+    args = [ctypes.byref(shape)] + [p(t[k]) for k in NAMES] + [None, None, None, p(y), None, None, p(hl)]
+    side = torch.cuda.Stream(device=dev)
+    with torch.cuda.stream(side):
+        assert lib.mpa_sscan_fwd_noalloc(*args, scan._stream(dev)) == 0   # outside the capture
+    side.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        assert lib.mpa_sscan_fwd_noalloc(*args, scan._stream(dev)) == 0
+    ws = torch.empty(need, dtype=torch.uint8, device=dev)
+    for rep in range(3):
+        new = so.make_inputs(Bs, L, ED, N, seed=8111 + rep)
+        for k in ("x", "delta", "B", "C"):
+            t[k].copy_(new[k].to(dev))
+        y.fill_(float("nan"))
+        graph.replay()
+        torch.cuda.synchronize()
+        y_graph, h_graph = y.clone(), hl.clone()
+        y.fill_(float("nan"))
+        assert lib.mpa_sscan_fwd(*args, p(ws), need, scan._stream(dev)) == 0   # eager, between the replays
+        torch.cuda.synchronize()
+        assert torch.isfinite(y_graph).all()
+        assert torch.equal(y_graph, y) and torch.equal(h_graph, hl)
+        ref = c_oracle.sscan_fwd(*[new[k] if k in ("x", "delta", "B", "C") else inp[k] for k in NAMES])
+        assert rel_err(y_graph, ref) <= TOL[torch.float32]
 
 
 def test_noalloc_refuses_what_does_not_fit(pkg, dev):
