@@ -63,6 +63,11 @@ class MambaConfig:
             self.mup_width_mult = self.d_model / self.mup_base_width
 
 
+# x_proj / dt_proj run on zero-padded copies of their weights where that gives the GEMM library better
+# tile shapes (see MambaBlock._padded_projections); False runs them on the parameters as they are
+PAD_PROJECTIONS = True
+
+
 def _frozen_f32(owner, key, p, fn=None):
     """float32 form of a small parameter (optionally fn(parameter)) for the kernels that take
     float32 constants.  Inside autograd the parameter itself is returned and the conversion is
@@ -77,12 +82,13 @@ def _frozen_f32(owner, key, p, fn=None):
     if fn is None and p.dtype == torch.float32:
         return p
     cache = owner.__dict__.setdefault("_f32_cache", {})
-    tag = (p._version, p.data_ptr(), p.device)
+    tag = (p._version, p.data_ptr(), p.device, p.dtype)
     hit = cache.get(key)
     if hit is None or hit[0] != tag:
         with torch.no_grad():
             fresh = p.detach().float() if fn is None else fn(p.detach())
-            if hit is not None and hit[1].shape == fresh.shape and hit[1].device == fresh.device:
+            if hit is not None and hit[1].shape == fresh.shape and hit[1].device == fresh.device \
+                    and hit[1].dtype == fresh.dtype:
                 hit[1].copy_(fresh)
                 fresh = hit[1]
         cache[key] = (tag, fresh)
@@ -180,6 +186,33 @@ class MambaBlock(nn.Module):
     def _dt_bias(self):
         return _frozen_f32(self, "dt_bias", self.dt_proj.bias)
 
+    def _padded_projections(self):
+        """x_proj and dt_proj weights in the shape the GEMM library serves best, or None when the
+        layer's own shapes already are.  The low-rank width R = dt_rank (48 at d_model 768) is the K of
+        dt_proj and R + 2N (80) the N of x_proj; both land on generic tiles.  With R rounded up to a
+        multiple of 64 by zero columns, and the rows of x_proj regrouped as [delta rows | zeros up to
+        the rounded width | B rows | C rows | zeros up to a multiple of 64], the two products cost
+        21 + 26 us instead of 25 + 38 us at (8 x 4096) x 1536 in bfloat16, and the low-rank input of
+        dt_proj is a view of the x_proj output as before.  The parameters keep the reference's shapes
+        (state_dict keys x_proj.weight (R + 2N, ED), dt_proj.weight (ED, R)); the padded forms are
+        derived from them (inside autograd as part of the graph, outside it cached)."""
+        R, N = self.config.dt_rank, self.config.d_state
+        Rp = -(-R // 64) * 64
+        if Rp == R or self.dt_layernorm is not None or not PAD_PROJECTIONS:
+            return None
+        rows = -(-(Rp + 2 * N) // 64) * 64
+
+        def pad_x(w):
+            out = w.new_zeros(rows, w.shape[1])
+            out[:R] = w[:R]
+            out[Rp:Rp + 2 * N] = w[R:]
+            return out
+
+        def pad_dt(w):
+            return F.pad(w, (0, Rp - R))
+        return (_frozen_f32(self, "x_proj_padded", self.x_proj.weight, pad_x),
+                _frozen_f32(self, "dt_proj_padded", self.dt_proj.weight, pad_dt), Rp)
+
     def _conv_wb(self):
         return (_frozen_f32(self, "conv_w", self.conv1d.weight), _frozen_f32(self, "conv_b", self.conv1d.bias))
 
@@ -232,10 +265,18 @@ class MambaBlock(nn.Module):
         (mambapy/mamba.py:236-272); with z the result is already gated, y * silu(z), as on the
         reference's fused path (mamba.py:259-260, 225-227)."""
         A, D = self._A(), self._D()
-        dlow, Bm, C = self._split_projection(self.x_proj(x))
-        # (B, L, ED) with unit stride along ED, the layout of x: the reference forms the transposed
-        # product (mamba.py:247) only because its fused backend wants (B, ED, L)
-        delta = F.linear(dlow, self.dt_proj.weight)
+        padded = self._padded_projections() if x.is_cuda else None
+        if padded is None:
+            dlow, Bm, C = self._split_projection(self.x_proj(x))
+            # (B, L, ED) with unit stride along ED, the layout of x: the reference forms the transposed
+            # product (mamba.py:247) only because its fused backend wants (B, ED, L)
+            delta = F.linear(dlow, self.dt_proj.weight)
+        else:
+            wx, wdt, Rp = padded
+            N = self.config.d_state
+            dbc = F.linear(x, wx)
+            Bm, C = dbc[..., Rp:Rp + N], dbc[..., Rp + N:Rp + 2 * N]
+            delta = F.linear(dbc[..., :Rp], wdt)     # the zero columns meet the zero rows
         if self.config.fused_softplus:
             return selective_scan_fn(x, delta, A, Bm, C, D, z=z, delta_bias=self._dt_bias(),
                                      delta_softplus=True, h0=h0, return_last_state=return_last_state)
