@@ -102,6 +102,10 @@ typedef struct mpa_sscan_shape {
 /* Test hook: the bounded waits inside the kernels behave as if they had run out (see
  * mpa_sscan_bwd); every kernel still runs to its end. */
 #define MPA_PLAN_EXPIRE_WAITS 2
+/* Channels of a batch row that one workgroup owns: 64 always / 48 wherever the kernels have that form
+ * (neither bit: the library picks, see mpa_sscan_fwd). */
+#define MPA_PLAN_GROUP_64 4
+#define MPA_PLAN_GROUP_48 8
 
 int mpa_version(void);
 /* Host string naming the GPU architecture the kernels were compiled for ("gfx950"). */
@@ -135,6 +139,9 @@ const char* mpa_status_string(int status);
  * segments that run side by side (end states of all segments from zero, a carry pass, then the
  * real pass from the true initial states); checkpoints, h_last and y are the same as without the
  * cut up to float32 rounding.
+ * A launch that is not cut has batch * ceil(dim / 64) workgroups; where batch * ceil(dim / 48) still
+ * fit the 256 CUs in one round (and d_state <= 16), workgroups of 48 channels are used instead: more
+ * of the chip works, and every workgroup is faster (its scan waves have two SIMDs to themselves).
  */
 int mpa_sscan_fwd(const mpa_sscan_shape* s, const void* x, const void* delta, const float* A,
                   const void* B, const void* C, const float* D, const void* z,

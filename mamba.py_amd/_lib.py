@@ -14,6 +14,8 @@ MPA_SSCAN_DELTA_SOFTPLUS = 1
 MPA_SSCAN_REVERSE = 2
 MPA_PLAN_BWD_GENERAL = 1
 MPA_PLAN_EXPIRE_WAITS = 2
+MPA_PLAN_GROUP_64 = 4
+MPA_PLAN_GROUP_48 = 8
 MPA_DELTA_F32 = 1
 MPA_CONV_SILU = 1
 MPA_CKPT_STEPS = 16

@@ -773,6 +773,14 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
             }
             gBv[tt] = gB;
             ddv[tt] = dd;
+            if constexpr ((tt & 3) == 0) {
+                // the partial sums of a group of four steps leave as soon as they are complete: written
+                // together at the end of the tile, the stores of all scan waves (16 KB per wave) would
+                // meet in the LDS queue in front of the barrier
+                constexpr int q = tt >> 2;
+                tile_st(sP1 + w * kTileF, lane_now(), q, gBv[4 * q], gBv[4 * q + 1], gBv[4 * q + 2], gBv[4 * q + 3]);
+                tile_st(sP2 + w * kTileF, lane_now(), q, ddv[4 * q], ddv[4 * q + 1], ddv[4 * q + 2], ddv[4 * q + 3]);
+            }
 
             if (tt == 2) {
                 // fetch delta, u, B, C of the next tile (published two intervals ahead)
@@ -796,11 +804,6 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
                 rp_lane[tt * kWave] = r;
             }
         });
-#pragma unroll
-        for (int q = 0; q < NQ; ++q) {
-            tile_st(sP1 + w * kTileF, lane, q, gBv[4 * q], gBv[4 * q + 1], gBv[4 * q + 2], gBv[4 * q + 3]);
-            tile_st(sP2 + w * kTileF, lane, q, ddv[4 * q], ddv[4 * q + 1], ddv[4 * q + 2], ddv[4 * q + 3]);
-        }
         __syncthreads();  // end of interval k: partial sums and dB/dC sums of tile k are visible
     };
 

@@ -33,6 +33,7 @@ struct FwdParams {
     // what `yacc` holds (strides of y) to its output before the gate.
     int a_st, h_st, ck_st;
     const void* yacc;
+    int group48;     // workgroups of 48 channels (six scan waves) instead of 64, see sscan_fwd.hip
     int softplus;
     int delta_f32;   // delta is float32 whatever the I/O type (MPA_DELTA_F32)
     int reverse;     // the walk runs from the last physical step to the first
@@ -63,6 +64,10 @@ struct SegPlan {
     size_t off_hend, off_h0, off_dsum, floats;
 };
 SegPlan seg_plan(const mpa_sscan_shape* s, int ns, int thin);
+// Channels per workgroup of a launch that is not cut: 48 where the kernels have that form (two states
+// per lane, d_state up to 16) and batch * ceil(dim / 48) workgroups still run in one round on the
+// chip's 256 CUs, else 64.  The plan flags pin either.
+int group_channels(const mpa_sscan_shape* s, int ns, int nseg);
 
 // Launch sscan_fwd_kernel in `mode` (FwdMode) for the (ns, nw) decomposition; the carry modes
 // exist for ns <= 8.

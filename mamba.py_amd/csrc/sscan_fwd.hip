@@ -97,54 +97,100 @@ constexpr int kService = kLoaders + kReducers;
 template <int NS>
 constexpr bool kBcastBC = NS <= 8;
 
-template <int NS, int NW>
+// A workgroup owns CH channels of a batch row: 64 (one channel per lane of a scan wave, the wave's
+// lanes all on the same NS states), or 48.  With 48, a row of 16 lanes is the unit: 3 rows of channels
+// times 8 groups of two states are 24 units, four per scan wave, six scan waves; the rows of a wave
+// then work on different state groups (B and C reach an FMA through a broadcast inside the row, so
+// every row can have its own).  Batch * dim/48 workgroups fill the chip for shapes where batch *
+// dim/64 leaves CUs idle (8 x 1536: 256 instead of 192), and the six scan waves occupy two SIMDs
+// alone: the service waves are given wave numbers that land on the other two.
+template <int NS, int NW, int CH>
+constexpr int kStateGroups = CH == 64 ? NW : 16 / NS;  // groups of NS states = partial readouts per channel
+
+template <int NS, int NW, int CH = 64>
 struct FwdLds {
+    static constexpr int NG = kStateGroups<NS, NW, CH>;
     // delta, u double-buffered (written two tiles ahead of use, read one tile ahead); D*x and
     // the gate in four buffers (written two tiles ahead, read one tile behind); readout
-    // partials double-buffered per scan wave; B/C tiles [2][B|C][state][step] double-buffered
-    static constexpr size_t tiles = (size_t)(2 * 2 + 2 * 4 + 2 * NW) * kWave * kCP;
-    static constexpr size_t floats = tiles + (kBcastBC<NS> ? 2 * 2 * NS * NW * kTile : 0);
+    // partials double-buffered per state group; B/C tiles [2][B|C][state][step] double-buffered
+    static constexpr size_t tiles = (size_t)(2 * 2 + 2 * 4 + 2 * NG) * kWave * kCP;
+    static constexpr size_t floats = tiles + (kBcastBC<NS> ? 2 * 2 * NS * NG * kTile : 0);
 };
 
 
 // One scan step / one group of four steps on the broadcast path: B and C of step TT come out of
 // lane TT of the registers vb[i] / vc[i] inside the FMA (fmac_bcast).
+// The decay factors a = 2^(delta * A2) of a group of four steps.  They do not depend on the state, so a
+// scan wave computes them one group ahead of the recurrence: the multiply and the exponential (the
+// longest latencies of a step) then sit off the chain h -> a*h -> +B*u -> next h, and a wave has
+// independent work to issue while that chain waits for its own results.
+template <int NS>
+struct Decay4 {
+    float a[4][NS];
+};
+template <int Q, int NS>
+__device__ __forceinline__ void decay_group(const float (&dl)[kTile], const float (&A2)[NS], Decay4<NS>& out) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int i = 0; i < NS; ++i) out.a[j][i] = fast_exp2(dl[4 * Q + j] * A2[i]);
+}
 template <int TT, int NS, int MODE>
-__device__ __forceinline__ float scan_step_bcast(float dlv, float uuv, const float (&A2)[NS], float (&h)[NS],
+__device__ __forceinline__ float scan_step_bcast(const float (&a)[NS], float uuv, float (&h)[NS],
                                                  const float (&vb)[NS], const float (&vc)[NS]) {
     float sum = 0.0f;
 #pragma unroll
     for (int i = 0; i < NS; ++i) {
-        const float a = fast_exp2(dlv * A2[i]);
         if constexpr (MODE == kGCarry) {
-            h[i] = a * fmac_bcast<TT>(h[i], vb[i], uuv);
+            h[i] = a[i] * fmac_bcast<TT>(h[i], vb[i], uuv);
         } else {
-            h[i] = fmac_bcast<TT>(a * h[i], vb[i], uuv);
+            h[i] = fmac_bcast<TT>(a[i] * h[i], vb[i], uuv);
         }
         if constexpr (MODE == kScan) sum = i == 0 ? mul_bcast<TT>(vc[i], h[i]) : fmac_bcast<TT>(sum, vc[i], h[i]);
     }
     return sum;
 }
 template <int Q, int NS, int MODE>
-__device__ __forceinline__ float4 scan_group_bcast(const float (&dl)[kTile], const float (&uu)[kTile],
-                                                   const float (&A2)[NS], float (&h)[NS],
+__device__ __forceinline__ float4 scan_group_bcast(const Decay4<NS>& dk, const float (&uu)[kTile], float (&h)[NS],
                                                    const float (&vb)[NS], const float (&vc)[NS]) {
     float4 y;
-    y.x = scan_step_bcast<4 * Q + 0, NS, MODE>(dl[4 * Q + 0], uu[4 * Q + 0], A2, h, vb, vc);
-    y.y = scan_step_bcast<4 * Q + 1, NS, MODE>(dl[4 * Q + 1], uu[4 * Q + 1], A2, h, vb, vc);
-    y.z = scan_step_bcast<4 * Q + 2, NS, MODE>(dl[4 * Q + 2], uu[4 * Q + 2], A2, h, vb, vc);
-    y.w = scan_step_bcast<4 * Q + 3, NS, MODE>(dl[4 * Q + 3], uu[4 * Q + 3], A2, h, vb, vc);
+    y.x = scan_step_bcast<4 * Q + 0, NS, MODE>(dk.a[0], uu[4 * Q + 0], h, vb, vc);
+    y.y = scan_step_bcast<4 * Q + 1, NS, MODE>(dk.a[1], uu[4 * Q + 1], h, vb, vc);
+    y.z = scan_step_bcast<4 * Q + 2, NS, MODE>(dk.a[2], uu[4 * Q + 2], h, vb, vc);
+    y.w = scan_step_bcast<4 * Q + 3, NS, MODE>(dk.a[3], uu[4 * Q + 3], h, vb, vc);
     return y;
 }
 
-// waves of a workgroup: the carry modes store no output and run without reducer waves
-template <int NW, int MODE>
-constexpr int kFwdWaves = NW + (MODE == kScan ? kService : kLoaders);
+// waves of a workgroup: the carry modes store no output and run without reducer waves; a 48-channel
+// workgroup has sixteen wave numbers of which four do nothing (see service_role)
+template <int NW, int MODE, int CH = 64>
+constexpr int kFwdWaves = CH == 48 ? 16 : NW + (MODE == kScan ? kService : kLoaders);
 
-template <typename IO, int NS, int NW, bool HAS_Z, int MODE>
-__global__ void __launch_bounds__((kFwdWaves<NW, MODE>) * kWave) sscan_fwd_kernel(const FwdParams p) {
+// Role of wave w >= NW: 0..3 loaders, 4..7 reducers, -1 none.  Waves w and w + 4 of a workgroup share
+// a SIMD.  In a 48-channel workgroup the six scan waves are waves 0..5 (two each on SIMDs 0 and 1, one
+// each on SIMDs 2 and 3); its three loaders and three reducers (192 items of (channel, 4 steps)) take
+// the wave numbers of SIMDs 2 and 3, and the numbers in between end at once.
+template <int NW, int CH>
+__device__ __forceinline__ int service_role(int w) {
+    if constexpr (CH == 64) return w - NW;
+    switch (w) {
+        case 6: return 0;
+        case 7: return 1;
+        case 10: return 2;
+        case 11: return 4;
+        case 14: return 5;
+        case 15: return 6;
+        default: return -1;
+    }
+}
+
+template <typename IO, int NS, int NW, bool HAS_Z, int MODE, int CH = 64>
+__global__ void __launch_bounds__((kFwdWaves<NW, MODE, CH>) * kWave) sscan_fwd_kernel(const FwdParams p) {
     constexpr int NQ = kTile / 4;  // step groups (of 4) per tile
     static_assert(kLoaders == NQ && kReducers == NQ, "a tile has 64 * NQ items of (channel, 4 steps)");
+    static_assert(CH == 64 || (CH == 48 && NS == 2 && NW == 6 && MODE == kScan), "48-channel groups: six scan waves of two states per lane");
+    constexpr int NG = kStateGroups<NS, NW, CH>;
+    constexpr int kSvcThreads = (CH == 64 ? 4 : 3) * kWave;  // loader (and reducer) threads: one per item
 
     extern __shared__ float4 smem4[];
     typedef float CTile[kWave][kCP];  // [channel][step]
@@ -152,9 +198,9 @@ __global__ void __launch_bounds__((kFwdWaves<NW, MODE>) * kWave) sscan_fwd_kerne
     CTile* sU = sDl + 2;                           // [2]
     CTile* sDx = sU + 2;                           // [4] D*x
     CTile* sG = sDx + 4;                           // [4] gate silu(z) (only with z)
-    CTile* sY = sG + 4;                            // [2][NW]
-    float* const sBC = reinterpret_cast<float*>(sY + 2 * NW);  // [2][B|C][NP states][kTile steps]
-    constexpr int NP = NS * NW;
+    CTile* sY = sG + 4;                            // [2][NG]
+    float* const sBC = reinterpret_cast<float*>(sY + 2 * NG);  // [2][B|C][NP states][kTile steps]
+    constexpr int NP = NS * NG;
     constexpr bool kBcast = kBcastBC<NS>;
     static_assert(MODE == kScan || kBcast, "the carry modes exist on the broadcast path only");
 
@@ -177,7 +223,7 @@ __global__ void __launch_bounds__((kFwdWaves<NW, MODE>) * kWave) sscan_fwd_kerne
     const int last_chunk = p.nchunks - 1;
     auto phys_chunk = [&](int k) { return rev ? last_chunk - (tile0 + k) : tile0 + k; };
     const bool ragged_seq = p.nchunks * kTile > p.L;
-    const int d0 = blockIdx.x * kWave;
+    const int d0 = blockIdx.x * CH;
     constexpr bool has_z = HAS_Z;
 
     if (w >= NW) {
@@ -189,20 +235,21 @@ __global__ void __launch_bounds__((kFwdWaves<NW, MODE>) * kWave) sscan_fwd_kerne
         // 6-10 clocks and pays tens of clocks for every branch, so the per-tile code of these
         // waves is kept short (offsets precomputed, one uniform branch for the ragged edge)
         // and spread over four waves per role.
-        const int sw = w - NW;                       // 0..3: loaders   4..7: reducers
+        const int sw = service_role<NW, CH>(w);      // 0..3: loaders   4..7: reducers
+        if (CH != 64 && sw < 0) return;
         // With softplus or the gate the service waves carry long dependent chains of
         // transcendental functions and must still publish their tile before the interval ends:
         // they then go first whenever they are ready (gated forward at the headline shape: 0.258 ms at
         // priority 3, 0.277 at 2, 0.282 at 1; without gate and softplus priority 1 is best)
         if (has_z || p.softplus) __builtin_amdgcn_s_setprio(3);
         else __builtin_amdgcn_s_setprio(1);
-        const int cmax = min(kWave, p.ED - d0) - 1;  // last valid channel of the group
-        const int item = (sw & 3) * kWave + lane;    // 0 .. 255
+        const int cmax = min(CH, p.ED - d0) - 1;     // last valid channel of the group
+        const int item = (sw & 3) * kWave + lane;    // 0 .. 4 * CH - 1
         constexpr uint32_t kES = sizeof(IO);
         if (sw < kLoaders) {
             // ------------------------------- loaders -------------------------------
-            const int ci = p.in_tmajor ? item / NQ : item % kWave;
-            const int qi = p.in_tmajor ? item % NQ : item / kWave;  // walk step group of the item
+            const int ci = p.in_tmajor ? item / NQ : item % CH;
+            const int qi = p.in_tmajor ? item % NQ : item / CH;     // walk step group of the item
             const int qp = rev ? NQ - 1 - qi : qi;                  // its physical step group
             const bool ci_ok = ci <= cmax;
             const int cic = min(ci, cmax);
@@ -239,19 +286,19 @@ __global__ void __launch_bounds__((kFwdWaves<NW, MODE>) * kWave) sscan_fwd_kerne
             // are masked at staging) as long as the address is inside the tensor: the ragged
             // chunk is read through windows that end with the tensor's last element, whatever
             // the strides (out-of-window loads return zero).
-            const bool group_full = cmax == kWave - 1;
-            // B/C of a tile: kTile * NP elements each, kBcPer per loader thread, step fastest
-            constexpr int kBcPer = kBcast ? NP * kTile / (kLoaders * kWave) : 0;
-            static_assert(!kBcast || NP * kTile % (kLoaders * kWave) == 0, "whole elements per thread");
+            const bool group_full = cmax == CH - 1;
+            // B/C of a tile: kTile * NP elements each, kBcPer per loader thread (the last of them only
+            // for some threads when the division leaves a rest), step fastest
+            constexpr int kBcPer = kBcast ? (NP * kTile + kSvcThreads - 1) / kSvcThreads : 0;
             const IO* const Bg = static_cast<const IO*>(p.Bm) + b * p.bc_sb;
             const IO* const Cg = static_cast<const IO*>(p.C) + b * p.bc_sb;
             int bct[kBcPer > 0 ? kBcPer : 1], bcn[kBcPer > 0 ? kBcPer : 1];
             uint32_t offbc[kBcPer > 0 ? kBcPer : 1];
 #pragma unroll
             for (int r = 0; r < kBcPer; ++r) {
-                const int e = item + r * (kLoaders * kWave);
+                const int e = min(item + r * kSvcThreads, NP * kTile - 1);
                 bct[r] = e % kTile;  // walk step
-                bcn[r] = e / kTile;
+                bcn[r] = item + r * kSvcThreads < NP * kTile ? e / kTile : 2 * NP;  // (beyond the tile: never staged)
                 offbc[r] = ((uint32_t)(rev ? kTile - 1 - bct[r] : bct[r]) * (uint32_t)p.bc_sl +
                             (uint32_t)min(bcn[r], p.N - 1)) * kES;
             }
@@ -318,6 +365,7 @@ __global__ void __launch_bounds__((kFwdWaves<NW, MODE>) * kWave) sscan_fwd_kerne
                     // states beyond d_state: B = C = 0 (padded steps need no care: u = 0 there
                     // and their y is never stored)
                     const bool ok = bcn[r] < p.N;
+                    if (NP * kTile % kSvcThreads != 0 && bcn[r] >= NP) continue;
                     float* dst = sBC + (k & 1) * (2 * NP * kTile) + bcn[r] * kTile + bct[r];
                     dst[0] = ok ? to_float(raw.b[r]) : 0.0f;
                     if constexpr (MODE == kScan) dst[NP * kTile] = ok ? to_float(raw.c[r]) : 0.0f;
@@ -404,8 +452,8 @@ __global__ void __launch_bounds__((kFwdWaves<NW, MODE>) * kWave) sscan_fwd_kerne
             if (p.dsum && ci_ok) p.dsum[((int64_t)bs * NQ + qi) * p.ED + d0 + ci] = dsum;
         } else if constexpr (MODE == kScan) {
             // ------------------------------- reducers -------------------------------
-            const int co = p.out_tmajor ? item / NQ : item % kWave;
-            const int qo = p.out_tmajor ? item % NQ : item / kWave;  // walk step group
+            const int co = p.out_tmajor ? item / NQ : item % CH;
+            const int qo = p.out_tmajor ? item % NQ : item / CH;     // walk step group
             const int qpo = rev ? NQ - 1 - qo : qo;                  // physical step group
             const bool co_ok = co <= cmax;
             const int q4 = 4 * qo;
@@ -439,8 +487,8 @@ __global__ void __launch_bounds__((kFwdWaves<NW, MODE>) * kWave) sscan_fwd_kerne
                 IO* ypk = ypg + (int64_t)pc * kTile * p.y_sl;
                 float4 s = *reinterpret_cast<const float4*>(&sDx[k & 3][co][q4]);
 #pragma unroll
-                for (int ww = 0; ww < NW; ++ww) {
-                    const float4 v = *reinterpret_cast<const float4*>(&sY[(k & 1) * NW + ww][co][q4]);
+                for (int ww = 0; ww < NG; ++ww) {
+                    const float4 v = *reinterpret_cast<const float4*>(&sY[(k & 1) * NG + ww][co][q4]);
                     s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
                 }
                 if (p.yacc) {
@@ -480,12 +528,19 @@ __global__ void __launch_bounds__((kFwdWaves<NW, MODE>) * kWave) sscan_fwd_kerne
     }
 
     // ================================= scan waves =================================
-    const int d = d0 + lane;
+    // lane -> (channel inside the group, group of NS states): see FwdLds
+    int ch = lane, sg = w;
+    if constexpr (CH == 48) {
+        const int unit = 4 * w + (lane >> 4);
+        sg = unit / 3;
+        ch = (unit - 3 * sg) * 16 + (lane & 15);
+    }
+    const int d = d0 + ch;
     const bool dvalid = d < p.ED;
     float A2[NS], h[NS];
 #pragma unroll
     for (int i = 0; i < NS; ++i) {
-        const int n = w * NS + i;
+        const int n = sg * NS + i;
         const bool ok = dvalid && n < p.N;
         const int dc = min(d, p.ED - 1), nc = min(n, p.N - 1);
         const float av = p.A[(int64_t)dc * p.a_st + nc];
@@ -502,13 +557,13 @@ __global__ void __launch_bounds__((kFwdWaves<NW, MODE>) * kWave) sscan_fwd_kerne
     auto read_tile = [&](int k, TileRegs& r) {
 #pragma unroll
         for (int q = 0; q < NQ; ++q) {
-            const float4 v = *reinterpret_cast<const float4*>(&sDl[k & 1][lane][4 * q]);
-            const float4 u4 = *reinterpret_cast<const float4*>(&sU[k & 1][lane][4 * q]);
+            const float4 v = *reinterpret_cast<const float4*>(&sDl[k & 1][ch][4 * q]);
+            const float4 u4 = *reinterpret_cast<const float4*>(&sU[k & 1][ch][4 * q]);
             r.dl[4 * q] = v.x; r.dl[4 * q + 1] = v.y; r.dl[4 * q + 2] = v.z; r.dl[4 * q + 3] = v.w;
             r.uu[4 * q] = u4.x; r.uu[4 * q + 1] = u4.y; r.uu[4 * q + 2] = u4.z; r.uu[4 * q + 3] = u4.w;
         }
         if constexpr (kBcast) {
-            const float* bck = sBC + (k & 1) * (2 * NP * kTile) + (w * NS) * kTile + (lane & (kTile - 1));
+            const float* bck = sBC + (k & 1) * (2 * NP * kTile) + (sg * NS) * kTile + (lane & (kTile - 1));
 #pragma unroll
             for (int i = 0; i < NS; ++i) {
                 r.vb[i] = bck[i * kTile];
@@ -522,7 +577,7 @@ __global__ void __launch_bounds__((kFwdWaves<NW, MODE>) * kWave) sscan_fwd_kerne
         if (MODE == kScan && p.ckpt && dvalid && tile0 + k < last_chunk) {
 #pragma unroll
             for (int i = 0; i < NS; ++i) {
-                const int n = w * NS + i;
+                const int n = sg * NS + i;
                 if (n < p.N) p.ckpt[(((int64_t)b * p.nchunks + tile0 + k) * p.ck_st + n) * p.ED + d] = h[i];
             }
         }
@@ -536,34 +591,44 @@ __global__ void __launch_bounds__((kFwdWaves<NW, MODE>) * kWave) sscan_fwd_kerne
     // handling.
     TileRegs ra, rb;
     if constexpr (kBcast) {
+        Decay4<NS> d0q;  // decay factors of the first four steps of the tile that comes next
         auto tile_compute = [&](int k, const TileRegs& cur, TileRegs& next) {
-            CTile& yt = sY[(k & 1) * NW + w];
+            CTile& yt = sY[(k & 1) * NG + sg];
             // The scan waves of a SIMD share its VALU and the hardware prefers the older one, which
             // would run ahead and then wait at the barrier while the younger one works alone (a
             // lone wave cannot keep the SIMD busy).  A wave's priority falls as it advances
             // through the tile, so the wave that is behind goes first.
             __builtin_amdgcn_s_setprio(3);
-            const float4 y0 = scan_group_bcast<0, NS, MODE>(cur.dl, cur.uu, A2, h, cur.vb, cur.vc);
-            if constexpr (MODE == kScan) *reinterpret_cast<float4*>(&yt[lane][0]) = y0;
+            Decay4<NS> d1, d2, d3;
+            decay_group<1, NS>(cur.dl, A2, d1);
+            const float4 y0 = scan_group_bcast<0, NS, MODE>(d0q, cur.uu, h, cur.vb, cur.vc);
+            if constexpr (MODE == kScan) *reinterpret_cast<float4*>(&yt[ch][0]) = y0;
             __builtin_amdgcn_sched_barrier(0);
             read_tile(k + 1, next);
             __builtin_amdgcn_sched_barrier(0);
             __builtin_amdgcn_s_setprio(2);
-            const float4 y1 = scan_group_bcast<1, NS, MODE>(cur.dl, cur.uu, A2, h, cur.vb, cur.vc);
+            decay_group<2, NS>(cur.dl, A2, d2);
+            const float4 y1 = scan_group_bcast<1, NS, MODE>(d1, cur.uu, h, cur.vb, cur.vc);
+            // (every group's readout leaves as soon as it is complete: written together at the end of the
+            // tile, the stores of all scan waves would meet in the LDS queue in front of the barrier)
+            if constexpr (MODE == kScan) *reinterpret_cast<float4*>(&yt[ch][4]) = y1;
+            __builtin_amdgcn_sched_barrier(0);
             __builtin_amdgcn_s_setprio(1);
-            const float4 y2 = scan_group_bcast<2, NS, MODE>(cur.dl, cur.uu, A2, h, cur.vb, cur.vc);
+            decay_group<3, NS>(cur.dl, A2, d3);
+            const float4 y2 = scan_group_bcast<2, NS, MODE>(d2, cur.uu, h, cur.vb, cur.vc);
+            if constexpr (MODE == kScan) *reinterpret_cast<float4*>(&yt[ch][8]) = y2;
+            __builtin_amdgcn_sched_barrier(0);
             __builtin_amdgcn_s_setprio(0);
-            const float4 y3 = scan_group_bcast<3, NS, MODE>(cur.dl, cur.uu, A2, h, cur.vb, cur.vc);
-            if constexpr (MODE == kScan) {
-                *reinterpret_cast<float4*>(&yt[lane][4]) = y1;
-                *reinterpret_cast<float4*>(&yt[lane][8]) = y2;
-                *reinterpret_cast<float4*>(&yt[lane][12]) = y3;
-            }
+            // (the first group of the next tile, whose delta has arrived in `next` by now)
+            decay_group<0, NS>(next.dl, A2, d0q);
+            const float4 y3 = scan_group_bcast<3, NS, MODE>(d3, cur.uu, h, cur.vb, cur.vc);
+            if constexpr (MODE == kScan) *reinterpret_cast<float4*>(&yt[ch][12]) = y3;
             store_ckpt(k);
         };
         __syncthreads();
         read_tile(0, ra);
         __syncthreads();
+        decay_group<0, NS>(ra.dl, A2, d0q);
         for (int k = 0; k < ntiles; k += 2) {
             tile_compute(k, ra, rb);
             __syncthreads();
@@ -637,7 +702,7 @@ __global__ void __launch_bounds__((kFwdWaves<NW, MODE>) * kWave) sscan_fwd_kerne
     if (p.hlast && dvalid) {
 #pragma unroll
         for (int i = 0; i < NS; ++i) {
-            const int n = w * NS + i;
+            const int n = sg * NS + i;
             if (n < p.N) p.hlast[((int64_t)bs * p.ED + d) * p.h_st + n] = h[i];
         }
     }
@@ -705,20 +770,30 @@ SegPlan seg_plan(const mpa_sscan_shape* s, int ns, int thin) {
     return sp;
 }
 
-template <typename IO, int NS, int NW, bool HAS_Z, int MODE>
+int group_channels(const mpa_sscan_shape* s, int ns, int nseg) {
+    if (ns != 2 || s->dstate > 16 || nseg > 1 || (s->plan_flags & MPA_PLAN_GROUP_64)) return 64;
+    if (s->plan_flags & MPA_PLAN_GROUP_48) return 48;
+    return s->batch * ((s->dim + 47) / 48) <= 256 ? 48 : 64;
+}
+
+template <typename IO, int NS, int NW, bool HAS_Z, int MODE, int CH = 64>
 static int launch_fwd(const FwdParams& p, hipStream_t stream) {
-    dim3 grid((p.ED + kWave - 1) / kWave, p.batch * (p.nseg > 1 ? p.nseg : 1));
-    dim3 block(kFwdWaves<NW, MODE> * kWave);
-    constexpr size_t lds = sizeof(float) * FwdLds<NS, NW>::floats;
+    dim3 grid((p.ED + CH - 1) / CH, p.batch * (p.nseg > 1 ? p.nseg : 1));
+    dim3 block(kFwdWaves<NW, MODE, CH> * kWave);
+    constexpr size_t lds = sizeof(float) * FwdLds<NS, NW, CH>::floats;
     static LdsLimitOnce lds_limit;
-    const int attr_rc = lds_limit.ensure(sscan_fwd_kernel<IO, NS, NW, HAS_Z, MODE>, lds);
+    const int attr_rc = lds_limit.ensure(sscan_fwd_kernel<IO, NS, NW, HAS_Z, MODE, CH>, lds);
     if (attr_rc != MPA_OK) return attr_rc;
-    hipLaunchKernelGGL((sscan_fwd_kernel<IO, NS, NW, HAS_Z, MODE>), grid, block, lds, stream, p);
+    hipLaunchKernelGGL((sscan_fwd_kernel<IO, NS, NW, HAS_Z, MODE, CH>), grid, block, lds, stream, p);
     return check_launch();
 }
 
 template <typename IO>
 static int dispatch_fwd(const FwdParams& p, int ns, int nw, int mode, hipStream_t stream) {
+    if (p.group48) {  // (chosen by the host only where this instance exists: see fwd_group_channels)
+        if (ns != 2 || mode != kScan) return MPA_ERR_BAD_SHAPE;
+        return p.z ? launch_fwd<IO, 2, 6, true, kScan, 48>(p, stream) : launch_fwd<IO, 2, 6, false, kScan, 48>(p, stream);
+    }
 #define MPA_CASE(NS_, NW_)                                                        \
     if (ns == NS_ && nw == NW_ && mode == kScan)                                  \
         return p.z ? launch_fwd<IO, NS_, NW_, true, kScan>(p, stream)             \
@@ -904,7 +979,11 @@ static int sscan_fwd_impl(const mpa_sscan_shape* s, const void* x, const void* d
     // launch, or a sequence cut into segments (end states of every segment from zero, carry,
     // then the real pass)
     auto run_states = [&](const FwdParams& q, int ns, int nw, const SegPlan& sp) -> int {
-        if (sp.nseg <= 1) return launch_fwd_any(q, s->io_dtype, ns, nw, kScan, st);
+        if (sp.nseg <= 1) {
+            FwdParams q1 = q;
+            q1.group48 = q.N == s->dstate && group_channels(s, ns, 1) == 48 ? 1 : 0;
+            return launch_fwd_any(q1, s->io_dtype, ns, nw, kScan, st);
+        }
         FwdParams p1 = q;
         p1.nseg = sp.nseg; p1.seg_tiles = sp.seg_tiles;
         p1.z = nullptr; p1.y = nullptr; p1.ypre = nullptr; p1.yacc = nullptr; p1.h0 = nullptr; p1.ckpt = nullptr;

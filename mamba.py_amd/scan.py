@@ -62,9 +62,10 @@ class LaunchPlan:
         MPA_FWD_NSEG / MPA_BWD_NSEG   segments a sequence is cut into (1 = never cut)
         MPA_PSCAN_CHUNKS              pieces the generic scan cuts a sequence into (1 = never cut)
         MPA_BWD_GENERAL=1             general backward kernel even where the fast one applies
+        MPA_GROUP_CHANNELS            64 or 48 channels of a batch row per workgroup
     """
     _FIELDS = ("fwd_states_per_lane", "bwd_states_per_lane", "fwd_segments", "bwd_segments",
-               "bwd_general", "expire_waits", "pscan_chunks")
+               "bwd_general", "expire_waits", "pscan_chunks", "group_channels")
 
     def __init__(self):
         env = lambda k: int(os.environ[k]) if os.environ.get(k, "").strip() else None
@@ -75,12 +76,14 @@ class LaunchPlan:
         self.pscan_chunks = env("MPA_PSCAN_CHUNKS")
         self.bwd_general = os.environ.get("MPA_BWD_GENERAL", "") == "1"
         self.expire_waits = False  # test hook (MPA_PLAN_EXPIRE_WAITS)
+        self.group_channels = env("MPA_GROUP_CHANNELS")  # 64 or 48 channels per workgroup (None: the library picks)
 
     def fill(self, shape, backward):
         shape.plan_states_per_lane = (self.bwd_states_per_lane if backward else self.fwd_states_per_lane) or 0
         shape.plan_segments = (self.bwd_segments if backward else self.fwd_segments) or 0
         shape.plan_flags = (_lib.MPA_PLAN_BWD_GENERAL if self.bwd_general else 0) | \
-                           (_lib.MPA_PLAN_EXPIRE_WAITS if self.expire_waits else 0)
+                           (_lib.MPA_PLAN_EXPIRE_WAITS if self.expire_waits else 0) | \
+                           {None: 0, 64: _lib.MPA_PLAN_GROUP_64, 48: _lib.MPA_PLAN_GROUP_48}[self.group_channels]
 
 
 plan = LaunchPlan()
