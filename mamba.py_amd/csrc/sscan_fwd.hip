@@ -554,12 +554,18 @@ __global__ void __launch_bounds__((kFwdWaves<NW, MODE, CH>) * kWave) sscan_fwd_k
         float dl[kTile], uu[kTile];
         float vb[kBcast ? NS : 1], vc[kBcast ? NS : 1];
     };
-    auto read_tile = [&](int k, TileRegs& r) {
+    // (in two parts, so that a wave can spread its LDS reads over the tile: delta first, then u, B, C)
+    auto read_tile_delta = [&](int k, TileRegs& r) {
 #pragma unroll
         for (int q = 0; q < NQ; ++q) {
             const float4 v = *reinterpret_cast<const float4*>(&sDl[k & 1][ch][4 * q]);
-            const float4 u4 = *reinterpret_cast<const float4*>(&sU[k & 1][ch][4 * q]);
             r.dl[4 * q] = v.x; r.dl[4 * q + 1] = v.y; r.dl[4 * q + 2] = v.z; r.dl[4 * q + 3] = v.w;
+        }
+    };
+    auto read_tile_rest = [&](int k, TileRegs& r) {
+#pragma unroll
+        for (int q = 0; q < NQ; ++q) {
+            const float4 u4 = *reinterpret_cast<const float4*>(&sU[k & 1][ch][4 * q]);
             r.uu[4 * q] = u4.x; r.uu[4 * q + 1] = u4.y; r.uu[4 * q + 2] = u4.z; r.uu[4 * q + 3] = u4.w;
         }
         if constexpr (kBcast) {
@@ -570,6 +576,10 @@ __global__ void __launch_bounds__((kFwdWaves<NW, MODE, CH>) * kWave) sscan_fwd_k
                 if constexpr (MODE == kScan) r.vc[i] = bck[NP * kTile + i * kTile];
             }
         }
+    };
+    auto read_tile = [&](int k, TileRegs& r) {
+        read_tile_delta(k, r);
+        read_tile_rest(k, r);
     };
     // state after walk tile tile0 + k of the batch row (the state after the very last tile is
     // h_last, not a checkpoint)
@@ -604,7 +614,7 @@ __global__ void __launch_bounds__((kFwdWaves<NW, MODE, CH>) * kWave) sscan_fwd_k
             const float4 y0 = scan_group_bcast<0, NS, MODE>(d0q, cur.uu, h, cur.vb, cur.vc);
             if constexpr (MODE == kScan) *reinterpret_cast<float4*>(&yt[ch][0]) = y0;
             __builtin_amdgcn_sched_barrier(0);
-            read_tile(k + 1, next);
+            read_tile_delta(k + 1, next);
             __builtin_amdgcn_sched_barrier(0);
             __builtin_amdgcn_s_setprio(2);
             decay_group<2, NS>(cur.dl, A2, d2);
@@ -612,6 +622,8 @@ __global__ void __launch_bounds__((kFwdWaves<NW, MODE, CH>) * kWave) sscan_fwd_k
             // (every group's readout leaves as soon as it is complete: written together at the end of the
             // tile, the stores of all scan waves would meet in the LDS queue in front of the barrier)
             if constexpr (MODE == kScan) *reinterpret_cast<float4*>(&yt[ch][4]) = y1;
+            __builtin_amdgcn_sched_barrier(0);
+            read_tile_rest(k + 1, next);
             __builtin_amdgcn_sched_barrier(0);
             __builtin_amdgcn_s_setprio(1);
             decay_group<3, NS>(cur.dl, A2, d3);
