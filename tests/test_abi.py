@@ -55,9 +55,11 @@ def test_status_codes_without_launch(pkg):
     assert lib.mpa_sscan_ckpt_elems(ctypes.byref(s)) == 1 * 1 * 16 * 8
     assert lib.mpa_sscan_bwd_workspace_bytes(ctypes.byref(s)) > 0
     assert lib.mpa_sscan_fwd_workspace_bytes(ctypes.byref(s), 0) > 0
-    s.reserved = 1
-    assert lib.mpa_sscan_fwd(ctypes.byref(s), *([None] * 14), 0, None) == 2  # reserved field must be 0
-    s.reserved = 0
+    s.delta_dtype = 7
+    assert lib.mpa_sscan_fwd(ctypes.byref(s), *([None] * 14), 0, None) == 3  # delta_dtype: 0 or MPA_DELTA_F32
+    s.delta_dtype = L.MPA_DELTA_F32
+    assert lib.mpa_sscan_fwd(ctypes.byref(s), *([None] * 14), 0, None) == 1  # accepted: next complaint is the pointers
+    s.delta_dtype = 0
     assert lib.mpa_status_string(6) == b"workspace too small"
     p = L.PscanShape()
     assert lib.mpa_pscan_fwd(ctypes.byref(p), None, None, None, None, 0, None) == 2
