@@ -741,7 +741,9 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
         }
         __builtin_amdgcn_s_setprio(2);
         float gBv[kTile], ddv[kTile];
-        float* const rp_lane = sRP + w * kRpW + lane_now();
+        const int ln = lane_now();
+        float* const rp_lane = sRP + w * kRpW + ln;
+        float* const p_lane = sP1 + w * kTileF + tile_off(ln, 0);  // (sP2 is NW tiles further: a constant offset)
         static_for<0, kTile>([&](auto RT) {
             constexpr int tt = kTile - 1 - decltype(RT)::value;
             if constexpr ((tt & 3) == 3 && tt >= 4) {
@@ -778,8 +780,10 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
                 // together at the end of the tile, the stores of all scan waves (16 KB per wave) would
                 // meet in the LDS queue in front of the barrier
                 constexpr int q = tt >> 2;
-                tile_st(sP1 + w * kTileF, lane_now(), q, gBv[4 * q], gBv[4 * q + 1], gBv[4 * q + 2], gBv[4 * q + 3]);
-                tile_st(sP2 + w * kTileF, lane_now(), q, ddv[4 * q], ddv[4 * q + 1], ddv[4 * q + 2], ddv[4 * q + 3]);
+                *reinterpret_cast<float4*>(p_lane + q * kPlane) =
+                    make_float4(gBv[4 * q], gBv[4 * q + 1], gBv[4 * q + 2], gBv[4 * q + 3]);
+                *reinterpret_cast<float4*>(p_lane + NW * kTileF + q * kPlane) =
+                    make_float4(ddv[4 * q], ddv[4 * q + 1], ddv[4 * q + 2], ddv[4 * q + 3]);
             }
 
             if (tt == 2) {
