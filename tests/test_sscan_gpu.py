@@ -596,3 +596,34 @@ def test_float32_delta_gated_reverse_and_cut(pkg, dev):
         tol = TOL[torch.float32] if k in ("ddelta", "dA", "dD", "dbias") else TOL[torch.bfloat16]
         e = rel_err(got[k], ref[k])
         assert e <= tol, f"{k} rel err {e:.3e} > {tol}"
+
+
+@pytest.mark.parametrize("Bs,L,ED,N,dtype,gated", [
+    (2, 100, 48, 16, torch.float32, False), (1, 33, 47, 16, torch.float32, True), (2, 200, 150, 12, torch.bfloat16, True),
+    (3, 64, 200, 16, torch.bfloat16, False), (1, 17, 1, 3, torch.float32, False),
+])
+def test_forward_group_sizes_agree_bit_for_bit(pkg, dev, Bs, L, ED, N, dtype, gated):
+    # Workgroups of 64 or of 48 channels are two mappings of lanes to (channel, state group) for the same
+    # arithmetic in the same order: outputs, checkpoints (through the backward) and last states are equal
+    # bit for bit, and both match the oracle.
+    inp = so.make_inputs(Bs, L, ED, N, seed=5000 + ED, dtype=dtype)
+    g = torch.Generator().manual_seed(5001)
+    z = torch.randn(Bs, L, ED, generator=g).to(dtype)
+    raw = (torch.randn(Bs, L, ED, generator=g) * 0.5 - 4.0).to(dtype)
+    bias = torch.randn(ED, generator=g) * 0.3
+    h0 = torch.randn(Bs, ED, N, generator=g)
+    outs = []
+    for ch in (64, 48):
+        t = lambda v: v.to(dev).requires_grad_()
+        gx, gd, gA, gB, gC, gD, gz, gb = map(t, (inp["x"], raw if gated else inp["delta"], inp["A"], inp["B"], inp["C"],
+                                               inp["D"], z, bias))
+        kw = dict(z=gz, delta_bias=gb, delta_softplus=True) if gated else {}
+        with pkg.plan_override(group_channels=ch):
+            y, hl = pkg.selective_scan_fn(gx, gd, gA, gB, gC, gD, h0=h0.to(dev), return_last_state=True, **kw)
+            y.backward(inp["dy"].to(dev))
+        outs.append((y.detach(), hl, gx.grad, gd.grad, gA.grad, gB.grad, gC.grad))
+    for a, b in zip(*outs):
+        assert torch.equal(a, b)
+    if not gated:
+        ref, hr = c_oracle.sscan_fwd(*[inp[k] for k in ("x", "delta", "A", "B", "C", "D")], h0=h0, return_last_state=True)
+        assert rel_err(outs[1][0], ref) <= TOL[dtype] and rel_err(outs[1][1], hr) <= TOL[dtype]
