@@ -124,16 +124,33 @@ struct FwdLds {
 // scan wave computes them one group ahead of the recurrence: the multiply and the exponential (the
 // longest latencies of a step) then sit off the chain h -> a*h -> +B*u -> next h, and a wave has
 // independent work to issue while that chain waits for its own results.
+// (With 8 states per lane a wave has eight independent chains and no registers to spare: the factors
+// of a step are then computed when the step needs them.)
+template <int NS>
+constexpr bool kDecayAhead = NS <= 4;
 template <int NS>
 struct Decay4 {
-    float a[4][NS];
+    float a[kDecayAhead<NS> ? 4 : 1][NS];
+    const float* dl;  // without look-ahead: the group's four values of delta, and A2
+    const float* A2;
 };
 template <int Q, int NS>
 __device__ __forceinline__ void decay_group(const float (&dl)[kTile], const float (&A2)[NS], Decay4<NS>& out) {
+    if constexpr (kDecayAhead<NS>) {
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
+        for (int j = 0; j < 4; ++j)
 #pragma unroll
-        for (int i = 0; i < NS; ++i) out.a[j][i] = fast_exp2(dl[4 * Q + j] * A2[i]);
+            for (int i = 0; i < NS; ++i) out.a[j][i] = fast_exp2(dl[4 * Q + j] * A2[i]);
+    } else {
+        out.dl = dl + 4 * Q;
+        out.A2 = A2;
+    }
+}
+// decay factors of step j of the group
+template <int NS>
+__device__ __forceinline__ void decay_step(const Decay4<NS>& dk, int j, float (&a)[NS]) {
+#pragma unroll
+    for (int i = 0; i < NS; ++i) a[i] = kDecayAhead<NS> ? dk.a[kDecayAhead<NS> ? j : 0][i] : fast_exp2(dk.dl[j] * dk.A2[i]);
 }
 template <int TT, int NS, int MODE>
 __device__ __forceinline__ float scan_step_bcast(const float (&a)[NS], float uuv, float (&h)[NS],
@@ -154,10 +171,15 @@ template <int Q, int NS, int MODE>
 __device__ __forceinline__ float4 scan_group_bcast(const Decay4<NS>& dk, const float (&uu)[kTile], float (&h)[NS],
                                                    const float (&vb)[NS], const float (&vc)[NS]) {
     float4 y;
-    y.x = scan_step_bcast<4 * Q + 0, NS, MODE>(dk.a[0], uu[4 * Q + 0], h, vb, vc);
-    y.y = scan_step_bcast<4 * Q + 1, NS, MODE>(dk.a[1], uu[4 * Q + 1], h, vb, vc);
-    y.z = scan_step_bcast<4 * Q + 2, NS, MODE>(dk.a[2], uu[4 * Q + 2], h, vb, vc);
-    y.w = scan_step_bcast<4 * Q + 3, NS, MODE>(dk.a[3], uu[4 * Q + 3], h, vb, vc);
+    float a[NS];
+    decay_step<NS>(dk, 0, a);
+    y.x = scan_step_bcast<4 * Q + 0, NS, MODE>(a, uu[4 * Q + 0], h, vb, vc);
+    decay_step<NS>(dk, 1, a);
+    y.y = scan_step_bcast<4 * Q + 1, NS, MODE>(a, uu[4 * Q + 1], h, vb, vc);
+    decay_step<NS>(dk, 2, a);
+    y.z = scan_step_bcast<4 * Q + 2, NS, MODE>(a, uu[4 * Q + 2], h, vb, vc);
+    decay_step<NS>(dk, 3, a);
+    y.w = scan_step_bcast<4 * Q + 3, NS, MODE>(a, uu[4 * Q + 3], h, vb, vc);
     return y;
 }
 
