@@ -532,6 +532,29 @@ def test_config2_full_size_gated_softplus_bf16(pkg, dev):
         assert e <= TOL[dt], f"gated config2: {k} rel err {e:.3e}"
 
 
+def test_config4_scan_shape_full_size_gated_bf16(pkg, dev):
+    # the scan of one layer of configs[4] (B=8, L=4096, ED=1536, N=16, gate + softplus + bias, bf16):
+    # 192 workgroups of 64 channels would leave a quarter of the chip idle, so the forward runs as 256
+    # workgroups of 48 channels; every output at full size against the float64 C oracle
+    Bs, L, ED, N = 8, 4096, 1536, 16
+    dt = torch.bfloat16
+    inp = so.make_inputs(Bs, L, ED, N, seed=1004, dtype=dt)
+    g = torch.Generator().manual_seed(2004)
+    z = torch.randn(Bs, L, ED, generator=g).to(dt)
+    raw = (torch.randn(Bs, L, ED, generator=g) * 0.5 - 4.0).to(dt)
+    bias = torch.randn(ED, generator=g) * 0.3
+    ref = _gated_reference_from_c_oracle(inp, raw, z, bias)
+    t = lambda v: v.to(dev).requires_grad_()
+    gx, gr, gA, gB, gC, gD, gz, gb = map(t, (inp["x"], raw, inp["A"], inp["B"], inp["C"], inp["D"], z, bias))
+    y = pkg.selective_scan_fn(gx, gr, gA, gB, gC, gD, z=gz, delta_bias=gb, delta_softplus=True)
+    y.backward(inp["dy"].to(dev))
+    got = dict(y=y, dx=gx.grad, ddelta=gr.grad, dA=gA.grad, dB=gB.grad, dC=gC.grad, dD=gD.grad, dz=gz.grad,
+               dbias=gb.grad)
+    for k in ref:
+        e = rel_err(got[k], ref[k])
+        assert e <= TOL[dt], f"gated config4 scan: {k} rel err {e:.3e}"
+
+
 # ---------------------------------------------------------------------------------------------
 # float32 delta next to bfloat16 tensors (the reference's call under torch.autocast)
 # ---------------------------------------------------------------------------------------------
