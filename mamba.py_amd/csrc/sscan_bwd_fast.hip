@@ -216,6 +216,11 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
         else __builtin_amdgcn_s_setprio(MPA_PRIO_SVC);
         constexpr uint32_t kES = sizeof(IO);
         const bool group_full = cmax == kWave - 1;
+        // With a gate the service waves carry two more input streams, set the kernel's register count
+        // and spill; the forms below marked kLean (less work for the vector unit, a few more live
+        // values) made that worse when they were tried there (gated backward 0.75 -> 0.78 .. 0.89 ms),
+        // so a gated kernel keeps the plainer forms.
+        constexpr bool kLean = !HAS_Z;
 
         // ---- input side: item -> (channel, step group), offsets that never change ----
         const int ci = p.in_tmajor ? item / NQ : item % kWave;
@@ -239,18 +244,43 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
         const uint32_t offy = ((uint32_t)(4 * qp) * (uint32_t)p.y_sl + (uint32_t)cic * (uint32_t)p.y_sd) * kES;
         const uint32_t offzi = ((uint32_t)(4 * qp) * (uint32_t)p.z_sl + (uint32_t)cic * (uint32_t)p.z_sd) * kES;
         const uint32_t offz = ((uint32_t)(4 * qp) * (uint32_t)p.g_sl + (uint32_t)cic * (uint32_t)p.g_sd) * kES;  // dz
-        // scalar byte offsets of an item's four walk steps, per tensor, computed once
-        // (readfirstlane: told to the compiler as wave-uniform, so that they stay in scalar
-        // registers; an offset it takes for per-lane costs a loop over its values per access)
-        uint32_t sxj[4], sdj[4], syj[4], szj[4], sgj[4];
+        // Scalar byte offsets of an item's four walk steps: jw(j) row strides.  Only the row stride of
+        // each tensor is kept (one scalar register); the four products are formed by the scalar unit
+        // where they are used.  Computed once and kept, the twenty offsets did not fit the scalar
+        // register file next to the tensor addresses: they were parked in lanes of a vector register
+        // and every access paid a lane read on the vector unit and its wait states.
+        // (readfirstlane: told to the compiler as wave-uniform; an offset it takes for per-lane costs
+        // a loop over its values per access)
+        const uint32_t rowx = __builtin_amdgcn_readfirstlane((uint32_t)p.u_sl * kES);
+        const uint32_t rowd = __builtin_amdgcn_readfirstlane((uint32_t)p.d_sl * kESd);
+        const uint32_t rowy = __builtin_amdgcn_readfirstlane((uint32_t)p.y_sl * kES);
+        const uint32_t rowz = __builtin_amdgcn_readfirstlane((uint32_t)p.z_sl * kES);
+        const uint32_t rowg = __builtin_amdgcn_readfirstlane((uint32_t)p.g_sl * kES);
+        // the four offsets of a tensor, from a copy of the stride that the compiler cannot trace back
+        // (it would otherwise hoist the products out of the tile loop and keep all of them again)
+        // (With a gate the balance is the other way round: the service waves carry two more input
+        // streams, the kernel spills either way, and forming the offsets per tile measured 3 % slower
+        // than keeping them; there they are computed once.)
+        struct Steps { uint32_t at[4]; };
+        Steps keptx, keptd, kepty, keptz, keptg;
+        if constexpr (!kLean) {
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            sxj[j] = __builtin_amdgcn_readfirstlane(jw(j) * (uint32_t)p.u_sl * kES);
-            sdj[j] = __builtin_amdgcn_readfirstlane(jw(j) * (uint32_t)p.d_sl * kESd);
-            syj[j] = __builtin_amdgcn_readfirstlane(jw(j) * (uint32_t)p.y_sl * kES);
-            szj[j] = __builtin_amdgcn_readfirstlane(jw(j) * (uint32_t)p.z_sl * kES);
-            sgj[j] = __builtin_amdgcn_readfirstlane(jw(j) * (uint32_t)p.g_sl * kES);
+            for (int j = 0; j < 4; ++j) {
+                keptx.at[j] = __builtin_amdgcn_readfirstlane(jw(j) * (uint32_t)p.u_sl * kES);
+                keptd.at[j] = __builtin_amdgcn_readfirstlane(jw(j) * (uint32_t)p.d_sl * kESd);
+                kepty.at[j] = __builtin_amdgcn_readfirstlane(jw(j) * (uint32_t)p.y_sl * kES);
+                keptz.at[j] = __builtin_amdgcn_readfirstlane(jw(j) * (uint32_t)p.z_sl * kES);
+                keptg.at[j] = __builtin_amdgcn_readfirstlane(jw(j) * (uint32_t)p.g_sl * kES);
+            }
         }
+        auto steps_of = [&](uint32_t row, const Steps& kept) {
+            if constexpr (!kLean) return kept;
+            asm volatile("" : "+s"(row));
+            Steps r;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) r.at[j] = jw(j) * row;
+            return r;
+        };
         // tensor origins of this (batch row, channel group)
         const IO* const xb = static_cast<const IO*>(p.x) + (b * p.u_sb + (int64_t)d0 * p.u_sd);
         const char* const db = static_cast<const char*>(p.delta) + (b * p.d_sb + (int64_t)d0 * p.d_sd) * (int64_t)kESd;
@@ -338,21 +368,23 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
                 wz = left(p.z_sb, p.z_sl, p.z_sd, p.ED);
                 wbc = window_bytes((p.batch - 1) * p.bc_sb + (p.L - 1) * p.bc_sl + p.N, b * p.bc_sb + tb * p.bc_sl, kES);
             }
+            const Steps sx = steps_of(rowx, keptx), sy = steps_of(rowy, kepty), sd = steps_of(rowd, keptd);
+            const Steps sz = steps_of(rowz, keptz);
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                raw.x[j] = ld_off(xk, offx, sxj[j], wx);
-                raw.y[j] = ld_off(yk, offy, syj[j], wy);
+                raw.x[j] = ld_off(xk, offx, sx.at[j], wx);
+                raw.y[j] = ld_off(yk, offy, sy.at[j], wy);
                 if constexpr (HAS_Z) {
-                    raw.z[j] = ld_off(zk, offzi, szj[j], wz);
-                    raw.yp[j] = ld_off(ypk, offy, syj[j], wy);
+                    raw.z[j] = ld_off(zk, offzi, sz.at[j], wz);
+                    raw.yp[j] = ld_off(ypk, offy, sy.at[j], wy);
                 }
             }
             if (d_wide) {
 #pragma unroll
-                for (int j = 0; j < 4; ++j) raw.d[j] = ld_bits32(dk, offd, sdj[j], wd);
+                for (int j = 0; j < 4; ++j) raw.d[j] = ld_bits32(dk, offd, sd.at[j], wd);
             } else {
 #pragma unroll
-                for (int j = 0; j < 4; ++j) raw.d[j] = ld_bits16(dk, offd, sdj[j], wd);
+                for (int j = 0; j < 4; ++j) raw.d[j] = ld_bits16(dk, offd, sd.at[j], wd);
             }
 #pragma unroll
             for (int r = 0; r < kBcPer; ++r) {
@@ -387,13 +419,14 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
             const bool ragged = !group_full || (ragged_seq && pc == last_chunk);
             if constexpr (HAS_Z && !ACC) {
                 IO* dzk = dzg + (int64_t)pc * kTile * p.g_sl;
+                const Steps sg = steps_of(rowg, keptg);
                 if (!ragged) {
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) st_off(dzk, offz, from_float<IO>(dzv[j]), sgj[j]);
+                    for (int j = 0; j < 4; ++j) st_off(dzk, offz, from_float<IO>(dzv[j]), sg.at[j]);
                 } else {
                     const int t0 = pc * kTile + 4 * qp_now();
                     for (int j = 0; j < 4; ++j)
-                        if (ci_ok && t0 + (int)jw(j) < p.L) st_off(dzk, offz, from_float<IO>(dzv[j]), sgj[j]);
+                        if (ci_ok && t0 + (int)jw(j) < p.L) st_off(dzk, offz, from_float<IO>(dzv[j]), sg.at[j]);
                 }
             }
             if (ragged) {
@@ -441,17 +474,18 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
                 wg = window_bytes(end, b * p.g_sb + (int64_t)pc * kTile * p.g_sl + (int64_t)d0 * p.g_sd, kES);
                 wgd = window_bytes(end, b * p.g_sb + (int64_t)pc * kTile * p.g_sl + (int64_t)d0 * p.g_sd, kESd);
             }
+            const Steps sg = steps_of(rowg, keptg);
 #pragma unroll
-            for (int j = 0; j < 4; ++j) acc.dx[j] = ld_off(dxk, offg, sgj[j], wg);
+            for (int j = 0; j < 4; ++j) acc.dx[j] = ld_off(dxk, offg, sg.at[j], wg);
             if (dd_wide) {
 #pragma unroll
-                for (int j = 0; j < 4; ++j) acc.dd[j] = ld_bits32(ddgf + (int64_t)pc * kTile * p.g_sl, offg * 2u, sgj[j] * 2u, wgd);
+                for (int j = 0; j < 4; ++j) acc.dd[j] = ld_bits32(ddgf + (int64_t)pc * kTile * p.g_sl, offg * 2u, sg.at[j] * 2u, wgd);
             } else if (sizeof(IO) == 4) {
 #pragma unroll
-                for (int j = 0; j < 4; ++j) acc.dd[j] = ld_bits32(ddk, offg, sgj[j], wgd);
+                for (int j = 0; j < 4; ++j) acc.dd[j] = ld_bits32(ddk, offg, sg.at[j], wgd);
             } else {
 #pragma unroll
-                for (int j = 0; j < 4; ++j) acc.dd[j] = ld_bits16(ddk, offg, sgj[j], wgd);
+                for (int j = 0; j < 4; ++j) acc.dd[j] = ld_bits16(ddk, offg, sg.at[j], wgd);
             }
         };
         auto reduce_tile = [&](int k) {
@@ -485,8 +519,12 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
             asm volatile("" : "+v"(fw[0]), "+v"(fw[1]));
             __builtin_amdgcn_sched_barrier(0);
             float4 gB = make_float4(0.f, 0.f, 0.f, 0.f), dd = gB;
+            if constexpr (kLean) {
+                gB = tile_ld(sP1, co, qo);
+                dd = tile_ld(sP2, co, qo);
+            }
 #pragma unroll
-            for (int ww = 0; ww < NW; ++ww) {
+            for (int ww = kLean ? 1 : 0; ww < NW; ++ww) {
                 const float4 a = tile_ld(sP1 + ww * kTileF, co, qo);
                 const float4 e = tile_ld(sP2 + ww * kTileF, co, qo);
                 gB.x += a.x; gB.y += a.y; gB.z += a.z; gB.w += a.w;
@@ -527,16 +565,30 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
             IO* dxk = dxg + (int64_t)pc * kTile * p.g_sl;
             IO* ddk = ddg + (int64_t)pc * kTile * p.g_sl;
             float* ddkf = ddgf + (int64_t)pc * kTile * p.g_sl;
+            const Steps sg = steps_of(rowg, keptg);
             auto st_dd = [&](int j, float v) {
-                if (dd_wide) st_off(ddkf, offg * 2u, v, sgj[j] * 2u);
-                else st_off(ddk, offg, from_float<IO>(v), sgj[j]);
+                if (dd_wide) st_off(ddkf, offg * 2u, v, sg.at[j] * 2u);
+                else st_off(ddk, offg, from_float<IO>(v), sg.at[j]);
             };
             float* fwk = fw_base + (int64_t)pc * kTile * p.Nst;
             if (group_full && !(ragged_seq && pc == last_chunk) && fw_vec) {
+                if constexpr (kLean) {
 #pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    st_off(dxk, offg, from_float<IO>(dxv[j]), sgj[j]);
-                    st_dd(j, dv[j]);
+                    for (int j = 0; j < 4; ++j) st_off(dxk, offg, from_float<IO>(dxv[j]), sg.at[j]);
+                    // (one branch per tile on the width of ddelta, not one per element)
+                    if (dd_wide) {
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) st_off(ddkf, offg * 2u, dv[j], sg.at[j] * 2u);
+                    } else {
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) st_off(ddk, offg, from_float<IO>(dv[j]), sg.at[j]);
+                    }
+                } else {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        st_off(dxk, offg, from_float<IO>(dxv[j]), sg.at[j]);
+                        st_dd(j, dv[j]);
+                    }
                 }
                 if constexpr (kFw == 2)
                     st_off(reinterpret_cast<float2*>(fwk), fw_off, make_float2(fw[0], fw[1]));
@@ -546,7 +598,7 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
                 const int t0 = pc * kTile + 4 * (rev ? NQ - 1 - qo : qo);
                 for (int j = 0; j < 4; ++j)
                     if (co_ok && t0 + (int)jw(j) < p.L) {
-                        st_off(dxk, offg, from_float<IO>(dxv[j]), sgj[j]);
+                        st_off(dxk, offg, from_float<IO>(dxv[j]), sg.at[j]);
                         st_dd(j, dv[j]);
                     }
                 for (int i = 0; i < kFw; ++i)
@@ -637,21 +689,48 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
         ag[i] = ok ? ag_in : 0.0f;
         dAacc[i] = 0.0f;
     }
-    // state at the start of chunk c: checkpoint written after chunk c-1, or h0 / zero
-    // (uniform base + 32-bit lane offset, the offset rebuilt from lane_now() at each use)
+    // state at the start of chunk c: checkpoint written after chunk c-1, or h0 / zero.  A checkpoint is
+    // fetched with one buffer instruction per state: wave-uniform slot address and state row (scalar
+    // registers) + the lane's channel offset, the one per-lane value, kept for the whole kernel (built
+    // from the lane index at every tile, the address cost each scan wave a dozen half-rate instructions
+    // per tile).  With a gate the service waves set the kernel's register count and already spill:
+    // there the scan waves rebuild their per-lane offsets from the lane index where they are used
+    // (lane_now) instead of keeping them.
+    constexpr bool kKeepLaneOffsets = !HAS_Z;
+    const uint32_t ck_voff_kept = (uint32_t)min(d, p.ED - 1) * 4u;
+    auto lane_here = [&]() { return kKeepLaneOffsets ? lane : lane_now(); };
     auto load_state = [&](int k, float (&hs)[NS]) {
         const int c = chunk_of(min(k, ntiles - 1));
-        const uint32_t ck_lane = (uint32_t)min(d0 + lane_now(), p.ED - 1);
-        const float* ck_base = p.ckpt + ((int64_t)b * p.nchunks + max(c - 1, 0)) * p.Nst * p.ED;
-        const float* h0_base = p.h0 ? p.h0 + (int64_t)b * p.ED * p.Nst : ck_base;
-        const bool first = c == 0;
+        if constexpr (!kKeepLaneOffsets) {
+            // branch-free form: chunk 0 reads slot 0 (or h0) and the value is masked below
+            const uint32_t ck_lane = (uint32_t)min(d0 + lane_now(), p.ED - 1);
+            const float* ck_base = p.ckpt + ((int64_t)b * p.nchunks + max(c - 1, 0)) * p.Nst * p.ED;
+            const float* h0_base = p.h0 ? p.h0 + (int64_t)b * p.ED * p.Nst : ck_base;
+            const bool first = c == 0;
 #pragma unroll
-        for (int i = 0; i < NS; ++i) {
-            const uint32_t n = (uint32_t)min(w * NS + i, p.N - 1);
-            // branch-free: chunk 0 reads slot 0 (or h0) and the value is masked below
-            const uint32_t off = first && p.h0 ? ck_lane * (uint32_t)p.Nst + n : n * (uint32_t)p.ED + ck_lane;
-            const float v = (first ? h0_base : ck_base)[off];
-            hs[i] = (!first || p.h0) ? v : 0.0f;
+            for (int i = 0; i < NS; ++i) {
+                const uint32_t n = (uint32_t)min(w * NS + i, p.N - 1);
+                const uint32_t off = first && p.h0 ? ck_lane * (uint32_t)p.Nst + n : n * (uint32_t)p.ED + ck_lane;
+                const float v = (first ? h0_base : ck_base)[off];
+                hs[i] = (!first || p.h0) ? v : 0.0f;
+            }
+            return;
+        }
+        const uint32_t ck_voff = ck_voff_kept;
+        if (c > 0) {
+            const float* ck_base = p.ckpt + ((int64_t)b * p.nchunks + (c - 1)) * p.Nst * p.ED;
+#pragma unroll
+            for (int i = 0; i < NS; ++i) {
+                const uint32_t n = (uint32_t)min(w * NS + i, p.N - 1);
+                hs[i] = ld_off(ck_base, ck_voff, __builtin_amdgcn_readfirstlane(n * (uint32_t)p.ED * 4u));
+            }
+        } else {
+            // the row starts here: its initial state, or zero
+#pragma unroll
+            for (int i = 0; i < NS; ++i) {
+                const int n = min(w * NS + i, p.N - 1);
+                hs[i] = p.h0 ? p.h0[((int64_t)b * p.ED + min(d, p.ED - 1)) * p.Nst + n] : 0.0f;
+            }
         }
     };
 
@@ -668,7 +747,7 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
             r.dl[4 * q] = v.x; r.dl[4 * q + 1] = v.y; r.dl[4 * q + 2] = v.z; r.dl[4 * q + 3] = v.w;
             r.uu[4 * q] = u4.x; r.uu[4 * q + 1] = u4.y; r.uu[4 * q + 2] = u4.z; r.uu[4 * q + 3] = u4.w;
         }
-        const float* bck = sBC + (k & 1) * kBcF + (w * NS) * kTile + (lane_now() & (kTile - 1));
+        const float* bck = sBC + (k & 1) * kBcF + (w * NS) * kTile + (lane_here() & (kTile - 1));
 #pragma unroll
         for (int i = 0; i < NS; ++i) {
             r.vb[i] = bck[i * kTile];
@@ -741,7 +820,7 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
         }
         __builtin_amdgcn_s_setprio(2);
         float gBv[kTile], ddv[kTile];
-        const int ln = lane_now();
+        const int ln = lane_here();
         float* const rp_lane = sRP + w * kRpW + ln;
         float* const p_lane = sP1 + w * kTileF + tile_off(ln, 0);  // (sP2 is NW tiles further: a constant offset)
         static_for<0, kTile>([&](auto RT) {
