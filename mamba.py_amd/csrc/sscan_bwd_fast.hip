@@ -258,23 +258,8 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
         const uint32_t rowg = __builtin_amdgcn_readfirstlane((uint32_t)p.g_sl * kES);
         // the four offsets of a tensor, from a copy of the stride that the compiler cannot trace back
         // (it would otherwise hoist the products out of the tile loop and keep all of them again)
-        // (With a gate the balance is the other way round: the service waves carry two more input
-        // streams, the kernel spills either way, and forming the offsets per tile measured 3 % slower
-        // than keeping them; there they are computed once.)
         struct Steps { uint32_t at[4]; };
-        Steps keptx, keptd, kepty, keptz, keptg;
-        if constexpr (!kLean) {
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                keptx.at[j] = __builtin_amdgcn_readfirstlane(jw(j) * (uint32_t)p.u_sl * kES);
-                keptd.at[j] = __builtin_amdgcn_readfirstlane(jw(j) * (uint32_t)p.d_sl * kESd);
-                kepty.at[j] = __builtin_amdgcn_readfirstlane(jw(j) * (uint32_t)p.y_sl * kES);
-                keptz.at[j] = __builtin_amdgcn_readfirstlane(jw(j) * (uint32_t)p.z_sl * kES);
-                keptg.at[j] = __builtin_amdgcn_readfirstlane(jw(j) * (uint32_t)p.g_sl * kES);
-            }
-        }
-        auto steps_of = [&](uint32_t row, const Steps& kept) {
-            if constexpr (!kLean) return kept;
+        auto steps_of = [&](uint32_t row) {
             asm volatile("" : "+s"(row));
             Steps r;
 #pragma unroll
@@ -368,8 +353,8 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
                 wz = left(p.z_sb, p.z_sl, p.z_sd, p.ED);
                 wbc = window_bytes((p.batch - 1) * p.bc_sb + (p.L - 1) * p.bc_sl + p.N, b * p.bc_sb + tb * p.bc_sl, kES);
             }
-            const Steps sx = steps_of(rowx, keptx), sy = steps_of(rowy, kepty), sd = steps_of(rowd, keptd);
-            const Steps sz = steps_of(rowz, keptz);
+            const Steps sx = steps_of(rowx), sy = steps_of(rowy), sd = steps_of(rowd);
+            const Steps sz = steps_of(rowz);
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 raw.x[j] = ld_off(xk, offx, sx.at[j], wx);
@@ -419,7 +404,7 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
             const bool ragged = !group_full || (ragged_seq && pc == last_chunk);
             if constexpr (HAS_Z && !ACC) {
                 IO* dzk = dzg + (int64_t)pc * kTile * p.g_sl;
-                const Steps sg = steps_of(rowg, keptg);
+                const Steps sg = steps_of(rowg);
                 if (!ragged) {
 #pragma unroll
                     for (int j = 0; j < 4; ++j) st_off(dzk, offz, from_float<IO>(dzv[j]), sg.at[j]);
@@ -474,7 +459,7 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
                 wg = window_bytes(end, b * p.g_sb + (int64_t)pc * kTile * p.g_sl + (int64_t)d0 * p.g_sd, kES);
                 wgd = window_bytes(end, b * p.g_sb + (int64_t)pc * kTile * p.g_sl + (int64_t)d0 * p.g_sd, kESd);
             }
-            const Steps sg = steps_of(rowg, keptg);
+            const Steps sg = steps_of(rowg);
 #pragma unroll
             for (int j = 0; j < 4; ++j) acc.dx[j] = ld_off(dxk, offg, sg.at[j], wg);
             if (dd_wide) {
@@ -565,7 +550,7 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
             IO* dxk = dxg + (int64_t)pc * kTile * p.g_sl;
             IO* ddk = ddg + (int64_t)pc * kTile * p.g_sl;
             float* ddkf = ddgf + (int64_t)pc * kTile * p.g_sl;
-            const Steps sg = steps_of(rowg, keptg);
+            const Steps sg = steps_of(rowg);
             auto st_dd = [&](int j, float v) {
                 if (dd_wide) st_off(ddkf, offg * 2u, v, sg.at[j] * 2u);
                 else st_off(ddk, offg, from_float<IO>(v), sg.at[j]);
