@@ -794,16 +794,25 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
         // they are still being read, so the wave poisons its sums of dA: the call then returns NaN
         // in dA for these channels (and in one element of dx and ddelta per channel, see the end of the
         // kernel) instead of silently wrong gradients.
-        if (k >= 1) {
-            int spins = 0;
-            while (consumed < kSvc * k && ++spins < (1 << 20)) {
-                __builtin_amdgcn_s_sleep(1);
-                consumed = __hip_atomic_load(sConsumed, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP);
+        auto wait_consumed = [&]() {
+            if (k >= 1) {
+                int spins = 0;
+                while (consumed < kSvc * k && ++spins < (1 << 20)) {
+                    __builtin_amdgcn_s_sleep(1);
+                    consumed = __hip_atomic_load(sConsumed, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP);
+                }
+                // (added to the sums at the very end of the kernel)
+                if (consumed < kSvc * k || p.expire_waits) poison = __builtin_nanf("");
             }
-            // (added to the sums at the very end of the kernel)
-            if (consumed < kSvc * k || p.expire_waits) poison = __builtin_nanf("");
-        }
+        };
+        // With a gate the service waves need longer for the previous tile, and the wait moves four
+        // steps into the sweep: the lane-group sums of those steps are held in registers, and they and
+        // the group's partial sums are stored behind the wait (gated backward 0.757 -> 0.746 ms; without
+        // a gate the signal has come by the end of the recomputation and holding the values cost 1.5 %).
+        constexpr bool kHoldFour = HAS_Z;
+        if constexpr (!kHoldFour) wait_consumed();
         __builtin_amdgcn_s_setprio(2);
+        float rhold[4];
         float gBv[kTile], ddv[kTile];
         const int ln = lane_here();
         float* const rp_lane = sRP + w * kRpW + ln;
@@ -839,16 +848,18 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
             }
             gBv[tt] = gB;
             ddv[tt] = dd;
-            if constexpr ((tt & 3) == 0) {
-                // the partial sums of a group of four steps leave as soon as they are complete: written
-                // together at the end of the tile, the stores of all scan waves (16 KB per wave) would
-                // meet in the LDS queue in front of the barrier
+            // the partial sums of a group of four steps leave as soon as they are complete: written
+            // together at the end of the tile, the stores of all scan waves (16 KB per wave) would
+            // meet in the LDS queue in front of the barrier
+            auto store_p_group = [&]() {
                 constexpr int q = tt >> 2;
                 *reinterpret_cast<float4*>(p_lane + q * kPlane) =
                     make_float4(gBv[4 * q], gBv[4 * q + 1], gBv[4 * q + 2], gBv[4 * q + 3]);
                 *reinterpret_cast<float4*>(p_lane + NW * kTileF + q * kPlane) =
                     make_float4(ddv[4 * q], ddv[4 * q + 1], ddv[4 * q + 2], ddv[4 * q + 3]);
-            }
+            };
+            // (the first group of a gated kernel's sweep goes behind the wait, below)
+            if constexpr ((tt & 3) == 0 && !(kHoldFour && tt == kTile - 4)) store_p_group();
 
             if (tt == 2) {
                 // fetch delta, u, B, C of the next tile (published two intervals ahead)
@@ -869,7 +880,19 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
                     const float a2 = rs_stage<1>(pB[2], pC[2], lane), a3 = rs_stage<1>(pB[3], pC[3], lane);
                     r = rs_stage<3>(rs_stage<2>(a0, a2, lane), rs_stage<2>(a1, a3, lane), lane);
                 }
-                rp_lane[tt * kWave] = r;
+                if constexpr (kHoldFour && tt >= kTile - 4) {
+                    rhold[tt - (kTile - 4)] = r;
+                    if constexpr (tt == kTile - 4) {
+                        __builtin_amdgcn_sched_barrier(0);
+                        wait_consumed();
+                        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                        for (int j = 3; j >= 0; --j) rp_lane[(kTile - 4 + j) * kWave] = rhold[j];
+                        store_p_group();
+                    }
+                } else {
+                    rp_lane[tt * kWave] = r;
+                }
             }
         });
         __syncthreads();  // end of interval k: partial sums and dB/dC sums of tile k are visible
