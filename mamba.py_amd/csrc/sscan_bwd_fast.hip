@@ -805,14 +805,17 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
                 if (consumed < kSvc * k || p.expire_waits) poison = __builtin_nanf("");
             }
         };
-        // With a gate the service waves need longer for the previous tile, and the wait moves four
+        // With a gate the service waves need longer for the previous tile, and the wait moves eight
         // steps into the sweep: the lane-group sums of those steps are held in registers, and they and
-        // the group's partial sums are stored behind the wait (gated backward 0.757 -> 0.746 ms; without
-        // a gate the signal has come by the end of the recomputation and holding the values cost 1.5 %).
-        constexpr bool kHoldFour = HAS_Z;
-        if constexpr (!kHoldFour) wait_consumed();
+        // the two groups' partial sums are stored behind the wait (gated backward at configs[2]: 0.752
+        // ms waiting at the start, 0.744 with four steps held, 0.715 with eight, 0.750 with twelve;
+        // without a gate the signal has come by the end of the recomputation and holding values costs
+        // 1.5 %).
+        constexpr bool kHoldSteps = HAS_Z;
+        constexpr int kHold = 8;  // steps held (a multiple of four)
+        if constexpr (!kHoldSteps) wait_consumed();
         __builtin_amdgcn_s_setprio(2);
-        float rhold[4];
+        float rhold[kHold];
         float gBv[kTile], ddv[kTile];
         const int ln = lane_here();
         float* const rp_lane = sRP + w * kRpW + ln;
@@ -859,7 +862,7 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
                     make_float4(ddv[4 * q], ddv[4 * q + 1], ddv[4 * q + 2], ddv[4 * q + 3]);
             };
             // (the first group of a gated kernel's sweep goes behind the wait, below)
-            if constexpr ((tt & 3) == 0 && !(kHoldFour && tt == kTile - 4)) store_p_group();
+            if constexpr ((tt & 3) == 0 && !(kHoldSteps && tt >= kTile - kHold)) store_p_group();
 
             if (tt == 2) {
                 // fetch delta, u, B, C of the next tile (published two intervals ahead)
@@ -880,15 +883,21 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
                     const float a2 = rs_stage<1>(pB[2], pC[2], lane), a3 = rs_stage<1>(pB[3], pC[3], lane);
                     r = rs_stage<3>(rs_stage<2>(a0, a2, lane), rs_stage<2>(a1, a3, lane), lane);
                 }
-                if constexpr (kHoldFour && tt >= kTile - 4) {
-                    rhold[tt - (kTile - 4)] = r;
-                    if constexpr (tt == kTile - 4) {
+                if constexpr (kHoldSteps && tt >= kTile - kHold) {
+                    rhold[tt - (kTile - kHold)] = r;
+                    if constexpr (tt == kTile - kHold) {
                         __builtin_amdgcn_sched_barrier(0);
                         wait_consumed();
                         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                        for (int j = 3; j >= 0; --j) rp_lane[(kTile - 4 + j) * kWave] = rhold[j];
-                        store_p_group();
+                        for (int j = kHold - 1; j >= 0; --j) rp_lane[(kTile - kHold + j) * kWave] = rhold[j];
+#pragma unroll
+                        for (int q = NQ - 1; q >= NQ - kHold / 4; --q) {
+                            *reinterpret_cast<float4*>(p_lane + q * kPlane) =
+                                make_float4(gBv[4 * q], gBv[4 * q + 1], gBv[4 * q + 2], gBv[4 * q + 3]);
+                            *reinterpret_cast<float4*>(p_lane + NW * kTileF + q * kPlane) =
+                                make_float4(ddv[4 * q], ddv[4 * q + 1], ddv[4 * q + 2], ddv[4 * q + 3]);
+                        }
                     }
                 } else {
                     rp_lane[tt * kWave] = r;
