@@ -25,7 +25,7 @@
 enum Stream {
     kFmaIndependent, kFmaDependent, kExp, kExpDependent, kDppBroadcast, kLaneSwap32, kForwardMix, kForwardMixPlain,
     kBackwardMix, kBackwardMixPlain, kFmaSgpr, kForwardMixSgpr,
-    kG0, kG1, kG2, kG3, kG4, kG5, kG6, kG7, kG8, kG9, kG10, kG11, kG12, kG13, kG14, kG15, kMixBatched, kMixAlt, kMixAlt2
+    kG0, kG1, kG2, kG3, kG4, kG5, kG6, kG7, kG8, kG9, kG10, kG11, kG12, kG13, kG14, kG15, kG16, kG17, kG18, kG19, kMixBatched, kMixAlt, kMixAlt2
 };
 #define GEN8(T) T("0") T("1") T("2") T("3") T("4") T("5") T("6") T("7")
 #define G0(i) "v_fmac_f32 %" i ", 1.0, %9\n"
@@ -43,6 +43,10 @@ enum Stream {
 #define G13(i) "v_max_f32 %" i ", %" i ", %9\n"
 #define G14(i) "v_cvt_pk_bf16_f32 %" i ", %" i ", %9\n"
 #define G15(i) "v_writelane_b32 %" i ", s22, 5\n"
+#define G16(i) "v_add_f32_dpp %" i ", %" i ", %9 quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf\n"
+#define G17(i) "v_add_f32_dpp %" i ", %" i ", %9 row_mirror row_mask:0xf bank_mask:0xf\n"
+#define G18(i) "v_mov_b32_dpp %" i ", %9 quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf\n"
+#define G19(i) "v_add_f32_sdwa %" i ", %" i ", %9 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:DWORD\n"
 #define G9(i) "v_add_f32_dpp %" i ", %" i ", %9 row_shr:1 row_mask:0xf bank_mask:0x5\n"
 
 
@@ -221,6 +225,30 @@ __global__ void probe_kernel(float* out, long long* ticks, int iters) {
                              "v_fmac_f32_dpp %1, %8, %9" BC3 "v_fmac_f32_dpp %3, %8, %9" BC3 "v_fmac_f32_dpp %5, %8, %9" BC5 "v_fmac_f32_dpp %7, %8, %9" BC5
                              : "+v"(v0), "+v"(v1), "+v"(v2), "+v"(v3), "+v"(v4), "+v"(v5), "+v"(v6), "+v"(v7)
                              : "v"(c), "v"(d));
+        } else if constexpr (STREAM == kG16) {
+#pragma unroll
+            for (int r = 0; r < 8; ++r)
+                asm volatile(GEN8(G16)
+                             : "+v"(v0), "+v"(v1), "+v"(v2), "+v"(v3), "+v"(v4), "+v"(v5), "+v"(v6), "+v"(v7)
+                             : "v"(c), "v"(d) : "vcc");
+        } else if constexpr (STREAM == kG17) {
+#pragma unroll
+            for (int r = 0; r < 8; ++r)
+                asm volatile(GEN8(G17)
+                             : "+v"(v0), "+v"(v1), "+v"(v2), "+v"(v3), "+v"(v4), "+v"(v5), "+v"(v6), "+v"(v7)
+                             : "v"(c), "v"(d) : "vcc");
+        } else if constexpr (STREAM == kG18) {
+#pragma unroll
+            for (int r = 0; r < 8; ++r)
+                asm volatile(GEN8(G18)
+                             : "+v"(v0), "+v"(v1), "+v"(v2), "+v"(v3), "+v"(v4), "+v"(v5), "+v"(v6), "+v"(v7)
+                             : "v"(c), "v"(d) : "vcc");
+        } else if constexpr (STREAM == kG19) {
+#pragma unroll
+            for (int r = 0; r < 8; ++r)
+                asm volatile(GEN8(G19)
+                             : "+v"(v0), "+v"(v1), "+v"(v2), "+v"(v3), "+v"(v4), "+v"(v5), "+v"(v6), "+v"(v7)
+                             : "v"(c), "v"(d) : "vcc");
         } else if constexpr (STREAM == kFmaDependent) {
 #pragma unroll
             for (int r = 0; r < 64; ++r) asm volatile("v_fma_f32 %0, %0, %1, %2" : "+v"(v0) : "v"(c), "v"(d));
@@ -385,6 +413,10 @@ int main() {
     rc |= run<kMixBatched>("forward mix batched by kind", out, ticks, clock_hz);
     rc |= run<kMixAlt>("plain / DPP alternating", out, ticks, clock_hz);
     rc |= run<kMixAlt2>("plain / DPP in runs of four", out, ticks, clock_hz);
+    rc |= run<kG16>("v_add_f32_dpp quad_perm", out, ticks, clock_hz);
+    rc |= run<kG17>("v_add_f32_dpp row_mirror", out, ticks, clock_hz);
+    rc |= run<kG18>("v_mov_b32_dpp quad_perm", out, ticks, clock_hz);
+    rc |= run<kG19>("v_add_f32_sdwa (dword sel)", out, ticks, clock_hz);
     rc |= run<kFmaDependent>("v_fma_f32, one dependent chain", out, ticks, clock_hz);
     rc |= run<kExp>("v_exp_f32, independent", out, ticks, clock_hz);
     rc |= run<kExpDependent>("v_exp_f32, one dependent chain", out, ticks, clock_hz);
