@@ -778,7 +778,9 @@ def main():
             other = {}
             cpu = not args.no_cpu_baseline
             other["c0"] = _brief(bench_sscan(args, torch, pkg, dev, "c0", max(10, args.steps), 3, 0, cpu=cpu))
-            other["c1"] = _brief(bench_sscan(args, torch, pkg, dev, "c1", max(10, args.steps // 2), 3, 10, cpu=cpu))
+            # (the CPU baseline of the headline record has just left the GPU idle for seconds: as many
+            # untimed start-up steps as make about 40 ms of GPU work, like the headline's own 40)
+            other["c1"] = _brief(bench_sscan(args, torch, pkg, dev, "c1", max(10, args.steps // 2), 3, 100, cpu=cpu))
             other["c3"] = _brief(bench_decode(args, torch, pkg, dev),
                                  ("kernel_step_us_called_from_python", "block_step_us", "graphed_layer_step_us"))
             torch.cuda.empty_cache()
