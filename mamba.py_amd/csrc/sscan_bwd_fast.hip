@@ -266,6 +266,23 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
             for (int j = 0; j < 4; ++j) r.at[j] = jw(j) * row;
             return r;
         };
+        // origin of physical chunk pc in a tensor whose rows are `row` bytes (`stride` elements of the
+        // pointer's type) apart.  Without a gate: a 32 x 32 -> 64 bit product of the scalar unit on the
+        // stride register that steps_of uses (with the 64-bit element strides of the arguments, each
+        // tensor keeps two more scalar registers alive and every tile pays a 64 x 64 bit product:
+        // configs[1] backward 0.302 -> 0.297 ms).  The gated kernels measured 2 % slower with it (their
+        // register allocation again) and keep the 64-bit form.
+        auto at_chunk = [&](auto* base, int pc, uint32_t row, int64_t stride) {
+            typedef decltype(base) P;
+            if constexpr (kLean) {
+                const uint64_t off = (uint64_t)(uint32_t)(pc * kTile) * (uint64_t)row;
+                return reinterpret_cast<P>(reinterpret_cast<uintptr_t>(base) + off);
+            } else {
+                return base + (int64_t)pc * kTile * stride;
+            }
+        };
+        const uint32_t rowbc = __builtin_amdgcn_readfirstlane((uint32_t)p.bc_sl * kES);
+        const uint32_t rowfw = __builtin_amdgcn_readfirstlane((uint32_t)p.Nst * 4u);
         // tensor origins of this (batch row, channel group)
         const IO* const xb = static_cast<const IO*>(p.x) + (b * p.u_sb + (int64_t)d0 * p.u_sd);
         const char* const db = static_cast<const char*>(p.delta) + (b * p.d_sb + (int64_t)d0 * p.d_sd) * (int64_t)kESd;
@@ -332,13 +349,13 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
             // as whatever follows inside the tensor (or zero past its end) and masked at staging
             const int k = min(kk, ntiles - 1);
             const int pc = phys_of(chunk_of(k));
-            const IO* xk = xb + (int64_t)pc * kTile * p.u_sl;
-            const char* dk = db + ((int64_t)pc * kTile * p.d_sl) * kESd;
-            const IO* yk = yb + (int64_t)pc * kTile * p.y_sl;
-            const IO* zk = zb + (int64_t)pc * kTile * p.z_sl;
-            const IO* ypk = ypb + (int64_t)pc * kTile * p.y_sl;
-            const IO* Bk = Bb + (int64_t)pc * kTile * p.bc_sl;
-            const IO* Ck = Cb + (int64_t)pc * kTile * p.bc_sl;
+            const IO* xk = at_chunk(xb, pc, rowx, p.u_sl);
+            const char* dk = at_chunk(db, pc, rowd, p.d_sl * (int64_t)kESd);
+            const IO* yk = at_chunk(yb, pc, rowy, p.y_sl);
+            const IO* zk = at_chunk(zb, pc, rowz, p.z_sl);
+            const IO* ypk = at_chunk(ypb, pc, rowy, p.y_sl);
+            const IO* Bk = at_chunk(Bb, pc, rowbc, p.bc_sl);
+            const IO* Ck = at_chunk(Cb, pc, rowbc, p.bc_sl);
             uint32_t wx = 0xffffffffu, wd = wx, wy = wx, wz = wx, wbc = wx;
             if (ragged_seq && pc == last_chunk) {
                 // elements from this chunk's origin to one past the tensor's last element
@@ -403,7 +420,7 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
             }
             const bool ragged = !group_full || (ragged_seq && pc == last_chunk);
             if constexpr (HAS_Z && !ACC) {
-                IO* dzk = dzg + (int64_t)pc * kTile * p.g_sl;
+                IO* dzk = at_chunk(dzg, pc, rowg, p.g_sl);
                 const Steps sg = steps_of(rowg);
                 if (!ragged) {
 #pragma unroll
@@ -451,8 +468,8 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
         auto load_acc = [&](int kk) {
             if constexpr (!ACC) return;
             const int pc = phys_of(chunk_of(min(kk, ntiles - 1)));
-            const IO* dxk = dxg + (int64_t)pc * kTile * p.g_sl;
-            const IO* ddk = ddg + (int64_t)pc * kTile * p.g_sl;
+            const IO* dxk = at_chunk(dxg, pc, rowg, p.g_sl);
+            const IO* ddk = at_chunk(ddg, pc, rowg, p.g_sl);
             uint32_t wg = 0xffffffffu, wgd = 0xffffffffu;
             if (ragged_seq && pc == last_chunk) {
                 const int64_t end = (p.batch - 1) * p.g_sb + (p.L - 1) * p.g_sl + (p.ED - 1) * p.g_sd + 1;
@@ -464,7 +481,7 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
             for (int j = 0; j < 4; ++j) acc.dx[j] = ld_off(dxk, offg, sg.at[j], wg);
             if (dd_wide) {
 #pragma unroll
-                for (int j = 0; j < 4; ++j) acc.dd[j] = ld_bits32(ddgf + (int64_t)pc * kTile * p.g_sl, offg * 2u, sg.at[j] * 2u, wgd);
+                for (int j = 0; j < 4; ++j) acc.dd[j] = ld_bits32(at_chunk(ddgf, pc, rowg * 2u, p.g_sl), offg * 2u, sg.at[j] * 2u, wgd);
             } else if (sizeof(IO) == 4) {
 #pragma unroll
                 for (int j = 0; j < 4; ++j) acc.dd[j] = ld_bits32(ddk, offg, sg.at[j], wgd);
@@ -547,15 +564,15 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
                     dv[j] += bits_to_float(acc.dd[j], dshift);
                 }
             }
-            IO* dxk = dxg + (int64_t)pc * kTile * p.g_sl;
-            IO* ddk = ddg + (int64_t)pc * kTile * p.g_sl;
-            float* ddkf = ddgf + (int64_t)pc * kTile * p.g_sl;
+            IO* dxk = at_chunk(dxg, pc, rowg, p.g_sl);
+            IO* ddk = at_chunk(ddg, pc, rowg, p.g_sl);
+            float* ddkf = at_chunk(ddgf, pc, rowg * 2u, p.g_sl);  // (float32 next to bfloat16 tensors: rows twice as wide)
             const Steps sg = steps_of(rowg);
             auto st_dd = [&](int j, float v) {
                 if (dd_wide) st_off(ddkf, offg * 2u, v, sg.at[j] * 2u);
                 else st_off(ddk, offg, from_float<IO>(v), sg.at[j]);
             };
-            float* fwk = fw_base + (int64_t)pc * kTile * p.Nst;
+            float* fwk = at_chunk(fw_base, pc, rowfw, p.Nst);
             if (group_full && !(ragged_seq && pc == last_chunk) && fw_vec) {
                 if constexpr (kLean) {
 #pragma unroll

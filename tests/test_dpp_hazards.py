@@ -16,8 +16,16 @@ import pytest
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 CSRC = os.path.join(ROOT, "mamba.py_amd", "csrc")
-FLAGS = ["-O3", "--offload-arch=gfx950", "-std=c++17", "-Xclang", "-target-feature", "-Xclang",
-         "-packed-fp32-ops", "-Wno-unused-command-line-argument", "-S", "--cuda-device-only"]
+
+
+def _build_recipe():
+    """the flags libmambapy_amd.so is built with (the checked code must be the shipped code)"""
+    import importlib.util
+    spec = importlib.util.spec_from_file_location("mpa_build", os.path.join(ROOT, "mamba.py_amd", "build.py"))
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    return mod
+
 
 
 def _vgprs(tok):
@@ -72,7 +80,10 @@ def test_no_dpp_operand_is_read_too_early(src, tmp_path):
     if not os.path.exists(hipcc):
         pytest.skip("hipcc not available")
     out = tmp_path / (src + ".s")
-    res = subprocess.run([hipcc, *FLAGS, os.path.join(CSRC, src), "-o", str(out)], capture_output=True, text=True)
+    recipe = _build_recipe()
+    flags = [recipe.OPT_LEVEL.get(src, recipe.DEFAULT_OPT_LEVEL), *[f for f in recipe.HIPCC_FLAGS if f != "-fPIC"],
+             "-S", "--cuda-device-only"]
+    res = subprocess.run([hipcc, *flags, os.path.join(CSRC, src), "-o", str(out)], capture_output=True, text=True)
     assert res.returncode == 0, res.stderr[-2000:]
     ndpp, hazards = find_dpp_hazards(out.read_text())
     assert ndpp > 100, "the kernels are expected to contain DPP instructions"
