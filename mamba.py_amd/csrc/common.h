@@ -113,16 +113,6 @@ __device__ __forceinline__ void st_off(float4* base, uint32_t voff, float4 v, ui
     __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v), make_rsrc(base), voff, soff, 0);
 }
 
-// Lane index recomputed on the spot (two VALU instructions).  Per-lane addresses that are used
-// once per tile are derived from this instead of a value computed before the loop: the
-// compiler would keep such a value alive across the whole tile and, under register pressure,
-// spill it to scratch memory, where every reload costs a round trip of several hundred clocks.
-__device__ __forceinline__ int lane_now() {
-    int l;
-    asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(l));
-    return l;
-}
-
 __device__ __forceinline__ int wave_id() {
     // threadIdx.x / 64, told to the compiler as wave-uniform
     return __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x) >> 6);

@@ -217,9 +217,9 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
         constexpr uint32_t kES = sizeof(IO);
         const bool group_full = cmax == kWave - 1;
         // With a gate the service waves carry two more input streams, set the kernel's register count
-        // and spill; the forms below marked kLean (less work for the vector unit, a few more live
-        // values) made that worse when they were tried there (gated backward 0.75 -> 0.78 .. 0.89 ms),
-        // so a gated kernel keeps the plainer forms.
+        // and spill scalar registers into vector lanes; three of the forms below (marked kLean: a few
+        // instructions less, a few more live values) measured slower there (gated backward +1.5 % with
+        // the first two, +2 % with the third) and a gated kernel keeps the plainer ones.
         constexpr bool kLean = !HAS_Z;
 
         // ---- input side: item -> (channel, step group), offsets that never change ----
@@ -695,30 +695,10 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
     // fetched with one buffer instruction per state: wave-uniform slot address and state row (scalar
     // registers) + the lane's channel offset, the one per-lane value, kept for the whole kernel (built
     // from the lane index at every tile, the address cost each scan wave a dozen half-rate instructions
-    // per tile).  With a gate the service waves set the kernel's register count and already spill:
-    // there the scan waves rebuild their per-lane offsets from the lane index where they are used
-    // (lane_now) instead of keeping them.
-    constexpr bool kKeepLaneOffsets = !HAS_Z;
-    const uint32_t ck_voff_kept = (uint32_t)min(d, p.ED - 1) * 4u;
-    auto lane_here = [&]() { return kKeepLaneOffsets ? lane : lane_now(); };
+    // per tile).
+    const uint32_t ck_voff = (uint32_t)min(d, p.ED - 1) * 4u;
     auto load_state = [&](int k, float (&hs)[NS]) {
         const int c = chunk_of(min(k, ntiles - 1));
-        if constexpr (!kKeepLaneOffsets) {
-            // branch-free form: chunk 0 reads slot 0 (or h0) and the value is masked below
-            const uint32_t ck_lane = (uint32_t)min(d0 + lane_now(), p.ED - 1);
-            const float* ck_base = p.ckpt + ((int64_t)b * p.nchunks + max(c - 1, 0)) * p.Nst * p.ED;
-            const float* h0_base = p.h0 ? p.h0 + (int64_t)b * p.ED * p.Nst : ck_base;
-            const bool first = c == 0;
-#pragma unroll
-            for (int i = 0; i < NS; ++i) {
-                const uint32_t n = (uint32_t)min(w * NS + i, p.N - 1);
-                const uint32_t off = first && p.h0 ? ck_lane * (uint32_t)p.Nst + n : n * (uint32_t)p.ED + ck_lane;
-                const float v = (first ? h0_base : ck_base)[off];
-                hs[i] = (!first || p.h0) ? v : 0.0f;
-            }
-            return;
-        }
-        const uint32_t ck_voff = ck_voff_kept;
         if (c > 0) {
             const float* ck_base = p.ckpt + ((int64_t)b * p.nchunks + (c - 1)) * p.Nst * p.ED;
 #pragma unroll
@@ -749,7 +729,7 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
             r.dl[4 * q] = v.x; r.dl[4 * q + 1] = v.y; r.dl[4 * q + 2] = v.z; r.dl[4 * q + 3] = v.w;
             r.uu[4 * q] = u4.x; r.uu[4 * q + 1] = u4.y; r.uu[4 * q + 2] = u4.z; r.uu[4 * q + 3] = u4.w;
         }
-        const float* bck = sBC + (k & 1) * kBcF + (w * NS) * kTile + (lane_here() & (kTile - 1));
+        const float* bck = sBC + (k & 1) * kBcF + (w * NS) * kTile + (lane & (kTile - 1));
 #pragma unroll
         for (int i = 0; i < NS; ++i) {
             r.vb[i] = bck[i * kTile];
@@ -834,7 +814,7 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
         __builtin_amdgcn_s_setprio(2);
         float rhold[kHold];
         float gBv[kTile], ddv[kTile];
-        const int ln = lane_here();
+        const int ln = lane;
         float* const rp_lane = sRP + w * kRpW + ln;
         float* const p_lane = sP1 + w * kTileF + tile_off(ln, 0);  // (sP2 is NW tiles further: a constant offset)
         static_for<0, kTile>([&](auto RT) {
