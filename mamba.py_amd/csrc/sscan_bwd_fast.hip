@@ -9,8 +9,8 @@
 //         g[t] = dy[t]*C[t] + a[t+1]*g[t+1]
 //         d(delta*A) = g*a*h[t-1]   -> dA += .*delta ;  ddelta += .*A
 //         sum_n g*B                 -> dx = delta*. ;   ddelta += x*.
-//         g*u (u = delta*x), dy*h   -> dB, dC, summed over the 64 channels of the wave by an
-//                                      in-register reduce-scatter (rs_stage).
+//         g*u (u = delta*x), dy*h   -> dB, dC: summed over the lanes of a row as far as plain DPP
+//                                      additions go (rs_stage), the rest by the service waves.
 //     B and C of a tile sit in one register per state whose lane t of every row of 16 lanes
 //     holds step t; the FMAs pick their step with a DPP row broadcast (fmac_bcast), so B and C
 //     cost neither scalar registers nor extra instructions.
@@ -52,25 +52,20 @@ __device__ __forceinline__ void tile_st(float* tile, int ch, int q, float a, flo
     *reinterpret_cast<float4*>(tile + tile_off(ch, q)) = make_float4(a, b, c, d);
 }
 
-// ---- in-register reduce-scatter over the 64 lanes of a wave ------------------------------
-// 64 values per lane are summed over all lanes in six halving stages; after stage s only
-// half of the registers remain, and a lane keeps the value whose index bit s equals the
-// matching lane bit, so that at the end lane l holds the complete sum of value number l and
-// each value cost (32+16+8+4+2+1)/64 adds plus the data movement, all on the VALU (no LDS
-// round trip sits in the dependency chain of the reverse sweep).
-//   stage 1: DPP row_mirror      (lane bit 3)     stage 4: DPP quad_perm 1032  (lane bit 0)
-//   stage 2: DPP row_half_mirror (lane bit 2)     stage 5: v_permlane16_swap   (lane bit 4)
-//   stage 3: DPP quad_perm 3210  (lane bit 1)     stage 6: v_permlane32_swap   (lane bit 5)
+// ---- reduce-scatter over the lanes of a row (first part of the dB / dC channel sums) ---------
+// A sum over the lanes of a wave can be taken in halving stages: a stage combines two registers
+// into one, a lane keeping the value whose index bit equals the stage's lane bit and receiving
+// its partner lane's share of it, so each value costs less than one addition per stage and no
+// LDS round trip sits in the dependency chain of the reverse sweep.  The scan waves run only the
+// stages that stay inside a row of 16 lanes and are plain DPP additions (two at two states per
+// lane, three at four); the 16 / 2^stages partial sums per value and row that are left go to LDS
+// as they are and the service waves add them one tile later (the stages across rows are lane
+// swaps at twice the cost of a DPP addition each, and the scattered stores that followed them
+// cost more than the 30 additions per service thread that replaced them).
+//   stage 1: DPP row_mirror      (lane bit 3)     stage 3: DPP quad_perm 3210  (lane bit 1)
+//   stage 2: DPP row_half_mirror (lane bit 2)
 // (every stage's partner lane agrees with the lane in the bits of the stages before it)
 // `lo` is the value with index bit 0 (kept by lanes whose bit is clear), `hi` the other one.
-__device__ __forceinline__ float rs_swap32(float lo, float hi) {
-    const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(lo), __float_as_uint(hi), false, false);
-    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
-}
-__device__ __forceinline__ float rs_swap16(float lo, float hi) {
-    const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(lo), __float_as_uint(hi), false, false);
-    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
-}
 template <int CTRL>
 __device__ __forceinline__ float rs_dpp(float lo, float hi, bool lane_bit) {
     const float keep = lane_bit ? hi : lo;
@@ -79,7 +74,7 @@ __device__ __forceinline__ float rs_dpp(float lo, float hi, bool lane_bit) {
         __builtin_amdgcn_update_dpp(0u, __float_as_uint(send), CTRL, 0xf, 0xf, false));
     return keep + got;
 }
-// Stages 3 and 4 without selects: the lanes whose bit is clear form whole banks (groups of four
+// Stages 1 and 2 without selects: the lanes whose bit is clear form whole banks (groups of four
 // lanes) of a row, so two additions that each write only their banks do the work: lanes with the
 // bit clear get lo + lo[partner], the others hi + hi[partner].  (The compiler does not see into
 // inline assembly: the two wait states a DPP read needs after a VALU write of the same register
@@ -102,20 +97,13 @@ __device__ __forceinline__ float rs_mirror4(float lo, float hi) {
         : "v"(lo), "v"(hi));
     return r;
 }
-// stage number (1..6) -> combine.  The stages inside a row of 16 lanes come first: they work on
-// the most values, and a DPP addition costs the SIMD half of what a lane swap across rows costs.
+// stage number (1..3) -> combine
 template <int STAGE>
 __device__ __forceinline__ float rs_stage(float lo, float hi, int lane) {
+    static_assert(STAGE >= 1 && STAGE <= 3, "the scan waves run the stages inside a row only");
     if constexpr (STAGE == 1) return rs_mirror8(lo, hi);
     else if constexpr (STAGE == 2) return rs_mirror4(lo, hi);
-    else if constexpr (STAGE == 3) return rs_dpp<0x1B>(lo, hi, (lane & 2) != 0);
-    else if constexpr (STAGE == 4) return rs_dpp<0xB1>(lo, hi, (lane & 1) != 0);
-    else if constexpr (STAGE == 5) return rs_swap16(lo, hi);
-    else return rs_swap32(lo, hi);
-}
-// lane bit that decides, in stage 1..6, which of the two values a lane keeps
-__device__ __forceinline__ constexpr int rs_lane_bit(int stage) {
-    return stage == 1 ? 3 : stage == 2 ? 2 : stage == 3 ? 1 : stage == 4 ? 0 : stage == 5 ? 4 : 5;
+    else return rs_dpp<0x1B>(lo, hi, (lane & 2) != 0);
 }
 
 constexpr int kSvc = 4;  // service waves per workgroup
@@ -270,8 +258,8 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
         // pointer's type) apart.  Without a gate: a 32 x 32 -> 64 bit product of the scalar unit on the
         // stride register that steps_of uses (with the 64-bit element strides of the arguments, each
         // tensor keeps two more scalar registers alive and every tile pays a 64 x 64 bit product:
-        // configs[1] backward 0.302 -> 0.297 ms).  The gated kernels measured 2 % slower with it (their
-        // register allocation again) and keep the 64-bit form.
+        // backward at B=8, L=2048, 1536 channels, float32: 0.302 -> 0.297 ms).  The gated kernels
+        // measured 2 % slower with it (their register allocation again) and keep the 64-bit form.
         auto at_chunk = [&](auto* base, int pc, uint32_t row, int64_t stride) {
             typedef decltype(base) P;
             if constexpr (kLean) {
@@ -804,8 +792,9 @@ __global__ void __launch_bounds__((NW + kSvc) * kWave) sscan_bwd_fast_kernel(con
         };
         // With a gate the service waves need longer for the previous tile, and the wait moves eight
         // steps into the sweep: the lane-group sums of those steps are held in registers, and they and
-        // the two groups' partial sums are stored behind the wait (gated backward at configs[2]: 0.752
-        // ms waiting at the start, 0.744 with four steps held, 0.715 with eight, 0.750 with twelve;
+        // the two groups' partial sums are stored behind the wait (gated backward at B=4, L=4096, 4096
+        // channels, bfloat16: 0.752 ms waiting at the start, 0.744 with four steps held, 0.715 with eight,
+        // 0.750 with twelve;
         // without a gate the signal has come by the end of the recomputation and holding values costs
         // 1.5 %).
         constexpr bool kHoldSteps = HAS_Z;
